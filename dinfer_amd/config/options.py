@@ -1,0 +1,36 @@
+"""Engine options: the names, meanings and defaults of the reference's command line
+(bins/dinfer/src/main.rs:30-131) and of its SchedulerConfig / CacheConfig
+(crates/core/src/config.rs:25-92), as far as they concern one GPU.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+
+@dataclass
+class EngineOptions:
+    dtype: str = "bfloat16"             # "bfloat16" or "float32"
+    max_model_len: int = 4096           # prompt + output per request; width of the block table
+    max_num_seqs: int = 16              # live requests; also the most logits rows of a serving step
+    max_num_batched_tokens: int = 2048  # per-step token budget
+    num_blocks: int | None = None       # cache pages per group; None: sized from free memory
+    block_size: int = 16                # tokens per page
+    gpu_memory_utilization: float = 0.9
+    decode_exempt_from_budget: bool = True   # a decode row does not consume the token budget
+    long_prefill_token_threshold: int = 0    # per-request cap on a prompt portion (0: none)
+    prefill_tokens_per_step: int = 0         # cap on all prompt tokens of a step (0: none)
+    enable_chunked_prefill: bool = True
+    hip_graph: bool = True              # replay decode steps from captured HIP graphs
+    device: int = 0
+    max_logits_rows: int | None = None  # None: max_num_seqs; replay and tests ask for more
+
+    def check(self) -> None:
+        if self.dtype not in ("bfloat16", "float32"):
+            raise ValueError(f"dtype must be 'bfloat16' or 'float32', got {self.dtype!r}")
+        for name in ("max_model_len", "max_num_seqs", "max_num_batched_tokens", "block_size"):
+            if getattr(self, name) <= 0:
+                raise ValueError(f"{name} must be positive, got {getattr(self, name)}")
+        if self.num_blocks is not None and self.num_blocks <= 0:
+            raise ValueError(f"num_blocks must be positive, got {self.num_blocks}")
+        if not (0.0 < self.gpu_memory_utilization <= 1.0):
+            raise ValueError(f"gpu_memory_utilization must be in (0, 1], got {self.gpu_memory_utilization}")

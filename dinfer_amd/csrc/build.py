@@ -1,0 +1,153 @@
+"""Compiles the HIP sources of this folder for gfx950, one shared library per
+source file, into ``dinfer_amd/_lib/`` (or a per-user temporary folder when the
+package folder is read-only).
+
+A library is built on first use and reused afterwards; ``build_all(force=True)``
+recompiles everything. Only what a caller asks for is compiled, so a program
+that never samples never builds the sampling library.
+"""
+from __future__ import annotations
+
+import hashlib
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import threading
+import time
+from pathlib import Path
+
+CSRC = Path(__file__).resolve().parent
+PACKAGE = CSRC.parent
+
+# library name -> source file. Headers that all of them include are hashed too.
+SOURCES = {
+    "elementwise": "elementwise.hip",
+    "norm": "norm.hip",
+    "rope": "rope.hip",
+    "attention_ref": "attention_ref.hip",
+    "attention": "attention.hip",
+    "gemm_ref": "gemm_ref.hip",
+    "gemm": "gemm.hip",
+    "sampling": "sampling.hip",
+}
+HEADERS = ["common.cuh"]
+
+ARCH = "gfx950"
+# -packed-fp32-ops is switched off for device code: hipcc -O3 otherwise forms packed
+# float instructions from ordinary float code. The host pass does not know the
+# feature and says so on stderr; that is harmless and filtered out below.
+FLAGS = [
+    f"--offload-arch={ARCH}",
+    "-O3",
+    "-std=c++17",
+    "-shared",
+    "-fPIC",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-result",
+]
+
+
+def _hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found: the HIP kernels cannot be built (looked in $HIPCC, PATH, /opt/rocm/bin)")
+
+
+def lib_dir() -> Path:
+    """Folder for built libraries: in the package if writable, else per-user temporary."""
+    d = PACKAGE / "_lib"
+    try:
+        d.mkdir(exist_ok=True)
+        probe = d / f".w{os.getpid()}"
+        probe.write_text("")
+        probe.unlink()
+        return d
+    except OSError:
+        alt = Path(tempfile.gettempdir()) / f"dinfer_amd_lib_{os.getuid()}"
+        alt.mkdir(parents=True, exist_ok=True)
+        return alt
+
+
+def source_hash(name: str) -> str:
+    h = hashlib.sha256()
+    for f in HEADERS + [SOURCES[name]]:
+        h.update((CSRC / f).read_bytes())
+    h.update(" ".join(FLAGS).encode())
+    return h.hexdigest()[:16]
+
+
+def lib_path(name: str) -> Path:
+    return lib_dir() / f"libdinfer_{name}.so"
+
+
+def find_built(name: str) -> Path | None:
+    """A library built earlier, in the package or in the per-user folder; None if absent."""
+    for d in (PACKAGE / "_lib", Path(tempfile.gettempdir()) / f"dinfer_amd_lib_{os.getuid()}"):
+        p = d / f"libdinfer_{name}.so"
+        if p.exists():
+            return p
+    return None
+
+
+def is_stale(name: str, path: Path) -> bool:
+    tag = path.with_suffix(".hash")
+    try:
+        return tag.read_text().strip() != source_hash(name)
+    except OSError:
+        return True
+
+
+def build(name: str, verbose: bool = True) -> Path:
+    """Compiles one library and returns its path. Prints a line now and then while hipcc runs."""
+    if name not in SOURCES:
+        raise KeyError(f"unknown kernel library {name!r}; known: {sorted(SOURCES)}")
+    out = lib_path(name)
+    tmp = out.with_name(f".{out.name}.{os.getpid()}.tmp")
+    cmd = [_hipcc(), *FLAGS, str(CSRC / SOURCES[name]), "-o", str(tmp)]
+    t0 = time.time()
+    if verbose:
+        print(f"[dinfer_amd] compiling {SOURCES[name]} for {ARCH} ...", file=sys.stderr, flush=True)
+    proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, cwd=str(CSRC))
+    done = threading.Event()
+
+    def ticker():
+        while not done.wait(20.0):
+            print(f"[dinfer_amd] still compiling {SOURCES[name]} ({time.time() - t0:.0f} s)", file=sys.stderr, flush=True)
+
+    th = threading.Thread(target=ticker, daemon=True)
+    if verbose:
+        th.start()
+    log, _ = proc.communicate()
+    done.set()
+    log = "\n".join(l for l in log.splitlines() if "packed-fp32-ops" not in l)
+    if proc.returncode != 0:
+        tmp.unlink(missing_ok=True)
+        raise RuntimeError(f"hipcc failed for {SOURCES[name]}:\n{log}")
+    os.replace(tmp, out)
+    out.with_suffix(".hash").write_text(source_hash(name))
+    if verbose:
+        print(f"[dinfer_amd] built {out.name} in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+    return out
+
+
+def build_all(force: bool = True, jobs: int = 4, verbose: bool = True) -> dict[str, Path]:
+    """Compiles every library (in parallel processes of hipcc)."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    names = [n for n in SOURCES if (CSRC / SOURCES[n]).exists()]
+
+    def one(n):
+        p = find_built(n)
+        if not force and p is not None and not is_stale(n, p):
+            return n, p
+        return n, build(n, verbose=verbose)
+
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        return dict(ex.map(one, names))
+
+
+if __name__ == "__main__":
+    build_all(force=True)

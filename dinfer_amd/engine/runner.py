@@ -1,0 +1,175 @@
+"""The model runner: owns the model, the cache pages and the step function.
+
+``step(entries)`` is the one step function of the engine: it runs exactly the
+tokens it is given, as one batch, against the cache that earlier steps left, and
+returns the logits at the wanted places. Generation, the scheduler's engine loop
+and trace replay all go through it; none of them has a forward pass, a cache or
+a loader of its own (models/qwen3/src/executor.rs:977-1031, model.rs:684-832).
+"""
+from __future__ import annotations
+
+import json
+from pathlib import Path
+
+import torch
+
+from ..cache import CacheManager, GroupSpec
+from ..config import EngineOptions, load_config
+from ..kernels import ops
+from ..parts import BuildContext, CacheView, DecoderModel, KVSpec, StateSpec
+from ..weights import WeightLoader
+from .batch import Entry, StepBatch
+
+_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+
+
+def _require_gpu(device_index: int) -> torch.device:
+    if not torch.cuda.is_available():
+        raise RuntimeError("dinfer_amd needs a GPU: no HIP device is visible and there is no CPU path")
+    if device_index >= torch.cuda.device_count():
+        raise RuntimeError(f"device {device_index} does not exist ({torch.cuda.device_count()} visible)")
+    dev = torch.device("cuda", device_index)
+    torch.cuda.set_device(dev)
+    return dev
+
+
+class ModelRunner:
+    def __init__(self, model: DecoderModel, options: EngineOptions, device: torch.device):
+        options.check()
+        self.model, self.options, self.device = model, options, device
+        self.dtype = _DTYPES[options.dtype]
+        spec = model.spec
+        if options.max_model_len > spec.max_positions:
+            raise ValueError(f"max_model_len {options.max_model_len} exceeds the model's "
+                             f"{spec.max_positions} positions")
+        self.page_size = options.block_size
+        self.max_rows = options.max_logits_rows or options.max_num_seqs
+        # decode rows may ride on top of the prompt budget (service.rs:206-210)
+        self.max_tokens = options.max_num_batched_tokens + (options.max_num_seqs if options.decode_exempt_from_budget else 0)
+        self.ctx = BuildContext(device, self.dtype, self.max_tokens, self.max_rows, self.page_size)
+        model.bind(self.ctx)
+        self._build_caches()
+        self.batch = StepBatch(device, self.max_tokens, options.max_num_seqs, self.max_rows,
+                               [self.max_blocks_per_seq] * len(self.group_specs))
+
+    # ---- construction --------------------------------------------------------------------------
+    @classmethod
+    def from_dir(cls, model_dir: str | Path, options: EngineOptions) -> "ModelRunner":
+        device = _require_gpu(options.device)
+        arch, cfg = load_config(model_dir)
+        model = DecoderModel(arch.build_spec(cfg))
+        loader = WeightLoader(model_dir, device, _DTYPES[options.dtype])
+        try:
+            model.load(loader)
+        finally:
+            loader.close()
+        r = cls(model, options, device)
+        r.config = cfg
+        return r
+
+    @classmethod
+    def from_config(cls, cfg, options: EngineOptions, seed: int = 0) -> "ModelRunner":
+        """Random weights drawn on the device (measurements; no file is written)."""
+        from ..config import get_architecture
+        device = _require_gpu(options.device)
+        model = DecoderModel(get_architecture(cfg.ARCHITECTURE).build_spec(cfg))
+        model.load_random(seed, device, _DTYPES[options.dtype])
+        r = cls(model, options, device)
+        r.config = cfg
+        return r
+
+    def _build_caches(self) -> None:
+        opt = self.options
+        needs = self.model.cache_needs()
+        self.max_blocks_per_seq = -(-opt.max_model_len // self.page_size)
+        # groups: run entries whose KV needs coincide share block tables
+        keys: list[tuple] = []
+        entry_group: list[int | None] = []
+        for need in needs:
+            if isinstance(need, KVSpec):
+                k = need.group_key()
+                if k not in keys:
+                    keys.append(k)
+                entry_group.append(keys.index(k))
+            else:
+                entry_group.append(None)
+        esize = torch.empty((), dtype=self.dtype).element_size()
+        page_bytes = sum(2 * n.kv_heads * n.head_dim * self.page_size * esize for n in needs if isinstance(n, KVSpec))
+        state_bytes = 0
+        for n in needs:
+            if isinstance(n, StateSpec):
+                e = torch.empty((), dtype=getattr(torch, n.dtype)).element_size()
+                numel = 1
+                for s in n.shape:
+                    numel *= s
+                state_bytes += numel * e * opt.max_num_seqs
+        if opt.num_blocks is not None:
+            num_blocks = opt.num_blocks
+        else:
+            # weights and activation buffers are allocated; the cache takes what is left
+            # (models/qwen3/src/model.rs:545-603): min(free, total * util - used) - reserve - logits
+            free, total = torch.cuda.mem_get_info(self.device)
+            used = total - free
+            reserve = 512 << 20
+            budget = min(free, int(total * opt.gpu_memory_utilization) - used) - reserve - state_bytes
+            budget -= 3 * self.max_rows * self.model.spec.vocab_size * 4
+            num_blocks = budget // max(page_bytes, 1) if page_bytes else 1
+            if num_blocks <= 0:
+                raise RuntimeError("no memory is left for the cache after weights and buffers")
+        if keys and self.max_blocks_per_seq > num_blocks:
+            raise RuntimeError(f"one request of max_model_len {opt.max_model_len} needs {self.max_blocks_per_seq} "
+                               f"pages, the pool has {num_blocks}")
+        self.num_blocks = int(num_blocks)
+        self.group_specs = [GroupSpec(self.page_size, self.num_blocks, window=k[3]) for k in keys]
+        self.cache = CacheManager(self.group_specs, opt.max_num_seqs)
+        self.cache_views: list[CacheView] = []
+        self.state_tensors: list[torch.Tensor] = []
+        own: dict[int, CacheView] = {}
+        for i, (e, need) in enumerate(zip(self.model.run, needs)):
+            if e.cache != i:
+                src = own[e.cache]
+                self.cache_views.append(CacheView(src.group, src.k, src.v, owner=False, state=src.state))
+                continue
+            if isinstance(need, KVSpec):
+                k = torch.empty((self.num_blocks, need.kv_heads, self.page_size, need.head_dim),
+                                dtype=self.dtype, device=self.device)
+                v = torch.empty((self.num_blocks, need.kv_heads, need.head_dim, self.page_size),
+                                dtype=self.dtype, device=self.device)
+                view = CacheView(entry_group[i], k, v, owner=True)
+            elif isinstance(need, StateSpec):
+                st = torch.zeros((opt.max_num_seqs, *need.shape), dtype=getattr(torch, need.dtype), device=self.device)
+                self.state_tensors.append(st)
+                view = CacheView(None, None, None, owner=True, state=st)
+            else:
+                view = CacheView(None, None, None, owner=True)
+            own[i] = view
+            self.cache_views.append(view)
+
+    # ---- the step function ---------------------------------------------------------------------
+    def step(self, entries: list[Entry]) -> torch.Tensor:
+        """Runs one batch. Pages for every entry's tokens must have been allocated.
+        Returns float32 logits [sum(len(e.want)), vocab] in the order of entries and of want
+        (a view of a buffer that the next step overwrites)."""
+        b = self.batch
+        b.fill(entries, self.cache)
+        b.upload()
+        fresh = self.cache.take_fresh_slots()
+        if fresh and self.state_tensors:
+            idx = torch.tensor(fresh, device=self.device, dtype=torch.long)
+            for st in self.state_tensors:
+                st.index_fill_(0, idx, 0)
+        return self.model.forward(b, self.cache_views)
+
+    # ---- request bookkeeping shared by replay and tests ------------------------------------------
+    def reserve(self, req_id, start: int, n: int) -> bool:
+        """Admits the request if new and allocates pages for tokens [start, start + n)."""
+        if not self.cache.has(req_id):
+            self.cache.admit(req_id)
+        return self.cache.allocate(req_id, start, n)
+
+    def advance(self, req_id, num_computed: int) -> None:
+        """After a step: gives back pages a window has passed."""
+        self.cache.release_passed(req_id, num_computed)
+
+    def finish(self, req_id) -> None:
+        self.cache.free(req_id)

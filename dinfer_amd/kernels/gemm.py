@@ -1,0 +1,28 @@
+"""Matrix products out = a . w^T.
+
+float32 operands: the vector-ALU kernel with a fixed summation order (the true
+32-bit path). bfloat16 operands: the hand-written MFMA kernel that streams the
+weight once for few rows (decode, LM head), and the vendor library for many
+rows, where the reference uses a library too (crates/kernels/src/gemm.rs:605-647).
+"""
+from __future__ import annotations
+
+import torch
+
+from . import ops
+
+
+def matmul_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int) -> torch.Tensor:
+    """out[:m] = a[:m] @ w.T; out has a's dtype, or float32 (logits)."""
+    if m <= 0:
+        return out
+    if a.dtype == torch.float32:
+        return ops.gemm_ref(a, w, out, m)
+    if not a.is_cuda:
+        raise RuntimeError("matrix products run on the GPU only")
+    if out.dtype == torch.float32:
+        tmp = torch.mm(a[:m], w.t())
+        ops.widen(tmp, out, m * w.shape[0]) if out.is_contiguous() else out[:m].copy_(tmp)
+        return out
+    torch.mm(a[:m], w.t(), out=out[:m])
+    return out

@@ -1,0 +1,101 @@
+"""Loads the compiled HIP libraries through ctypes and declares their C ABI.
+
+There is no fallback: if a library is missing it is compiled; if that fails, or
+no GPU is present when a kernel is called, the call raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import sys
+import threading
+from ctypes import c_float, c_int, c_int64, c_uint32, c_void_p
+
+from ..csrc import build as _build
+
+_P = c_void_p
+_I = c_int
+_L = c_int64
+_F = c_float
+
+# function name -> (library, argument types). Every function returns an int status.
+SIGNATURES = {
+    "dinfer_embedding": ("elementwise", [_I, _P, _P, _P, _L, _L, _L, _P]),
+    "dinfer_gated_act": ("elementwise", [_I, _I, _P, _P, _L, _L, _L, _P]),
+    "dinfer_add_inplace": ("elementwise", [_I, _P, _P, _L, _P]),
+    "dinfer_widen": ("elementwise", [_I, _P, _P, _L, _P]),
+    "dinfer_fill_u32": ("elementwise", [_P, c_uint32, _L, _P]),
+    "dinfer_rmsnorm": ("norm", [_I, _P, _P, _P, _P, _I, _P, _L, _L, _L, _L, _F, _F, _P]),
+    "dinfer_qkv_post": (
+        "rope",
+        [_I, _P, _L, _L, _L, _L, _L, _P, _P, _I, _F, _F, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _P],
+    ),
+    "dinfer_attn_paged_ref": (
+        "attention_ref",
+        [_I, _P, _L, _P, _L, _P, _P, _P, _L, _P, _P, _I, _L, _F, _I, _I, _I, _I, _I, _P],
+    ),
+    "dinfer_gemm_ref": ("gemm_ref", [_I, _I, _P, _L, _P, _L, _P, _L, _L, _L, _L, _P]),
+    "dinfer_argmax": ("sampling", [_P, _L, _P, _L, _L, _P]),
+    "dinfer_sample": ("sampling", [_P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _P]),
+    "dinfer_penalties": ("sampling", [_P, _L, _P, _P, _P, _P, _P, _P, _L, _L, _P]),
+}
+
+ERRORS = {
+    1: "unsupported dtype code",
+    2: "operand shapes or strides do not fit the kernel",
+    3: "size or option not supported by this kernel",
+    4: "kernel launch failed",
+    5: "workspace too small",
+}
+
+_libs: dict[str, ctypes.CDLL] = {}
+_funcs: dict[str, ctypes._CFuncPtr] = {}
+_lock = threading.Lock()
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def load_library(name: str) -> ctypes.CDLL:
+    with _lock:
+        lib = _libs.get(name)
+        if lib is not None:
+            return lib
+        path = _build.find_built(name)
+        if path is None:
+            path = _build.build(name)
+        elif _build.is_stale(name, path):
+            print(f"[dinfer_amd] warning: {path.name} is older than its source; rebuild with "
+                  f"`python -m dinfer_amd.csrc.build`", file=sys.stderr, flush=True)
+        try:
+            lib = ctypes.CDLL(str(path))
+        except OSError as e:
+            raise KernelError(f"cannot load {path}: {e}") from e
+        _libs[name] = lib
+        return lib
+
+
+def register(name: str, library: str, argtypes: list) -> None:
+    """Declares a further entry point (used by libraries added later)."""
+    SIGNATURES[name] = (library, argtypes)
+
+
+def get(name: str):
+    fn = _funcs.get(name)
+    if fn is None:
+        libname, argtypes = SIGNATURES[name]
+        fn = getattr(load_library(libname), name)
+        fn.argtypes = argtypes
+        fn.restype = c_int
+        _funcs[name] = fn
+    return fn
+
+
+def call(name: str, *args) -> None:
+    rc = get(name)(*args)
+    if rc != 0:
+        raise KernelError(f"{name}: {ERRORS.get(rc, f'status {rc}')}")
+
+
+def loaded_libraries() -> list[str]:
+    return sorted(_libs)

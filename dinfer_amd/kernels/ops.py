@@ -1,0 +1,237 @@
+"""Typed Python wrappers around the HIP kernels.
+
+Each wrapper checks on the host what the kernel assumes about its operands
+(device, dtype, strides, sizes) and launches on torch's current HIP stream, so
+the calls can be captured into a HIP graph like any other stream work.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import lib
+
+F32, BF16 = 0, 1
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    if dt == torch.float32:
+        return F32
+    if dt == torch.bfloat16:
+        return BF16
+    raise TypeError(f"kernels take float32 or bfloat16 storage, not {dt}")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _need_gpu(*tensors) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise lib.KernelError("kernel operands must live on the GPU; there is no CPU path")
+
+
+def _ptr(t) -> int:
+    return 0 if t is None else t.data_ptr()
+
+
+def _rows(t: torch.Tensor) -> int:
+    """Row stride of a 2-D tensor whose rows are contiguous."""
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise ValueError(f"expected a 2-D tensor with contiguous rows, got shape {tuple(t.shape)} stride {t.stride()}")
+    return t.stride(0)
+
+
+def _is_param_f32(w: torch.Tensor, act_dtype: torch.dtype) -> int:
+    if w.dtype == torch.float32:
+        return 1
+    if w.dtype != act_dtype:
+        raise TypeError(f"a parameter vector must be float32 or the activation dtype {act_dtype}, not {w.dtype}")
+    return 0
+
+
+def embedding(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t] = table[ids[t]]; ids int32 [T], table [V, W], out [T, W]."""
+    _need_gpu(ids, table, out)
+    assert ids.dtype == torch.int32 and ids.is_contiguous()
+    assert table.is_contiguous() and out.is_contiguous() and table.dtype == out.dtype
+    T = ids.numel()
+    V, W = table.shape
+    assert out.shape[0] >= T and out.shape[1] == W
+    lib.call("dinfer_embedding", dtype_code(table.dtype), ids.data_ptr(), table.data_ptr(), out.data_ptr(), T, V, W,
+             _stream())
+    return out
+
+
+def gated_act(gate_up: torch.Tensor, out: torch.Tensor, tokens: int, act: str = "silu") -> torch.Tensor:
+    """out[t, i] = act(gate_up[t, i]) * gate_up[t, I + i]."""
+    _need_gpu(gate_up, out)
+    if act != "silu":
+        raise lib.KernelError(f"gated activation {act!r} has no kernel (only 'silu')")
+    inter = out.shape[1]
+    assert gate_up.shape[1] == 2 * inter and gate_up.dtype == out.dtype and out.is_contiguous()
+    assert gate_up.shape[0] >= tokens and out.shape[0] >= tokens
+    lib.call("dinfer_gated_act", dtype_code(out.dtype), 0, gate_up.data_ptr(), out.data_ptr(), tokens, inter,
+             _rows(gate_up), _stream())
+    return out
+
+
+def add_inplace(dst: torch.Tensor, src: torch.Tensor, n: int | None = None) -> None:
+    """dst[:n] += src[:n] (flat), summed in float and rounded once."""
+    _need_gpu(dst, src)
+    assert dst.dtype == src.dtype and dst.is_contiguous() and src.is_contiguous()
+    n = dst.numel() if n is None else n
+    assert n <= dst.numel() and n <= src.numel()
+    lib.call("dinfer_add_inplace", dtype_code(dst.dtype), dst.data_ptr(), src.data_ptr(), n, _stream())
+
+
+def widen(src: torch.Tensor, dst: torch.Tensor, n: int | None = None) -> None:
+    _need_gpu(src, dst)
+    assert dst.dtype == torch.float32 and dst.is_contiguous() and src.is_contiguous()
+    n = src.numel() if n is None else n
+    lib.call("dinfer_widen", dtype_code(src.dtype), src.data_ptr(), dst.data_ptr(), n, _stream())
+
+
+def fill_zero(t: torch.Tensor) -> None:
+    """Zero-fills a tensor with a kernel (safe inside a captured graph)."""
+    _need_gpu(t)
+    nbytes = t.numel() * t.element_size()
+    assert t.is_contiguous() and nbytes % 4 == 0 and t.data_ptr() % 4 == 0
+    lib.call("dinfer_fill_u32", t.data_ptr(), 0, nbytes // 4, _stream())
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, eps: float, n_rows: int, *,
+            residual: torch.Tensor | None = None, rows: torch.Tensor | None = None,
+            weight_offset: float = 0.0) -> torch.Tensor:
+    """out[r] = rmsnorm(x[src(r)]) * (weight + weight_offset).
+
+    residual: updated in place to round(x + residual) first, and that sum is normed.
+    rows: int32 indices of the n_rows source rows (gather); default identity.
+    """
+    _need_gpu(x, weight, out, residual, rows)
+    width = out.shape[1]
+    assert x.shape[1] == width and weight.numel() == width and weight.is_contiguous() and out.is_contiguous()
+    assert x.dtype == out.dtype and out.shape[0] >= n_rows
+    if rows is None:
+        assert x.shape[0] >= n_rows
+    else:
+        assert rows.dtype == torch.int32 and rows.is_contiguous() and rows.numel() >= n_rows
+    if residual is not None:
+        assert residual.dtype == x.dtype and residual.shape == x.shape
+    lib.call("dinfer_rmsnorm", dtype_code(x.dtype), x.data_ptr(), _ptr(residual), _ptr(rows), weight.data_ptr(),
+             _is_param_f32(weight, x.dtype), out.data_ptr(), n_rows, width, _rows(x),
+             _rows(residual) if residual is not None else 0, float(eps), float(weight_offset), _stream())
+    return out
+
+
+def qkv_post(qkv: torch.Tensor, tokens: int, *, heads: int, kv_heads: int, head_dim: int, q_off: int, k_off: int,
+             v_off: int, q_gain: torch.Tensor | None, k_gain: torch.Tensor | None, eps: float, gain_offset: float,
+             positions: torch.Tensor, cos_sin: torch.Tensor | None, rotary_dim: int, rope_style: int,
+             k_cache: torch.Tensor | None, v_cache: torch.Tensor | None, slot_mapping: torch.Tensor | None,
+             page_size: int) -> None:
+    """Per-head q/k norm, rotation, q written back in place, k and v written to the cache pages.
+
+    k_cache [blocks, kv_heads, page, D], v_cache [blocks, kv_heads, D, page]; slot_mapping int64 [T]
+    (None: nothing is written to the cache).
+    """
+    _need_gpu(qkv, q_gain, k_gain, positions, cos_sin, k_cache, v_cache, slot_mapping)
+    ld = _rows(qkv)
+    assert qkv.shape[0] >= tokens
+    assert max(q_off + heads * head_dim, k_off + kv_heads * head_dim, v_off + kv_heads * head_dim) <= qkv.shape[1]
+    assert positions.dtype == torch.int32 and positions.numel() >= tokens
+    wf32 = 0
+    if q_gain is not None:
+        assert q_gain.numel() == head_dim and k_gain is not None and k_gain.numel() == head_dim
+        wf32 = _is_param_f32(q_gain, qkv.dtype)
+        assert _is_param_f32(k_gain, qkv.dtype) == wf32
+    if cos_sin is not None:
+        assert cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and cos_sin.shape[1] == rotary_dim
+    if slot_mapping is not None:
+        assert slot_mapping.dtype == torch.int64 and slot_mapping.numel() >= tokens
+        assert k_cache is not None and v_cache is not None
+        nb = k_cache.shape[0]
+        assert tuple(k_cache.shape) == (nb, kv_heads, page_size, head_dim) and k_cache.is_contiguous()
+        assert tuple(v_cache.shape) == (nb, kv_heads, head_dim, page_size) and v_cache.is_contiguous()
+        assert k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype
+    lib.call("dinfer_qkv_post", dtype_code(qkv.dtype), qkv.data_ptr(), tokens, ld, q_off, k_off, v_off,
+             _ptr(q_gain), _ptr(k_gain), wf32, float(eps), float(gain_offset), positions.data_ptr(), _ptr(cos_sin),
+             rotary_dim, rope_style, _ptr(k_cache), _ptr(v_cache), _ptr(slot_mapping), heads, kv_heads, head_dim,
+             page_size, _stream())
+
+
+def attn_paged_ref(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                   block_table: torch.Tensor, cu_seqlens: torch.Tensor, seq_lens: torch.Tensor, num_reqs: int,
+                   tokens: int, *, scale: float, window: int, heads: int, kv_heads: int, head_dim: int,
+                   page_size: int) -> torch.Tensor:
+    """Plain paged attention (any head size); q is a view whose row t holds the heads at columns h*D."""
+    _need_gpu(q, out, k_cache, v_cache, block_table, cu_seqlens, seq_lens)
+    assert q.dtype == out.dtype == k_cache.dtype == v_cache.dtype
+    assert block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous()
+    assert block_table.shape[0] >= num_reqs
+    assert cu_seqlens.dtype == torch.int32 and cu_seqlens.numel() >= num_reqs + 1
+    assert seq_lens.dtype == torch.int32 and seq_lens.numel() >= num_reqs
+    nb = k_cache.shape[0]
+    assert tuple(k_cache.shape) == (nb, kv_heads, page_size, head_dim) and k_cache.is_contiguous()
+    assert tuple(v_cache.shape) == (nb, kv_heads, head_dim, page_size) and v_cache.is_contiguous()
+    assert q.shape[1] >= heads * head_dim and out.shape[1] >= heads * head_dim
+    assert q.shape[0] >= tokens and out.shape[0] >= tokens
+    lib.call("dinfer_attn_paged_ref", dtype_code(q.dtype), q.data_ptr(), _rows(q), out.data_ptr(), _rows(out),
+             k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1],
+             cu_seqlens.data_ptr(), seq_lens.data_ptr(), num_reqs, tokens, float(scale), int(window), heads,
+             kv_heads, head_dim, page_size, _stream())
+    return out
+
+
+def gemm_ref(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int) -> torch.Tensor:
+    """out[:m] = a[:m] @ w.T on the vector ALUs with float accumulation (true 32-bit for float operands)."""
+    _need_gpu(a, w, out)
+    n, k = w.shape
+    assert a.shape[1] == k and out.shape[1] == n and a.dtype == w.dtype
+    assert a.shape[0] >= m and out.shape[0] >= m
+    out_f32 = 1 if out.dtype == torch.float32 else 0
+    if not out_f32:
+        assert out.dtype == a.dtype
+    lib.call("dinfer_gemm_ref", dtype_code(a.dtype), out_f32, a.data_ptr(), _rows(a), w.data_ptr(), _rows(w),
+             out.data_ptr(), _rows(out), m, n, k, _stream())
+    return out
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor, rows: int) -> torch.Tensor:
+    _need_gpu(logits, out)
+    assert logits.dtype == torch.float32 and out.dtype == torch.int32 and out.numel() >= rows
+    lib.call("dinfer_argmax", logits.data_ptr(), _rows(logits), out.data_ptr(), rows, logits.shape[1], _stream())
+    return out
+
+
+def sample(logits: torch.Tensor, work: torch.Tensor | None, out: torch.Tensor, rows: int, *,
+           temperature: torch.Tensor | None, top_k: torch.Tensor | None = None, top_p: torch.Tensor | None = None,
+           min_p: torch.Tensor | None = None, seeds: torch.Tensor | None = None,
+           offsets: torch.Tensor | None = None) -> torch.Tensor:
+    """One token per row. temperature None: all rows greedy. seeds/offsets are int64 holding the uint64 bits."""
+    _need_gpu(logits, work, out, temperature, top_k, top_p, min_p, seeds, offsets)
+    vocab = logits.shape[1]
+    assert logits.dtype == torch.float32 and out.dtype == torch.int32 and out.numel() >= rows
+    if temperature is not None:
+        assert temperature.dtype == torch.float32 and temperature.numel() >= rows
+        assert work is not None and work.dtype == torch.float32 and work.is_contiguous()
+        assert work.numel() >= rows * vocab
+        assert seeds is not None and offsets is not None
+        assert seeds.dtype == torch.int64 and offsets.dtype == torch.int64
+        assert seeds.numel() >= rows and offsets.numel() >= rows
+    for t, dt in ((top_k, torch.int32), (top_p, torch.float32), (min_p, torch.float32)):
+        assert t is None or (t.dtype == dt and t.numel() >= rows)
+    lib.call("dinfer_sample", logits.data_ptr(), _rows(logits), _ptr(work), _ptr(temperature), _ptr(top_k),
+             _ptr(top_p), _ptr(min_p), _ptr(seeds), _ptr(offsets), out.data_ptr(), rows, vocab, _stream())
+    return out
+
+
+def penalties(logits: torch.Tensor, rows: int, ids: torch.Tensor, counts: torch.Tensor, offsets: torch.Tensor,
+              repetition: torch.Tensor, frequency: torch.Tensor, presence: torch.Tensor) -> None:
+    """In place on logits: per row, entries offsets[b]..offsets[b+1] list the distinct tokens of the
+    row's history with their count among the outputs (0: prompt only)."""
+    _need_gpu(logits, ids, counts, offsets, repetition, frequency, presence)
+    assert logits.dtype == torch.float32
+    assert ids.dtype == counts.dtype == offsets.dtype == torch.int32 and offsets.numel() >= rows + 1
+    lib.call("dinfer_penalties", logits.data_ptr(), _rows(logits), ids.data_ptr(), counts.data_ptr(),
+             offsets.data_ptr(), repetition.data_ptr(), frequency.data_ptr(), presence.data_ptr(), rows,
+             logits.shape[1], _stream())

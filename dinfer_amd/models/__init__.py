@@ -1,0 +1,1 @@
+from . import qwen3  # noqa: F401  (registers Qwen3ForCausalLM)

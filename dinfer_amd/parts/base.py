@@ -1,0 +1,116 @@
+"""Interfaces of the parts a model is put together from.
+
+Every part gets its sizes and constants as constructor parameters, lists the
+tensors it wants from the weight file under local names, takes them in
+``load``, reserves its activation buffers in ``bind`` and computes in
+``forward``. No part knows which model it is in or which layer it is.
+"""
+from __future__ import annotations
+
+from typing import Callable
+
+import torch
+
+from .spec import KVSpec, StateSpec, TensorSpec
+
+
+class Workspace:
+    """Activation buffers [max_tokens, cols], shared by name between layers.
+
+    Layers run one after the other, so two layers asking for the same
+    (name, cols, dtype) get the same memory. Addresses never change after
+    ``bind``, which lets a step be captured as a HIP graph.
+    """
+
+    def __init__(self, device, dtype: torch.dtype, max_tokens: int):
+        self.device, self.dtype, self.max_tokens = device, dtype, max_tokens
+        self._bufs: dict[tuple, torch.Tensor] = {}
+
+    def buffer(self, name: str, cols: int, dtype: torch.dtype | None = None, rows: int | None = None) -> torch.Tensor:
+        dt = dtype or self.dtype
+        r = rows or self.max_tokens
+        k = (name, cols, dt, r)
+        b = self._bufs.get(k)
+        if b is None:
+            b = torch.empty((r, cols), dtype=dt, device=self.device)
+            self._bufs[k] = b
+        return b
+
+    def nbytes(self) -> int:
+        return sum(b.numel() * b.element_size() for b in self._bufs.values())
+
+
+class BuildContext:
+    """What a part may know about the engine it is built into."""
+
+    def __init__(self, device, dtype: torch.dtype, max_tokens: int, max_rows: int, page_size: int):
+        self.device, self.dtype = device, dtype
+        self.max_tokens, self.max_rows, self.page_size = max_tokens, max_rows, page_size
+        self.workspace = Workspace(device, dtype, max_tokens)
+
+
+class Part:
+    def tensors(self) -> dict[str, TensorSpec]:
+        """Local tensor name -> what the weight file must hold for it."""
+        return {}
+
+    def load(self, get: Callable[..., torch.Tensor]) -> None:
+        """get(local_name, compute=False) returns the tensor on the device.
+        compute=True asks for the engine's dtype (matrix-product operands)."""
+
+    def bind(self, ctx: BuildContext) -> None:
+        """Reserves buffers; called once before the first forward."""
+
+
+class Norm(Part):
+    def forward(self, x, out, n_rows: int, *, residual=None, rows=None):
+        """out[r] = norm(x[src r]); with residual: residual = x + residual first, normed after."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """Gives the rotation table the mixer's kernel applies to q and k."""
+    rotary_dim: int = 0
+    style: int = 0  # 0: pairs (i, i + rotary_dim/2); 1: pairs (2i, 2i+1)
+
+    def table(self) -> torch.Tensor | None:
+        """float32 [max_positions, rotary_dim] = [cos | sin], or None for no rotation."""
+        return None
+
+
+class CacheView:
+    """The cache of one run entry as its mixer sees it.
+
+    group: index of the page group (block tables, slot mappings in the batch);
+    k, v: this entry's page tensors; owner: False if the pages belong to another
+    entry (read only); state: [max_seqs, *shape] tensor for fixed-size state.
+    """
+
+    def __init__(self, group: int | None = None, k=None, v=None, owner: bool = True, state=None):
+        self.group, self.k, self.v, self.owner, self.state = group, k, v, owner, state
+
+
+class Mixer(Part):
+    def cache_spec(self) -> KVSpec | StateSpec | None:
+        return None
+
+    def forward(self, x: torch.Tensor, batch, cache: CacheView) -> torch.Tensor:
+        """x [T, hidden] -> [T, hidden] (a workspace buffer; valid until the same part runs again)."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x: torch.Tensor, batch) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block(Part):
+    """Arrangement of norm, mixer and feed-forward around the residual stream.
+
+    forward(hidden, pending, batch, cache) -> pending': `hidden` is the residual
+    stream, updated in place; `pending` is a branch output not yet added to it
+    (None at the first layer). Deferring the add lets the next norm kernel do it.
+    """
+
+    def forward(self, hidden, pending, batch, cache: CacheView):
+        raise NotImplementedError
