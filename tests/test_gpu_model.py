@@ -57,3 +57,158 @@ def test_whole_prompt(model_dirs, name, dtype):
         check_logits(got, want, dtype, f"{name} whole prompt of {n}")
         r.finish("x")
     r.cache.check()
+
+
+# ---- replay helpers ------------------------------------------------------------------------------
+def replay(runner, steps):
+    """steps: list of (entries, ends); entries: list of (id, tokens, want). Returns {(id, position): row}."""
+    from dinfer_amd.engine.batch import Entry
+    computed, rows = {}, {}
+    for entries, ends in steps:
+        es = []
+        for rid, toks, want in entries:
+            start = computed.get(rid, 0)
+            assert runner.reserve(rid, start, len(toks)), f"out of pages for {rid}"
+            es.append(Entry(rid, toks, start, want))
+        if es:
+            logits = runner.step(es).double().cpu()
+            i = 0
+            for e in es:
+                for w in e.want:
+                    rows[(e.req_id, e.start + w)] = logits[i]
+                    i += 1
+                computed[e.req_id] = e.start + len(e.tokens)
+                runner.advance(e.req_id, computed[e.req_id])
+        for rid in ends:
+            runner.finish(rid)
+            del computed[rid]
+        runner.cache.check()
+    return rows
+
+
+def compare_rows(rows, plain_logits, dtype, what):
+    """plain_logits: {id: [T, V]}; every replayed row against the whole-sequence logits."""
+    assert rows, "nothing was replayed"
+    for rid in {k[0] for k in rows}:
+        pos = sorted(p for (r, p) in rows if r == rid)
+        got = torch.stack([rows[(rid, p)] for p in pos])
+        check_logits(got, plain_logits[rid][pos], dtype, f"{what} request {rid}")
+
+
+def cut(ids, sizes):
+    out, i, k = [], 0, 0
+    while i < len(ids):
+        n = sizes[k % len(sizes)]
+        out.append(ids[i:i + n])
+        i += n
+        k += 1
+    return out
+
+
+DTYPES = ["float32", "bfloat16"]
+NAMES = ["A", "B", "C"]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_prompt_then_decode_one_by_one(model_dirs, name, dtype):
+    cfg, w = plain.load(model_dirs[name])
+    r = make_runner(model_dirs[name], name, dtype)
+    ids = tokens_for(name, 100, 5)
+    want = {"x": plain.forward(cfg, w, ids)}
+    steps = [([("x", ids[:68], [67])], [])]
+    steps += [([("x", [ids[p]], [0])], []) for p in range(68, 100)]
+    compare_rows(replay(r, steps), want, dtype, f"{name} decode after prompt")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_portions_of_changing_size(model_dirs, name, dtype):
+    cfg, w = plain.load(model_dirs[name])
+    r = make_runner(model_dirs[name], name, dtype)
+    ids = tokens_for(name, 117, 6)
+    want = {"x": plain.forward(cfg, w, ids)}
+    steps = [([("x", part, list(range(len(part))))], []) for part in cut(ids, [7, 16, 2, 5, 3, 33, 2, 8, 1])]
+    compare_rows(replay(r, steps), want, dtype, f"{name} portions")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_mixed_requests_with_reused_pages(model_dirs, name, dtype):
+    """Up to four live requests, portions of some beside decoded tokens of others; the pool is
+    so small that pages of finished requests go to later ones while stale keys still lie in them."""
+    cfg, w = plain.load(model_dirs[name])
+    page = PAGE[name]
+    lens = {"a": 70, "b": 41, "c": 9, "d": 55, "e": 64, "f": 1, "g": 37}
+    seqs = {k: tokens_for(name, n, 100 + i) for i, (k, n) in enumerate(lens.items())}
+    want = {k: plain.forward(cfg, w, v) for k, v in seqs.items()}
+    # a, b, c, d start; as each ends the next of e, f, g takes its pages
+    pool_tokens = sum(-(-lens[k] // page) * page for k in "abde") + 2 * page
+    r = make_runner(model_dirs[name], name, dtype, num_blocks=pool_tokens // page, max_len=128)
+    rng = random.Random(9)
+    todo = list(seqs)
+    live, fed, steps = [], {}, []
+    while todo or live:
+        while todo and len(live) < 4:
+            k = todo.pop(0)
+            live.append(k)
+            fed[k] = 0
+        entries, ends = [], []
+        for k in list(live):
+            left = lens[k] - fed[k]
+            if fed[k] > 0 and left <= 12:
+                n = 1  # decode the tail one by one
+            elif rng.random() < 0.2 and fed[k] > 0:
+                continue  # left out of this step, goes on later
+            else:
+                n = min(left, rng.choice([2, 3, 5, 8, 13, 16, 21]))
+            entries.append((k, seqs[k][fed[k]:fed[k] + n], list(range(n))))
+            fed[k] += n
+            if fed[k] == lens[k]:
+                ends.append(k)
+                live.remove(k)
+        steps.append((entries, ends))
+    rows = replay(r, steps)
+    assert len(rows) == sum(lens.values())
+    compare_rows(rows, want, dtype, f"{name} mixed")
+    assert r.cache.num_free(0) == r.num_blocks
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_decoding(model_dirs, dtype):
+    """Three requests decoded side by side for 200 steps from short prompts."""
+    name = "C"
+    cfg, w = plain.load(model_dirs[name])
+    r = make_runner(model_dirs[name], name, dtype, max_len=256)
+    seqs = {k: tokens_for(name, 3 + 200 + i, 40 + i) for i, k in enumerate("pqr")}
+    want = {k: plain.forward(cfg, w, v) for k, v in seqs.items()}
+    steps = [([(k, v[:3 + i], [2 + i]) for i, (k, v) in enumerate(seqs.items())], [])]
+    for s in range(200):
+        steps.append(([(k, [v[3 + i + s]], [0]) for i, (k, v) in enumerate(seqs.items())], []))
+    compare_rows(replay(r, steps), want, dtype, "long decoding")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_first_tokens(model_dirs, name, dtype):
+    """The first positions of a sequence, fed one token a step from the very first."""
+    cfg, w = plain.load(model_dirs[name])
+    r = make_runner(model_dirs[name], name, dtype)
+    ids = tokens_for(name, 6, 77)
+    want = {"x": plain.forward(cfg, w, ids)}
+    steps = [([("x", [t], [0])], []) for t in ids]
+    compare_rows(replay(r, steps), want, dtype, f"{name} first tokens")
+
+
+def test_modes_agree_closely_in_32bit(model_dirs):
+    """In 32-bit every row's arithmetic is fixed by its own position: whole, token by token and
+    chunked replays give the same logits to the last bits (not merely within the plain tolerance)."""
+    name = "B"
+    r = make_runner(model_dirs[name], name, "float32")
+    ids = tokens_for(name, 60, 8)
+    whole = replay(r, [([("x", ids, list(range(60)))], ["x"])])
+    single = replay(r, [([("y", [t], [0])], []) for t in ids])
+    parts = replay(r, [([("z", p, list(range(len(p))))], []) for p in cut(ids, [7, 2, 16, 5])])
+    for p in range(60):
+        assert torch.equal(whole[("x", p)], single[("y", p)]), f"position {p}: token-by-token differs"
+        assert torch.equal(whole[("x", p)], parts[("z", p)]), f"position {p}: portions differ"
