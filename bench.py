@@ -1,0 +1,159 @@
+#!/usr/bin/env python3
+"""In-process throughput of the engine on one MI355X: Qwen3-8B-shaped random weights.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L]
+
+Prints ONE JSON line. `value` is decoded tokens per second at the default batch (8), each
+request with a 2,048-token prompt in a 4,096-token context; a "step" is one decode step
+through the engine's entry point (schedule, batch build, model step, greedy sampling,
+token ids back on the host). On the same line:
+
+  prefill   tokens per second of one 2,048-token prompt step; `frac` = the step's flops /
+            time / the dense bf16 MFMA peak (2.5 PFLOP/s; fp32: 157.3 TFLOP/s);
+  roofline  the decode step against HBM: bytes it has to read (every weight it uses once,
+            and the cache of the live requests) / time, against 8 TB/s;
+  points    decode tokens per second at batch 1 and 64.
+
+All data is synthetic: weights N(0, 0.02) / gains 1 + N(0, 0.1) drawn on the device, token
+ids uniform in the vocabulary. The reference publishes no number for this size or
+hardware, so vs_baseline is null.
+"""
+import argparse
+import json
+import random
+import sys
+import time
+from pathlib import Path
+
+sys.path.insert(0, str(Path(__file__).resolve().parent))
+
+# Qwen3-8B layer sizes (BASELINE.json configs[2])
+SIZES = dict(vocab_size=151936, hidden_size=4096, intermediate_size=12288, num_hidden_layers=36,
+             num_attention_heads=32, num_key_value_heads=8, head_dim=128, rms_norm_eps=1e-6, rope_theta=1e6,
+             max_position_embeddings=40960, tie_word_embeddings=False)
+PROMPT, CONTEXT = 2048, 4096
+HBM_PEAK = 8.0e12
+MFMA_PEAK = {"bfloat16": 2.5e15, "float32": 157.3e12}
+
+
+def model_numbers(c, dtype_bytes):
+    Hd, I, L = c["hidden_size"], c["intermediate_size"], c["num_hidden_layers"]
+    H, Hkv, D, V = c["num_attention_heads"], c["num_key_value_heads"], c["head_dim"], c["vocab_size"]
+    per_layer = (H + 2 * Hkv) * D * Hd + H * D * Hd + 3 * I * Hd
+    gains = L * (2 * Hd + 2 * D) + Hd
+    return dict(linear_params=L * per_layer, head_params=V * Hd, gains=gains,
+                kv_bytes_per_token=L * 2 * Hkv * D * dtype_bytes)
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=32)
+    ap.add_argument("--warmup", type=int, default=4)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration has (named in config)")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
+    ap.add_argument("--no-hip-graph", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print(f"bench.py measures one GPU only (this engine does not use a second one); got --gpus {a.gpus}")
+        return 2
+
+    import torch
+    from dinfer_amd import Engine, SamplingParams
+    from dinfer_amd.config.qwen3 import Qwen3Config
+
+    sizes = dict(SIZES)
+    full_layers = sizes["num_hidden_layers"]
+    if a.layers:
+        sizes["num_hidden_layers"] = a.layers
+    cfg = Qwen3Config.from_dict(sizes)
+    dbytes = 2 if a.dtype == "bfloat16" else 4
+    nums = model_numbers(sizes, dbytes)
+    max_b = max(a.batch, 1 if a.no_points else 64)
+    page = 16
+    eng = Engine(config=cfg, seed=0, dtype=a.dtype, max_model_len=CONTEXT, max_num_seqs=max_b,
+                 max_num_batched_tokens=PROMPT, block_size=page, num_blocks=max_b * CONTEXT // page + 64,
+                 hip_graph=not a.no_hip_graph)
+    rng = random.Random(0)
+    V = cfg.vocab_size
+
+    def prompt():
+        return [rng.randrange(V) for _ in range(PROMPT)]
+
+    def sync():
+        torch.cuda.synchronize()
+
+    greedy = SamplingParams(max_tokens=CONTEXT - PROMPT, temperature=0.0, ignore_eos=True)
+
+    # ---- prefill: one request, one step of 2,048 tokens (the step also samples its first token)
+    def time_prefill():
+        rid = eng.add_request(prompt(), greedy)
+        sync()
+        t0 = time.perf_counter()
+        eng.step()
+        sync()
+        dt = time.perf_counter() - t0
+        eng.abort(rid)
+        return dt
+
+    time_prefill()  # warm-up: library initialisation, first-use allocations
+    pre = min(time_prefill() for _ in range(3))
+    attn_flops = sizes["num_hidden_layers"] * 2 * PROMPT * PROMPT * cfg.head_dim * cfg.num_attention_heads
+    pre_flops = 2 * PROMPT * nums["linear_params"] + attn_flops + 2 * nums["head_params"]
+    prefill = {"value": round(PROMPT / pre, 1), "tokens": PROMPT, "ms": round(pre * 1e3, 3),
+               "frac": round(pre_flops / pre / MFMA_PEAK[a.dtype], 4)}
+
+    # ---- decode at a batch: B requests prefilled to 2,048 tokens, then timed decode steps
+    def decode(batch, steps, warmup):
+        ids = [eng.add_request(prompt(), greedy) for _ in range(batch)]
+        while any(r.num_computed < PROMPT for r in eng.scheduler.requests.values()):
+            eng.step()
+        for _ in range(warmup):
+            eng.step()
+        sync()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            eng.step()
+        sync()
+        dt = (time.perf_counter() - t0) / steps
+        ctx = PROMPT + 1 + warmup + steps / 2  # mean cached tokens per request over the timed steps
+        for i in ids:
+            eng.abort(i)
+        return dt, ctx
+
+    dt, ctx = decode(a.batch, a.steps, a.warmup)
+    weight_bytes = (nums["linear_params"] + nums["head_params"] + nums["gains"] + a.batch * cfg.hidden_size) * dbytes
+    step_bytes = weight_bytes + a.batch * ctx * nums["kv_bytes_per_token"]
+    achieved = step_bytes / dt
+    points = {}
+    if not a.no_points:
+        for b in (1, 64):
+            d, _ = decode(b, a.steps, a.warmup)
+            points[f"decode_b{b}"] = round(b / d, 1)
+
+    line = {
+        "metric": "decode tok/s (Qwen3-8B shape, batch 8, 2048-token prompts, context 4096)",
+        "value": round(a.batch / dt, 1), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if a.dtype == "bfloat16" else "fp32", "data": "synthetic",
+        "config": {
+            "model": "Qwen3-8B shape, random weights", "global_batch": a.batch, "seq_len": CONTEXT,
+            "prompt_len": PROMPT, "parallelism": "single GPU", "layers": sizes["num_hidden_layers"],
+            "layers_of_config": full_layers, "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads,
+            "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size,
+            "vocab": cfg.vocab_size, "rope_theta": cfg.rope_theta, "rms_norm_eps": cfg.rms_norm_eps,
+            "tied_head": cfg.tie_word_embeddings, "page_size": page, "hip_graph": not a.no_hip_graph,
+        },
+        "prefill": prefill,
+        "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK, 4)},
+        "points": points,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

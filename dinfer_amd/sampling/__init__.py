@@ -1,0 +1,3 @@
+from .params import GREEDY_EPS, SamplingParams
+
+__all__ = ["GREEDY_EPS", "SamplingParams"]

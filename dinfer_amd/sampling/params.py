@@ -1,0 +1,55 @@
+"""Sampling options of a request: names, defaults and ranges of the reference's
+SamplingParams (crates/core/src/sample.rs:81-139, validate :157-205), without the
+text-level and server-level fields (stop strings, logprobs, logit_bias, grammar).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+GREEDY_EPS = 1e-5  # temperature at or below this is greedy (sample.rs:143-145)
+
+
+@dataclass
+class SamplingParams:
+    max_tokens: int = 256
+    min_tokens: int = 0            # eos / stop ids are ignored until this many outputs
+    temperature: float = 1.0
+    top_p: float = 1.0
+    top_k: int = -1
+    min_p: float = 0.0
+    repetition_penalty: float = 1.0
+    frequency_penalty: float = 0.0
+    presence_penalty: float = 0.0
+    seed: int | None = None        # None: drawn at admission
+    stop_token_ids: list = field(default_factory=list)
+    ignore_eos: bool = False
+
+    @property
+    def is_greedy(self) -> bool:
+        return self.temperature <= GREEDY_EPS
+
+    @property
+    def has_penalties(self) -> bool:
+        return self.repetition_penalty != 1.0 or self.frequency_penalty != 0.0 or self.presence_penalty != 0.0
+
+    def validate(self) -> None:
+        if self.temperature < 0.0:
+            raise ValueError(f"temperature must be non-negative, got {self.temperature}")
+        if not (0.0 < self.top_p <= 1.0):
+            raise ValueError(f"top_p must be in (0, 1], got {self.top_p}")
+        if self.top_k < -1 or self.top_k == 0:
+            raise ValueError(f"top_k must be -1 (disable) or at least 1, got {self.top_k}")
+        if not (0.0 <= self.min_p <= 1.0):
+            raise ValueError(f"min_p must be in [0, 1], got {self.min_p}")
+        if not (0.0 < self.repetition_penalty <= 2.0):
+            raise ValueError(f"repetition_penalty must be in (0, 2], got {self.repetition_penalty}")
+        if not (-2.0 <= self.frequency_penalty <= 2.0):
+            raise ValueError(f"frequency_penalty must be in [-2, 2], got {self.frequency_penalty}")
+        if not (-2.0 <= self.presence_penalty <= 2.0):
+            raise ValueError(f"presence_penalty must be in [-2, 2], got {self.presence_penalty}")
+        if self.max_tokens < 1:
+            raise ValueError("max_tokens must be at least 1")
+        if self.min_tokens > self.max_tokens:
+            raise ValueError(f"min_tokens {self.min_tokens} > max_tokens {self.max_tokens}")
+        if self.seed is not None and not (0 <= self.seed < 1 << 64):
+            raise ValueError(f"seed must fit 64 unsigned bits, got {self.seed}")
