@@ -1,0 +1,421 @@
+// MFMA attention over the paged cache for bf16, gfx950.
+//
+// Both kernels compute S^T = K . Q^T and O^T = V^T . P with
+// v_mfma_f32_16x16x32_bf16, whose operands want, per lane, 8 consecutive
+// elements of the contraction dimension:
+//   A (16 x 32): lane l holds A[l % 16][8 * (l / 16) .. + 8]
+//   B (32 x 16): lane l holds B[8 * (l / 16) .. + 8][l % 16]
+//   D (16 x 16): lane l holds D[4 * (l / 16) + r][l % 16], r = 0..3
+// K pages [Hkv][page][D] give A = K rows straight from memory (contraction over
+// d); V pages [Hkv][D][page] (transposed) give A = V^T rows straight from memory
+// (contraction over keys). Nothing is staged through LDS.
+//
+// A block of 32 keys is scored by two MFMA chains (a = 0, 1). Row i of chain a
+// is key  kb + 8 * (i / 4) + 4 * a + (i % 4),  so lane group g = l / 16 ends up
+// with the scores of keys kb + 8 g .. kb + 8 g + 7 in its eight result
+// registers: exactly the B operand of the P.V product, with no shuffle.
+// A query (a column, l % 16) keeps its running maximum, sum and output column in
+// the same lanes through both products.
+//
+//   flash:  query rows with or without history, causal, optional window; one
+//           wave owns QT x 16 query rows of one head and walks its keys in
+//           blocks of 32 (online softmax in base 2).
+//   decode: all requests bring one row; the G query heads of a kv head are the
+//           16 columns, so K and V are read once per group; the keys are split
+//           over workgroups, each writing (m, l, o) partials; a merge kernel
+//           combines them.
+//
+// Sizes: head_dim a multiple of 16 from the instantiated list, page size a
+// multiple of 8, G <= 16 for decode. Anything else is refused (the caller then
+// uses the plain kernel).
+//
+// Reference behaviour: crates/kernels/cuda/gqa.cu:167-369 (flash prefill and
+// paged: 64-key tiles, base-2 online softmax, P rounded to bf16 before P.V),
+// gqa_decode_v3_core.cuh:72-242 and gqa.cu:1423-1461 (split-K decode, merge of
+// (m, l, o) partials).
+#include "common.cuh"
+
+using namespace dinfer;
+
+namespace {
+
+constexpr float LOG2E = 1.4426950408889634f;
+
+__device__ __forceinline__ bf16x8 zero8() {
+  bf16x8 z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = (bf16)0.f;
+  return z;
+}
+
+__device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+// One block of 32 keys against NT column tiles. Shared by both kernels.
+//   qf[t][ks]   B operands of the score product (queries or heads), whole head in registers
+//   col_lo/hi   per column tile and lane: the column's visible keys are [col_lo, col_hi)
+//   k_lo, k_hi  the keys this wave may touch at all (held pages, written slots)
+template <int DT, int NT>
+struct Tile {
+  static constexpr int KS = (DT + 1) / 2;  // 32-wide steps over the head dimension
+  f32x4 o[NT][DT];
+  float m[NT], l[NT];
+
+  __device__ __forceinline__ void init() {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      m[t] = -INFINITY;
+      l[t] = 0.f;
+#pragma unroll
+      for (int d = 0; d < DT; ++d) o[t][d] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+  }
+
+  __device__ __forceinline__ void block(const bf16x8 (&qf)[NT][KS], int kb, int k_lo, int k_hi, const int (&col_lo)[NT],
+                                        const int (&col_hi)[NT], bool need_mask, const bf16* __restrict__ kc,
+                                        const bf16* __restrict__ vc, const int32_t* __restrict__ bt, int hk, int Hkv,
+                                        int D, int ps, float scale_log2e) {
+    const int lane = threadIdx.x & 63, i16 = lane & 15, g4 = lane >> 4;
+    // ---- scores ----
+    const int kg_row = kb + 8 * (i16 >> 2);  // the 8-key group of this lane's two K rows (one page: ps % 8 == 0)
+    const int key0 = kg_row + (i16 & 3), key1 = key0 + 4;
+    const bool v0 = key0 >= k_lo && key0 < k_hi, v1 = key1 >= k_lo && key1 < k_hi;
+    const bf16* krow = kc;
+    if (v0 || v1) {
+      const int pg = bt[kg_row / ps];
+      krow = kc + (((int64_t)pg * Hkv + hk) * ps + (kg_row % ps) + (i16 & 3)) * D;
+    }
+    f32x4 s[NT][2];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) s[t][0] = s[t][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d = ks * 32 + g4 * 8;
+      const bool dv = d < D;  // D % 32 == 16: the upper half of the last step is padding
+      const bf16x8 k0 = (v0 && dv) ? *(const bf16x8*)(krow + d) : zero8();
+      const bf16x8 k1 = (v1 && dv) ? *(const bf16x8*)(krow + 4 * D + d) : zero8();
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        s[t][0] = mfma16(k0, qf[t][ks], s[t][0]);
+        s[t][1] = mfma16(k1, qf[t][ks], s[t][1]);
+      }
+    }
+    // ---- online softmax per column; this lane holds keys kb + 8 g4 + {0..7} of column i16 ----
+    const int kg = kb + 8 * g4;
+    bf16x8 pf[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      float x[8];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        x[r] = s[t][0][r] * scale_log2e;
+        x[4 + r] = s[t][1][r] * scale_log2e;
+      }
+      if (need_mask) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (kg + e < col_lo[t] || kg + e >= col_hi[t]) x[e] = -INFINITY;
+      }
+      float mx = x[0];
+#pragma unroll
+      for (int e = 1; e < 8; ++e) mx = fmaxf(mx, x[e]);
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m[t], mx);
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;  // nothing visible yet: keep everything zero
+      const float alpha = exp2f(m[t] - m_use);
+      m[t] = m_new;
+      float ps_ = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float p = exp2f(x[e] - m_use);
+        ps_ += p;
+        pf[t][e] = (bf16)p;
+      }
+      l[t] = l[t] * alpha + ps_;  // partial over this lane's keys; lane groups are summed at the end
+#pragma unroll
+      for (int d = 0; d < DT; ++d) o[t][d] *= alpha;
+    }
+    // ---- O^T += V^T . P ----
+    const bool vg = kg < k_hi && kg + 8 > k_lo;
+    const bf16* vrow = vc;
+    if (vg) {
+      const int pg = bt[kg / ps];
+      vrow = vc + (((int64_t)pg * Hkv + hk) * D + i16) * ps + (kg % ps);
+    }
+#pragma unroll
+    for (int d = 0; d < DT; ++d) {
+      bf16x8 vf = vg ? *(const bf16x8*)(vrow + (int64_t)d * 16 * ps) : zero8();
+      if (need_mask && vg) {
+        // a stale slot may hold anything; its weight is 0, but 0 * inf would poison the sum
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (kg + e < k_lo || kg + e >= k_hi) vf[e] = (bf16)0.f;
+      }
+#pragma unroll
+      for (int t = 0; t < NT; ++t) o[t][d] = mfma16(vf, pf[t], o[t][d]);
+    }
+  }
+
+  // total of l over the four lane groups of a column
+  __device__ __forceinline__ float sum_l(int t) const {
+    float v = l[t];
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
+    return v;
+  }
+};
+
+template <int DT, int QT>
+__global__ void __launch_bounds__(256) attn_flash_kernel(
+    const bf16* __restrict__ q, int64_t ld_q, bf16* __restrict__ out, int64_t ld_out, const bf16* __restrict__ kc,
+    const bf16* __restrict__ vc, const int32_t* __restrict__ block_table, int64_t max_blocks,
+    const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_lens, int tiles_x, float scale_log2e,
+    int window, int H, int Hkv, int ps, int skip_single) {
+  constexpr int D = DT * 16;
+  constexpr int KS = (DT + 1) / 2;
+  constexpr int QW = 16 * QT;   // query rows per wave
+  constexpr int QB = QW * 4;    // per workgroup
+  // Block order: the head index runs fastest and visits kv heads round-robin, so that the
+  // workgroups an XCD receives (linear id modulo 8) share kv heads, and with them the L2 lines
+  // of K and V. Late query tiles (most keys) are issued first.
+  const int L = blockIdx.x;
+  const int e = L % H, rest = L / H;
+  const int tile = tiles_x - 1 - rest % tiles_x, b = rest / tiles_x;
+  const int G = H / Hkv;
+  const int hk = e % Hkv, h = hk * G + e / Hkv;
+  const int q_begin = cu_seqlens[b];
+  const int q_len = cu_seqlens[b + 1] - q_begin;
+  const int hist = seq_lens[b] - q_len;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, i16 = lane & 15, g4 = lane >> 4;
+  const int q0 = tile * QB + wave * QW;
+  if (q0 >= q_len) return;  // no workgroup barrier below
+  if (skip_single && q_len == 1) return;  // single rows go to the split-K kernel
+  const int32_t* bt = block_table + (int64_t)b * max_blocks;
+
+  bf16x8 qf[QT][KS];
+  int col_lo[QT], col_hi[QT];
+#pragma unroll
+  for (int t = 0; t < QT; ++t) {
+    const int row = q0 + t * 16 + i16;
+    const int rc = row < q_len ? row : q_len - 1;  // rows past the end compute something harmless, never stored
+    const bf16* qp = q + (int64_t)(q_begin + rc) * ld_q + (int64_t)h * D;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d = ks * 32 + g4 * 8;
+      qf[t][ks] = d < D ? *(const bf16x8*)(qp + d) : zero8();
+    }
+    const int pos = hist + rc;
+    col_hi[t] = pos + 1;
+    col_lo[t] = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
+  }
+  const int p_first = hist + q0;
+  const int p_last = hist + (q0 + QW < q_len ? q0 + QW : q_len) - 1;
+  const int k_hi = p_last + 1;
+  const int k_lo = window > 0 ? (p_first - window + 1 > 0 ? p_first - window + 1 : 0) : 0;
+
+  Tile<DT, QT> tl;
+  tl.init();
+  for (int kb = k_lo & ~31; kb < k_hi; kb += 32) {
+    const bool need_mask = kb + 31 > p_first || kb < k_lo || (window > 0 && kb < p_last - window + 1);
+    tl.block(qf, kb, k_lo, k_hi, col_lo, col_hi, need_mask, kc, vc, bt, hk, Hkv, D, ps, scale_log2e);
+  }
+#pragma unroll
+  for (int t = 0; t < QT; ++t) {
+    const float lt = tl.sum_l(t);
+    const float inv = lt > 0.f ? 1.f / lt : 0.f;
+    const int row = q0 + t * 16 + i16;
+    if (row < q_len) {
+      bf16* op = out + (int64_t)(q_begin + row) * ld_out + (int64_t)h * D + 4 * g4;
+#pragma unroll
+      for (int d = 0; d < DT; ++d) {
+        bf16x4 r;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) r[k] = (bf16)(tl.o[t][d][k] * inv);
+        *(bf16x4*)(op + d * 16) = r;
+      }
+    }
+  }
+}
+
+// One wave per (split, kv head, request). part: [B, H, splits, D + 4] float = (m in base-2 units, l, -, -, o[D]).
+template <int DT>
+__global__ void __launch_bounds__(64) attn_decode_kernel(
+    const bf16* __restrict__ q, int64_t ld_q, float* __restrict__ part, const bf16* __restrict__ kc,
+    const bf16* __restrict__ vc, const int32_t* __restrict__ block_table, int64_t max_blocks,
+    const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_lens, int keys_per_split, int splits,
+    float scale_log2e, int window, int H, int Hkv, int ps) {
+  constexpr int D = DT * 16;
+  constexpr int KS = (DT + 1) / 2;
+  const int sp = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
+  const int G = H / Hkv;
+  int row = b;  // without cu_seqlens every request has exactly one row
+  if (cu_seqlens) {
+    row = cu_seqlens[b];
+    if (cu_seqlens[b + 1] - row != 1) return;  // a longer run of rows belongs to the flash kernel
+  }
+  const int seq = seq_lens[b];
+  const int first = window > 0 ? (seq - window > 0 ? seq - window : 0) : 0;  // the row's position is seq - 1
+  const int k_lo = sp * keys_per_split > first ? sp * keys_per_split : first;
+  const int k_hi = (sp + 1) * keys_per_split < seq ? (sp + 1) * keys_per_split : seq;
+  if (k_lo >= k_hi) return;  // a dead split writes nothing; the merge kernel knows which are live
+  const int lane = threadIdx.x & 63, i16 = lane & 15, g4 = lane >> 4;
+  const int32_t* bt = block_table + (int64_t)b * max_blocks;
+
+  bf16x8 qf[1][KS];
+  {
+    const int hh = i16 < G ? i16 : 0;
+    const bf16* qp = q + (int64_t)row * ld_q + (int64_t)(hk * G + hh) * D;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d = ks * 32 + g4 * 8;
+      qf[0][ks] = (d < D && i16 < G) ? *(const bf16x8*)(qp + d) : zero8();
+    }
+  }
+  const int col_lo[1] = {k_lo}, col_hi[1] = {k_hi};
+  Tile<DT, 1> tl;
+  tl.init();
+  for (int kb = k_lo & ~31; kb < k_hi; kb += 32) {
+    const bool need_mask = kb < k_lo || kb + 32 > k_hi;
+    tl.block(qf, kb, k_lo, k_hi, col_lo, col_hi, need_mask, kc, vc, bt, hk, Hkv, D, ps, scale_log2e);
+  }
+  const float lt = tl.sum_l(0);
+  if (i16 < G) {
+    float* pp = part + (((int64_t)b * H + hk * G + i16) * splits + sp) * (D + 4);
+    if (g4 == 0) {
+      pp[0] = tl.m[0];
+      pp[1] = lt;
+    }
+#pragma unroll
+    for (int d = 0; d < DT; ++d) *(f32x4*)(pp + 4 + d * 16 + 4 * g4) = tl.o[0][d];
+  }
+}
+
+// out[b, h, :] = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s over the live splits.
+__global__ void __launch_bounds__(256) attn_decode_merge_kernel(const float* __restrict__ part, bf16* __restrict__ out,
+                                                                int64_t ld_out, const int32_t* __restrict__ cu_seqlens,
+                                                                const int32_t* __restrict__ seq_lens,
+                                                                int keys_per_split, int splits, int window, int H,
+                                                                int D) {
+  const int h = blockIdx.x, b = blockIdx.y;
+  int row = b;
+  if (cu_seqlens) {
+    row = cu_seqlens[b];
+    if (cu_seqlens[b + 1] - row != 1) return;
+  }
+  const int seq = seq_lens[b];
+  const int first = window > 0 ? (seq - window > 0 ? seq - window : 0) : 0;
+  const int s_lo = first / keys_per_split;
+  const int s_hi = (seq + keys_per_split - 1) / keys_per_split;
+  const float* pp = part + ((int64_t)b * H + h) * splits * (D + 4);
+  float M = -INFINITY;
+  for (int s = s_lo; s < s_hi; ++s) M = fmaxf(M, pp[(int64_t)s * (D + 4)]);
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    float acc = 0.f, L = 0.f;
+    for (int s = s_lo; s < s_hi; ++s) {
+      const float* ps_ = pp + (int64_t)s * (D + 4);
+      const float a = ps_[0] == -INFINITY ? 0.f : exp2f(ps_[0] - M);
+      acc += a * ps_[4 + d];
+      L += a * ps_[1];
+    }
+    out[(int64_t)row * ld_out + (int64_t)h * D + d] = (bf16)(L > 0.f ? acc / L : 0.f);
+  }
+}
+
+inline bool aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
+
+template <int DT>
+int launch_flash(const bf16* q, int64_t ld_q, bf16* out, int64_t ld_out, const bf16* kc, const bf16* vc,
+                 const int32_t* bt, int64_t max_blocks, const int32_t* cu, const int32_t* sl, int num_reqs,
+                 int max_q_len, float scale, int window, int H, int Hkv, int ps, int skip_single, hipStream_t stream) {
+  const float sl2 = scale * LOG2E;
+  if (max_q_len > 64) {
+    constexpr int QB = 2 * 16 * 4;
+    const int tiles = (max_q_len + QB - 1) / QB;
+    const int64_t blocks = (int64_t)tiles * H * num_reqs;
+    if (blocks > 0x7fffffff) return ERR_UNSUPPORTED;
+    attn_flash_kernel<DT, 2><<<(unsigned)blocks, 256, 0, stream>>>(q, ld_q, out, ld_out, kc, vc, bt, max_blocks, cu, sl,
+                                                                  tiles, sl2, window, H, Hkv, ps, skip_single);
+  } else {
+    constexpr int QB = 16 * 4;
+    const int tiles = (max_q_len + QB - 1) / QB;
+    const int64_t blocks = (int64_t)tiles * H * num_reqs;
+    if (blocks > 0x7fffffff) return ERR_UNSUPPORTED;
+    attn_flash_kernel<DT, 1><<<(unsigned)blocks, 256, 0, stream>>>(q, ld_q, out, ld_out, kc, vc, bt, max_blocks, cu, sl,
+                                                                  tiles, sl2, window, H, Hkv, ps, skip_single);
+  }
+  return launch_status();
+}
+
+template <int DT>
+int launch_decode(const bf16* q, int64_t ld_q, bf16* out, int64_t ld_out, float* part, const bf16* kc, const bf16* vc,
+                  const int32_t* bt, int64_t max_blocks, const int32_t* cu, const int32_t* sl, int num_reqs, int keys_per_split,
+                  int splits, float scale, int window, int H, int Hkv, int ps, hipStream_t stream) {
+  attn_decode_kernel<DT><<<dim3((unsigned)splits, (unsigned)Hkv, (unsigned)num_reqs), 64, 0, stream>>>(
+      q, ld_q, part, kc, vc, bt, max_blocks, cu, sl, keys_per_split, splits, scale * LOG2E, window, H, Hkv, ps);
+  const int D = DT * 16;
+  attn_decode_merge_kernel<<<dim3((unsigned)H, (unsigned)num_reqs), D <= 64 ? 64 : (D <= 128 ? 128 : 256), 0, stream>>>(
+      part, out, ld_out, cu, sl, keys_per_split, splits, window, H, D);
+  return launch_status();
+}
+
+#define DINFER_DISPATCH_HEAD_DIM(head_dim, CALL) \
+  switch (head_dim) {                            \
+    case 32: { constexpr int DT = 2; CALL; }     \
+    case 48: { constexpr int DT = 3; CALL; }     \
+    case 64: { constexpr int DT = 4; CALL; }     \
+    case 96: { constexpr int DT = 6; CALL; }     \
+    case 128: { constexpr int DT = 8; CALL; }    \
+    case 256: { constexpr int DT = 16; CALL; }   \
+    default: return ERR_UNSUPPORTED;             \
+  }
+
+}  // namespace
+
+// 1 if the MFMA kernels take this geometry, else 0 (the caller uses the plain kernel).
+extern "C" int dinfer_attn_mfma_supports(int head_dim, int page_size, int heads, int kv_heads) {
+  switch (head_dim) {
+    case 32: case 48: case 64: case 96: case 128: case 256: break;
+    default: return 0;
+  }
+  return page_size > 0 && page_size % 8 == 0 && kv_heads > 0 && heads % kv_heads == 0 ? 1 : 0;
+}
+
+extern "C" int dinfer_attn_flash(const void* q, int64_t ld_q, void* out, int64_t ld_out, const void* k_cache,
+                                 const void* v_cache, const int32_t* block_table, int64_t max_blocks,
+                                 const int32_t* cu_seqlens, const int32_t* seq_lens, int num_reqs, int max_q_len,
+                                 float scale, int window, int heads, int kv_heads, int head_dim, int page_size,
+                                 int skip_single, hipStream_t stream) {
+  if (num_reqs <= 0 || max_q_len <= 0) return OK;
+  if (!dinfer_attn_mfma_supports(head_dim, page_size, heads, kv_heads)) return ERR_UNSUPPORTED;
+  if (window < 0 || max_blocks <= 0 || ld_q % 8 || ld_out % 4 || !aligned16(q) || !aligned16(k_cache) ||
+      !aligned16(v_cache) || ((uintptr_t)out % 8))
+    return ERR_BAD_SHAPE;
+  DINFER_DISPATCH_HEAD_DIM(head_dim, return launch_flash<DT>(
+      (const bf16*)q, ld_q, (bf16*)out, ld_out, (const bf16*)k_cache, (const bf16*)v_cache, block_table, max_blocks,
+      cu_seqlens, seq_lens, num_reqs, max_q_len, scale, window, heads, kv_heads, page_size, skip_single, stream));
+}
+
+// Single-row requests only. cu_seqlens null: every request brings exactly one row (row b belongs to
+// request b). cu_seqlens given: requests with one row are served, the others are left alone.
+// part: float workspace of num_reqs * heads * splits * (head_dim + 4) elements, where
+// splits = ceil(max_len / keys_per_split) and max_len bounds every seq_len.
+extern "C" int dinfer_attn_decode(const void* q, int64_t ld_q, void* out, int64_t ld_out, float* part,
+                                  int64_t part_elems, const void* k_cache, const void* v_cache,
+                                  const int32_t* block_table, int64_t max_blocks, const int32_t* cu_seqlens,
+                                  const int32_t* seq_lens, int num_reqs, int max_len, int keys_per_split, float scale, int window, int heads,
+                                  int kv_heads, int head_dim, int page_size, hipStream_t stream) {
+  if (num_reqs <= 0) return OK;
+  if (!dinfer_attn_mfma_supports(head_dim, page_size, heads, kv_heads)) return ERR_UNSUPPORTED;
+  if (heads / kv_heads > 16) return ERR_UNSUPPORTED;
+  if (window < 0 || max_blocks <= 0 || max_len <= 0 || keys_per_split <= 0 || keys_per_split % 32 || ld_q % 8 ||
+      !aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(part) || num_reqs > 65535 ||
+      kv_heads > 65535)
+    return ERR_BAD_SHAPE;
+  const int splits = (max_len + keys_per_split - 1) / keys_per_split;
+  if ((int64_t)num_reqs * heads * splits * (head_dim + 4) > part_elems) return 5;
+  DINFER_DISPATCH_HEAD_DIM(head_dim, return launch_decode<DT>(
+      (const bf16*)q, ld_q, (bf16*)out, ld_out, part, (const bf16*)k_cache, (const bf16*)v_cache, block_table,
+      max_blocks, cu_seqlens, seq_lens, num_reqs, keys_per_split, splits, scale, window, heads, kv_heads, page_size, stream));
+}

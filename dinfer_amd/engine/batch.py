@@ -71,6 +71,7 @@ class StepBatch:
         self.starts: list[int] = []
         self.max_q_len = self.max_seq_len = 0
         self.all_decode = False
+        self.max_len_bound = 0
         self.req_ids: list = []
         self.row_owner: list[tuple] = []  # (request index, token index) per logits row
         self._copied = torch.cuda.Event() if pin else None
@@ -125,6 +126,8 @@ class StepBatch:
         self.max_q_len = max(self.q_lens)
         self.max_seq_len = max(s + n for s, n in zip(self.starts, self.q_lens))
         self.all_decode = all(n == 1 for n in self.q_lens)
+        # what kernels may assume about every seq_len of this step (a replayed graph fixes it to the model's limit)
+        self.max_len_bound = self.max_seq_len
 
     def upload(self) -> None:
         self._dev.copy_(self._host, non_blocking=True)

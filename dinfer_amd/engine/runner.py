@@ -46,7 +46,8 @@ class ModelRunner:
         self.max_rows = options.max_logits_rows or options.max_num_seqs
         # decode rows may ride on top of the prompt budget (service.rs:206-210)
         self.max_tokens = options.max_num_batched_tokens + (options.max_num_seqs if options.decode_exempt_from_budget else 0)
-        self.ctx = BuildContext(device, self.dtype, self.max_tokens, self.max_rows, self.page_size)
+        self.ctx = BuildContext(device, self.dtype, self.max_tokens, self.max_rows, self.page_size,
+                                options.max_num_seqs)
         model.bind(self.ctx)
         self._build_caches()
         self.batch = StepBatch(device, self.max_tokens, options.max_num_seqs, self.max_rows,

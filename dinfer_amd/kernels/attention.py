@@ -1,7 +1,9 @@
-"""Chooses the attention kernel for a step.
+"""Chooses the attention kernels for a step.
 
 float32 storage: always the plain kernel (fixed key order, any sizes).
-bfloat16 storage: MFMA kernels where the sizes fit them, the plain kernel otherwise.
+bfloat16 storage: MFMA kernels where the geometry fits them (head size from the
+instantiated list, page size a multiple of 8): split-K decode for the requests that
+bring one row, flash for the others; the plain kernel otherwise.
 """
 from __future__ import annotations
 
@@ -9,17 +11,47 @@ import torch
 
 from . import ops
 
+TARGET_WAVES = 4096   # split-K aims at about this many waves in flight
+MIN_KEYS_PER_SPLIT = 64
+
 
 class Workspace:
-    """Scratch of the split-K decode kernel, sized once for the largest step."""
+    """Geometry checks and the split-K scratch of one attention shape, sized once."""
 
     def __init__(self, ctx, heads: int, kv_heads: int, head_dim: int):
-        self.ctx = ctx
+        self.max_reqs = ctx.max_reqs
+        self.mfma = (ctx.dtype == torch.bfloat16 and ops.attn_mfma_supports(head_dim, ctx.page_size, heads, kv_heads))
+        self.split_k = self.mfma and heads // kv_heads <= 16
+        self.part = None
+        if self.split_k:
+            max_units = TARGET_WAVES + ctx.max_reqs * kv_heads  # (request, kv head, split) triples at most
+            elems = max_units * (heads // kv_heads) * (head_dim + 4)
+            self.part = ctx.workspace.buffer("attn_partials", elems, dtype=torch.float32, rows=1)
+        self.kv_heads = kv_heads
+
+    def keys_per_split(self, num_reqs: int, max_len: int) -> int:
+        splits = max(1, TARGET_WAVES // (num_reqs * self.kv_heads))
+        kps = -(-max_len // splits)
+        return max(MIN_KEYS_PER_SPLIT, (kps + 31) // 32 * 32)
 
 
 def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k_cache, v_cache, batch, group: int, ws: Workspace, *,
                     scale: float, window: int, heads: int, kv_heads: int, head_dim: int, page_size: int):
     """q is read from the first heads*head_dim columns of qkv; out [T, heads*head_dim]."""
-    return ops.attn_paged_ref(qkv, out, k_cache, v_cache, batch.block_table[group], batch.cu_seqlens,
-                              batch.seq_lens, batch.num_reqs, batch.num_tokens, scale=scale, window=window,
-                              heads=heads, kv_heads=kv_heads, head_dim=head_dim, page_size=page_size)
+    geo = dict(scale=scale, window=window, heads=heads, kv_heads=kv_heads, head_dim=head_dim, page_size=page_size)
+    bt = batch.block_table[group]
+    B, T = batch.num_reqs, batch.num_tokens
+    if not ws.mfma:
+        return ops.attn_paged_ref(qkv, out, k_cache, v_cache, bt, batch.cu_seqlens, batch.seq_lens, B, T, **geo)
+    singles = sum(1 for n in batch.q_lens if n == 1) if ws.split_k else 0
+    # a few single rows beside long portions are not worth two more launches
+    use_decode = singles == B or singles >= 4
+    if use_decode:
+        max_len = batch.max_len_bound
+        kps = ws.keys_per_split(B, max_len)
+        ops.attn_decode(qkv, out, ws.part, k_cache, v_cache, bt, None if singles == B else batch.cu_seqlens,
+                        batch.seq_lens, B, max_len, kps, **geo)
+        if singles == B:
+            return out
+    return ops.attn_flash(qkv, out, k_cache, v_cache, bt, batch.cu_seqlens, batch.seq_lens, B, T, batch.max_q_len,
+                          skip_single=use_decode, **geo)

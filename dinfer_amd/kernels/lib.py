@@ -33,6 +33,15 @@ SIGNATURES = {
         "attention_ref",
         [_I, _P, _L, _P, _L, _P, _P, _P, _L, _P, _P, _I, _L, _F, _I, _I, _I, _I, _I, _P],
     ),
+    "dinfer_attn_mfma_supports": ("attention", [_I, _I, _I, _I]),
+    "dinfer_attn_flash": (
+        "attention",
+        [_P, _L, _P, _L, _P, _P, _P, _L, _P, _P, _I, _I, _F, _I, _I, _I, _I, _I, _I, _P],
+    ),
+    "dinfer_attn_decode": (
+        "attention",
+        [_P, _L, _P, _L, _P, _L, _P, _P, _P, _L, _P, _P, _I, _I, _I, _F, _I, _I, _I, _I, _I, _P],
+    ),
     "dinfer_gemm_ref": ("gemm_ref", [_I, _I, _P, _L, _P, _L, _P, _L, _L, _L, _L, _P]),
     "dinfer_argmax": ("sampling", [_P, _L, _P, _L, _L, _P]),
     "dinfer_sample": ("sampling", [_P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _P]),

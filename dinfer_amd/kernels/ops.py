@@ -182,6 +182,50 @@ def attn_paged_ref(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_
     return out
 
 
+def attn_mfma_supports(head_dim: int, page_size: int, heads: int, kv_heads: int) -> bool:
+    return bool(lib.get("dinfer_attn_mfma_supports")(head_dim, page_size, heads, kv_heads))
+
+
+def _check_paged(q, out, k_cache, v_cache, block_table, seq_lens, num_reqs, heads, kv_heads, head_dim, page_size):
+    assert q.dtype == out.dtype == k_cache.dtype == v_cache.dtype == torch.bfloat16
+    assert block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous()
+    assert block_table.shape[0] >= num_reqs and seq_lens.dtype == torch.int32 and seq_lens.numel() >= num_reqs
+    nb = k_cache.shape[0]
+    assert tuple(k_cache.shape) == (nb, kv_heads, page_size, head_dim) and k_cache.is_contiguous()
+    assert tuple(v_cache.shape) == (nb, kv_heads, head_dim, page_size) and v_cache.is_contiguous()
+    assert q.shape[1] >= heads * head_dim and out.shape[1] >= heads * head_dim
+
+
+def attn_flash(q, out, k_cache, v_cache, block_table, cu_seqlens, seq_lens, num_reqs: int, tokens: int,
+               max_q_len: int, *, scale: float, window: int, heads: int, kv_heads: int, head_dim: int,
+               page_size: int, skip_single: bool = False):
+    """MFMA flash attention over the pages: rows with or without history, causal, optional window."""
+    _need_gpu(q, out, k_cache, v_cache, block_table, cu_seqlens, seq_lens)
+    _check_paged(q, out, k_cache, v_cache, block_table, seq_lens, num_reqs, heads, kv_heads, head_dim, page_size)
+    assert cu_seqlens.dtype == torch.int32 and cu_seqlens.numel() >= num_reqs + 1
+    assert q.shape[0] >= tokens and out.shape[0] >= tokens
+    lib.call("dinfer_attn_flash", q.data_ptr(), _rows(q), out.data_ptr(), _rows(out), k_cache.data_ptr(),
+             v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1], cu_seqlens.data_ptr(),
+             seq_lens.data_ptr(), num_reqs, max_q_len, float(scale), int(window), heads, kv_heads, head_dim,
+             page_size, 1 if skip_single else 0, _stream())
+    return out
+
+
+def attn_decode(q, out, part, k_cache, v_cache, block_table, cu_seqlens, seq_lens, num_reqs: int, max_len: int,
+                keys_per_split: int, *, scale: float, window: int, heads: int, kv_heads: int, head_dim: int,
+                page_size: int):
+    """Split-K attention for requests that bring one row. cu_seqlens None: row b is request b;
+    given: only the requests with one row are served (mixed batches)."""
+    _need_gpu(q, out, part, k_cache, v_cache, block_table, cu_seqlens, seq_lens)
+    _check_paged(q, out, k_cache, v_cache, block_table, seq_lens, num_reqs, heads, kv_heads, head_dim, page_size)
+    assert part.dtype == torch.float32 and part.is_contiguous()
+    lib.call("dinfer_attn_decode", q.data_ptr(), _rows(q), out.data_ptr(), _rows(out), part.data_ptr(),
+             part.numel(), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1],
+             _ptr(cu_seqlens), seq_lens.data_ptr(), num_reqs, max_len, keys_per_split, float(scale), int(window),
+             heads, kv_heads, head_dim, page_size, _stream())
+    return out
+
+
 def gemm_ref(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int) -> torch.Tensor:
     """out[:m] = a[:m] @ w.T on the vector ALUs with float accumulation (true 32-bit for float operands)."""
     _need_gpu(a, w, out)

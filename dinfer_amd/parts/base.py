@@ -43,9 +43,10 @@ class Workspace:
 class BuildContext:
     """What a part may know about the engine it is built into."""
 
-    def __init__(self, device, dtype: torch.dtype, max_tokens: int, max_rows: int, page_size: int):
+    def __init__(self, device, dtype: torch.dtype, max_tokens: int, max_rows: int, page_size: int,
+                 max_reqs: int = 1):
         self.device, self.dtype = device, dtype
-        self.max_tokens, self.max_rows, self.page_size = max_tokens, max_rows, page_size
+        self.max_tokens, self.max_rows, self.page_size, self.max_reqs = max_tokens, max_rows, page_size, max_reqs
         self.workspace = Workspace(device, dtype, max_tokens)
 
 

@@ -1,0 +1,396 @@
+"""Each HIP kernel alone against a plain float64 torch reference of the same operation, at
+sizes other than the engine tests use (widths and vocabularies that are no power of two,
+head sizes 32..256, group sizes 1..8, page sizes 8..64, shuffled page order)."""
+import math
+import random
+
+import pytest
+import torch
+
+import plain_qwen3 as plain
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def ops():
+    from dinfer_amd.kernels import ops as o
+    return o
+
+
+def tol(dtype):
+    # bf16: one rounding of the result (2^-8 relative) plus input rounding noise
+    return dict(rtol=2e-2, atol=2e-2) if dtype == torch.bfloat16 else dict(rtol=1e-5, atol=1e-5)
+
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embedding(dtype):
+    V, W = 1000, 200  # rows of 400 / 800 bytes: vector path for both dtypes; plus an odd width below
+    for width in (W, 201):
+        table = torch.randn(V, width, device=DEV).to(dtype)
+        ids = torch.randint(0, V, (17,), device=DEV, dtype=torch.int32)
+        out = torch.empty(17, width, device=DEV, dtype=dtype)
+        ops().embedding(ids, table, out)
+        assert torch.equal(out, table[ids.long()])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("width", [1536, 100, 4096, 5120, 20000])
+def test_rmsnorm(dtype, width):
+    T, eps = 13, 1e-5
+    x = (torch.randn(T, width, device=DEV) * 2).to(dtype)
+    res = torch.randn(T, width, device=DEV).to(dtype)
+    w = (torch.rand(width, device=DEV) + 0.5).to(dtype)
+    out = torch.empty(T, width, device=DEV, dtype=dtype)
+    ops().rmsnorm(x, w, out, eps, T)
+    want = plain.rms_norm(x.double(), w.double(), eps)
+    torch.testing.assert_close(out.double(), want, **tol(dtype))
+    # fused add: the residual is rounded first, and the rounded sum is normed
+    res2 = res.clone()
+    ops().rmsnorm(x, w, out, eps, T, residual=res2)
+    summed = (x.float() + res.float()).to(dtype)
+    assert torch.equal(res2, summed)
+    torch.testing.assert_close(out.double(), plain.rms_norm(summed.double(), w.double(), eps), **tol(dtype))
+    # gather, with a gain stored in 32-bit and an offset of 1
+    rows = torch.tensor([12, 0, 5], device=DEV, dtype=torch.int32)
+    out3 = torch.empty(3, width, device=DEV, dtype=dtype)
+    ops().rmsnorm(x, w.float(), out3, eps, 3, rows=rows, weight_offset=1.0)
+    torch.testing.assert_close(out3.double(), plain.rms_norm(x[rows.long()].double(), w.double() + 1.0, eps), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gated_act(dtype):
+    for T, I in ((11, 2048), (3, 136), (5, 12288)):
+        x = torch.randn(T, 2 * I, device=DEV).to(dtype)
+        out = torch.empty(T, I, device=DEV, dtype=dtype)
+        ops().gated_act(x, out, T)
+        want = plain.silu(x[:, :I].double()) * x[:, I:].double()
+        torch.testing.assert_close(out.double(), want, **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gemm_ref(dtype):
+    for M, N, K in ((33, 96, 512), (1, 331, 80), (70, 100, 37)):
+        a = torch.randn(M, K, device=DEV).to(dtype)
+        w = (torch.randn(N, K, device=DEV) * 0.05).to(dtype)
+        out = torch.empty(M, N, device=DEV, dtype=dtype)
+        ops().gemm_ref(a, w, out, M)
+        want = a.double() @ w.double().T
+        torch.testing.assert_close(out.double(), want, **tol(dtype))
+        out32 = torch.empty(M, N, device=DEV, dtype=torch.float32)
+        ops().gemm_ref(a, w, out32, M)
+        torch.testing.assert_close(out32.double(), want, rtol=1e-5, atol=1e-5)
+
+
+# ---- qkv_post: per-head norm, rotation, cache write -----------------------------------------------
+def rope_table(max_pos, rd, theta):
+    ang = plain.rope_angles(list(range(max_pos)), rd, theta)
+    return torch.cat([ang.cos(), ang.sin()], dim=1).float()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,Hkv,D,page", [(16, 8, 128, 16), (6, 2, 48, 4), (5, 5, 80, 8), (4, 1, 256, 32)])
+def test_qkv_post(dtype, H, Hkv, D, page):
+    T, theta, eps, nblocks = 6, 1e6, 1e-6, 4
+    width = (H + 2 * Hkv) * D
+    qkv_in = torch.randn(T, width, device=DEV).to(dtype)
+    wq = (torch.rand(D, device=DEV) + 0.5).to(dtype)
+    wk = (torch.rand(D, device=DEV) + 0.5).to(dtype)
+    pos = torch.tensor([0, 3, 7, 15, 31, 100], device=DEV, dtype=torch.int32)
+    slots = torch.tensor([0, 1, 2, page + 1, page + 2, -1], device=DEV, dtype=torch.int64)  # the last token is not cached
+    table = rope_table(128, D, theta).to(DEV)
+    kc = torch.zeros(nblocks, Hkv, page, D, device=DEV, dtype=dtype)
+    vc = torch.zeros(nblocks, Hkv, D, page, device=DEV, dtype=dtype)
+    qkv = qkv_in.clone()
+    ops().qkv_post(qkv, T, heads=H, kv_heads=Hkv, head_dim=D, q_off=0, k_off=H * D, v_off=(H + Hkv) * D, q_gain=wq,
+                   k_gain=wk, eps=eps, gain_offset=0.0, positions=pos, cos_sin=table, rotary_dim=D, rope_style=0,
+                   k_cache=kc, v_cache=vc, slot_mapping=slots, page_size=page)
+    x = qkv_in.double().cpu()
+    ang = plain.rope_angles(pos.tolist(), D, theta)
+    q = plain.rope_neox(plain.rms_norm(x[:, :H * D].view(T, H, D), wq.double().cpu(), eps), ang)
+    k = plain.rope_neox(plain.rms_norm(x[:, H * D:(H + Hkv) * D].view(T, Hkv, D), wk.double().cpu(), eps), ang)
+    v = x[:, (H + Hkv) * D:].view(T, Hkv, D)
+    torch.testing.assert_close(qkv[:, :H * D].double().cpu().view(T, H, D), q, **tol(dtype))
+    want_k = torch.zeros(nblocks, Hkv, page, D, dtype=torch.float64)
+    want_v = torch.zeros(nblocks, Hkv, D, page, dtype=torch.float64)
+    for t, s in enumerate(slots.tolist()):
+        if s >= 0:
+            want_k[s // page, :, s % page, :] = k[t]
+            want_v[s // page, :, :, s % page] = v[t]
+    torch.testing.assert_close(kc.double().cpu(), want_k, **tol(dtype))
+    assert torch.equal(vc.double().cpu(), want_v)  # v is copied, not computed
+
+
+def test_qkv_post_partial_and_interleaved_rotation():
+    """rotary_dim smaller than the head, interleaved pairs, no norm: parameters, not constants."""
+    T, H, Hkv, D, RD, theta = 4, 2, 1, 64, 32, 1e4
+    qkv_in = torch.randn(T, (H + 2 * Hkv) * D, device=DEV)
+    pos = torch.tensor([5, 0, 9, 77], device=DEV, dtype=torch.int32)
+    table = rope_table(128, RD, theta).to(DEV)
+    for style in (0, 1):
+        qkv = qkv_in.clone()
+        ops().qkv_post(qkv, T, heads=H, kv_heads=Hkv, head_dim=D, q_off=0, k_off=H * D, v_off=(H + Hkv) * D,
+                       q_gain=None, k_gain=None, eps=0.0, gain_offset=0.0, positions=pos, cos_sin=table, rotary_dim=RD,
+                       rope_style=style, k_cache=None, v_cache=None, slot_mapping=None, page_size=8)
+        x = qkv_in[:, :H * D].double().cpu().view(T, H, D)
+        ang = plain.rope_angles(pos.tolist(), RD, theta)
+        want = x.clone()
+        if style == 0:
+            want[..., :RD] = plain.rope_neox(x[..., :RD], ang)
+        else:
+            a, b = x[..., 0:RD:2], x[..., 1:RD:2]
+            c, s = ang.cos()[:, None, :], ang.sin()[:, None, :]
+            want[..., 0:RD:2], want[..., 1:RD:2] = a * c - b * s, b * c + a * s
+        torch.testing.assert_close(qkv[:, :H * D].double().cpu().view(T, H, D), want, rtol=1e-5, atol=1e-5)
+
+
+# ---- attention ------------------------------------------------------------------------------------
+def paged_case(dtype, H, Hkv, D, page, hist, new, seed=0, spike=None):
+    """Requests with `hist` cached tokens and `new` rows each; pages in shuffled order.
+    Returns q [T, H*D], caches, metadata tensors and the expected output [T, H, D] in float64."""
+    g = torch.Generator().manual_seed(seed)
+    B = len(hist)
+    total = [h + n for h, n in zip(hist, new)]
+    max_blocks = max(-(-t // page) for t in total) + 1
+    nblocks = sum(-(-t // page) for t in total) + 3
+    order = list(range(nblocks))
+    random.Random(seed).shuffle(order)
+    kc = torch.randn(nblocks, Hkv, page, D, generator=g).to(dtype)  # stale content everywhere
+    vc = torch.randn(nblocks, Hkv, D, page, generator=g).to(dtype)
+    bt = torch.full((B, max_blocks), -1, dtype=torch.int32)
+    qs, outs = [], []
+    for b in range(B):
+        k = torch.randn(total[b], Hkv, D, generator=g).to(dtype)
+        v = torch.randn(total[b], Hkv, D, generator=g).to(dtype)
+        q = torch.randn(new[b], H, D, generator=g).to(dtype)
+        if spike is not None and total[b] > spike[0] and new[b] > 0:
+            # one far key that must win: scale a query and that key so that one score stands out
+            key, amp = spike
+            k[key] = k[key] * 0 + q[-1, ::H // Hkv][:, :].float().to(dtype) * amp
+        for i in range(-(-total[b] // page)):
+            blk = order.pop()
+            bt[b, i] = blk
+            n = min(page, total[b] - i * page)
+            kc[blk, :, :n] = k[i * page:i * page + n].transpose(0, 1)
+            vc[blk, :, :, :n] = v[i * page:i * page + n].permute(1, 2, 0)
+        qs.append(q)
+        outs.append((q.double(), k.double(), v.double()))
+    cu = torch.tensor([0] + list(torch.tensor(new).cumsum(0)), dtype=torch.int32)
+    meta = dict(bt=bt.to(DEV), cu=cu.to(DEV), sl=torch.tensor(total, dtype=torch.int32, device=DEV))
+    q_all = torch.cat(qs).reshape(sum(new), H * D).to(DEV)
+    return q_all, kc.to(DEV), vc.to(DEV), meta, outs
+
+
+def expected_attention(outs, hist, scale, window):
+    res = []
+    for (q, k, v), h in zip(outs, hist):
+        Tq, H, D = q.shape
+        G = H // k.shape[1]
+        o = torch.zeros_like(q)
+        pos = h + torch.arange(Tq)[:, None]
+        j = torch.arange(k.shape[0])[None, :]
+        hidden = j > pos
+        if window:
+            hidden = hidden | (j <= pos - window)
+        for hh in range(H):
+            s = (q[:, hh] @ k[:, hh // G].T) * scale
+            s = s.masked_fill(hidden, float("-inf"))
+            o[:, hh] = torch.softmax(s, -1) @ v[:, hh // G]
+        res.append(o)
+    return torch.cat(res)
+
+
+GEOS = [(4, 2, 32, 8), (16, 8, 128, 16), (6, 2, 48, 8), (5, 1, 64, 64), (8, 8, 96, 24), (16, 2, 256, 16)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [0, 40])
+def test_attention_plain_kernel(dtype, window):
+    H, Hkv, D, page = 6, 2, 40, 4  # a head size the MFMA kernels do not take
+    hist, new = [11, 0, 70, 6], [3, 17, 1, 1]
+    q, kc, vc, m, outs = paged_case(dtype, H, Hkv, D, page, hist, new)
+    out = torch.empty(sum(new), H * D, device=DEV, dtype=dtype)
+    ops().attn_paged_ref(q, out, kc, vc, m["bt"], m["cu"], m["sl"], len(hist), sum(new), scale=D ** -0.5,
+                         window=window, heads=H, kv_heads=Hkv, head_dim=D, page_size=page)
+    want = expected_attention(outs, hist, D ** -0.5, window)
+    torch.testing.assert_close(out.double().cpu().view(-1, H, D), want, **tol(dtype))
+
+
+@pytest.mark.parametrize("window", [0, 50])
+@pytest.mark.parametrize("H,Hkv,D,page", GEOS)
+def test_attention_flash(H, Hkv, D, page, window):
+    # prompts without history (70 / 33 / 5: several tiles, ragged tail, idle waves), portions with
+    # history that ends inside a page, single rows, and a long run that needs the two-tile kernel
+    hist, new = [0, 0, 0, 40, 70, 300, 129, 7], [70, 33, 5, 5, 1, 1, 150, 64]
+    q, kc, vc, m, outs = paged_case(torch.bfloat16, H, Hkv, D, page, hist, new, seed=3)
+    out = torch.zeros(sum(new), H * D, device=DEV, dtype=torch.bfloat16)
+    ops().attn_flash(q, out, kc, vc, m["bt"], m["cu"], m["sl"], len(hist), sum(new), max(new), scale=D ** -0.5,
+                     window=window, heads=H, kv_heads=Hkv, head_dim=D, page_size=page)
+    want = expected_attention(outs, hist, D ** -0.5, window)
+    torch.testing.assert_close(out.double().cpu().view(-1, H, D), want, rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("window", [0, 100])
+@pytest.mark.parametrize("H,Hkv,D,page", GEOS)
+def test_attention_decode_split_k(H, Hkv, D, page, window):
+    # 300 / 70 / 1: several splits, a short one, a single key; then 1..64 at batch 32
+    for hist, kps in (([299, 69, 0, 1000], 64), ([random.Random(7).randrange(64) for _ in range(32)], 256)):
+        new = [1] * len(hist)
+        q, kc, vc, m, outs = paged_case(torch.bfloat16, H, Hkv, D, page, hist, new, seed=5)
+        out = torch.zeros(len(hist), H * D, device=DEV, dtype=torch.bfloat16)
+        max_len = max(hist) + 1
+        splits = -(-max_len // kps)
+        part = torch.full((len(hist) * H * splits * (D + 4),), float("nan"), device=DEV)
+        ops().attn_decode(q, out, part, kc, vc, m["bt"], None, m["sl"], len(hist), max_len, kps, scale=D ** -0.5,
+                          window=window, heads=H, kv_heads=Hkv, head_dim=D, page_size=page)
+        want = expected_attention(outs, hist, D ** -0.5, window)
+        torch.testing.assert_close(out.double().cpu().view(-1, H, D), want, rtol=2e-2, atol=2e-2)
+
+
+def test_attention_mixed_routes_single_rows_to_split_k():
+    H, Hkv, D, page = 16, 4, 128, 16
+    hist, new = [500, 0, 64, 900, 33, 10], [1, 40, 1, 1, 20, 1]
+    q, kc, vc, m, outs = paged_case(torch.bfloat16, H, Hkv, D, page, hist, new, seed=9)
+    out = torch.zeros(sum(new), H * D, device=DEV, dtype=torch.bfloat16)
+    max_len, kps = max(h + n for h, n in zip(hist, new)), 128
+    part = torch.zeros(len(hist) * H * (-(-max_len // kps)) * (D + 4), device=DEV)
+    geo = dict(scale=D ** -0.5, window=0, heads=H, kv_heads=Hkv, head_dim=D, page_size=page)
+    ops().attn_decode(q, out, part, kc, vc, m["bt"], m["cu"], m["sl"], len(hist), max_len, kps, **geo)
+    ops().attn_flash(q, out, kc, vc, m["bt"], m["cu"], m["sl"], len(hist), sum(new), max(new), skip_single=True, **geo)
+    want = expected_attention(outs, hist, D ** -0.5, 0)
+    torch.testing.assert_close(out.double().cpu().view(-1, H, D), want, rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("kernel", ["plain", "flash", "decode"])
+def test_attention_finds_one_far_key(kernel):
+    """Random scores hide a key that is skipped or read from the wrong slot. Here key 5 of 700 is
+    made to dominate the last row's softmax, so the output must be (nearly) that key's value."""
+    H, Hkv, D, page = 8, 2, 64, 16
+    hist, new = [699], [1]
+    q, kc, vc, m, outs = paged_case(torch.bfloat16, H, Hkv, D, page, hist, new, seed=11, spike=(5, 3.0))
+    out = torch.zeros(1, H * D, device=DEV, dtype=torch.bfloat16)
+    geo = dict(scale=D ** -0.5, window=0, heads=H, kv_heads=Hkv, head_dim=D, page_size=page)
+    if kernel == "plain":
+        ops().attn_paged_ref(q, out, kc, vc, m["bt"], m["cu"], m["sl"], 1, 1, **geo)
+    elif kernel == "flash":
+        ops().attn_flash(q, out, kc, vc, m["bt"], m["cu"], m["sl"], 1, 1, 1, **geo)
+    else:
+        part = torch.zeros(H * 11 * (D + 4), device=DEV)
+        ops().attn_decode(q, out, part, kc, vc, m["bt"], None, m["sl"], 1, 700, 64, **geo)
+    want = expected_attention(outs, hist, D ** -0.5, 0)
+    torch.testing.assert_close(out.double().cpu().view(-1, H, D), want, rtol=2e-2, atol=2e-2)
+    # the spiked heads (one per kv head) really are dominated by key 5
+    (qq, kk, vv) = outs[0]
+    got = out.double().cpu().view(H, D)
+    for hk in range(Hkv):
+        assert (got[hk * (H // Hkv)] - vv[5, hk]).abs().max() < 0.1
+
+
+# ---- sampling -------------------------------------------------------------------------------------
+def test_argmax_ties_to_lowest_index():
+    V = 163841
+    logits = torch.randn(6, V, device=DEV) * 3
+    logits[2, 100] = logits[2, 90000] = 50.0
+    logits[3, :] = 1.0
+    out = torch.empty(6, device=DEV, dtype=torch.int32)
+    ops().argmax(logits, out, 6)
+    want = logits.argmax(-1).tolist()
+    want[2], want[3] = 100, 0
+    assert out.tolist() == want
+
+
+def draw(logits, temperature, seeds, offsets, **kw):
+    R, V = logits.shape
+    out = torch.empty(R, device=DEV, dtype=torch.int32)
+    work = torch.empty(R, V, device=DEV)
+    f = lambda xs, dt: torch.tensor(xs, device=DEV, dtype=dt)
+    ops().sample(logits, work, out, R, temperature=f(temperature, torch.float32), seeds=f(seeds, torch.int64),
+                 offsets=f(offsets, torch.int64),
+                 **{k: f(v, torch.int32 if k == "top_k" else torch.float32) for k, v in kw.items()})
+    return out.tolist()
+
+
+def test_sample_follows_the_inverse_cdf_rule():
+    """Each draw must be the token whose interval of the running sum holds u * total, with u from the
+    plain Philox. Draws whose target lies within rounding of an interval's edge are not judged."""
+    V = 331
+    logits = torch.randn(64, V, device=DEV) * 2
+    temps = [0.7] * 64
+    seeds = [12345 + i for i in range(64)]
+    offsets = [i * 3 for i in range(64)]
+    got = draw(logits, temps, seeds, offsets)
+    judged = 0
+    for r in range(64):
+        tok, slack = plain.sample_row(logits[r].cpu(), temps[r], seeds[r], offsets[r])
+        if slack > 1e-5:
+            judged += 1
+            assert got[r] == tok, f"row {r}: kernel chose {got[r]}, the rule says {tok}"
+    assert judged > 55
+
+
+def test_sample_does_not_depend_on_batch_position():
+    V = 1000
+    row = torch.randn(1, V, device=DEV)
+    other = torch.randn(5, V, device=DEV)
+    alone = draw(row, [0.9], [777], [4])[0]
+    batch = torch.cat([other[:3], row, other[3:]])
+    mixed = draw(batch, [1.0, 0.0, 0.5, 0.9, 1.3, 0.0], [1, 2, 3, 777, 5, 6], [0, 0, 0, 4, 0, 0])
+    assert mixed[3] == alone
+    assert mixed[1] == int(batch[1].argmax()) and mixed[5] == int(batch[5].argmax())  # greedy rows untouched
+
+
+def test_sample_frequencies_match_softmax():
+    """100k draws of one 64-token row at temperature 0.8: L1 distance to softmax below 0.03
+    (the reference's statistical test, crates/kernels/tests/ref_tests.rs:225-252)."""
+    V, N = 64, 100_000
+    row = torch.randn(V, device=DEV) * 2
+    counts = torch.zeros(V)
+    for chunk in range(N // 1000):
+        toks = draw(row.expand(1000, V).contiguous(), [0.8] * 1000, [42] * 1000, list(range(chunk * 1000, chunk * 1000 + 1000)))
+        counts += torch.bincount(torch.tensor(toks), minlength=V).float()
+    want = torch.softmax(row.cpu() / 0.8, -1)
+    assert (counts / N - want).abs().sum() < 0.03
+
+
+def test_sample_candidate_sets():
+    """min_p, top-k and top-p: every draw falls in the set the plain rule keeps."""
+    V = 512
+    logits = torch.randn(6, V, device=DEV) * 3
+    cases = [dict(top_k=1, top_p=1.0, min_p=0.0), dict(top_k=50, top_p=1.0, min_p=0.0),
+             dict(top_k=-1, top_p=0.9, min_p=0.0), dict(top_k=5, top_p=0.5, min_p=0.0),
+             dict(top_k=-1, top_p=1.0, min_p=0.2), dict(top_k=40, top_p=0.8, min_p=0.05)]
+    for r, c in enumerate(cases):
+        keep = plain.candidate_mask(logits[r].cpu().double() / 0.9, **c)
+        seen = set()
+        for off in range(0, 200, 50):
+            toks = draw(logits[r].expand(50, V).contiguous(), [0.9] * 50, [9] * 50, list(range(off, off + 50)),
+                        top_k=[c["top_k"]] * 50, top_p=[c["top_p"]] * 50, min_p=[c["min_p"]] * 50)
+            seen |= set(toks)
+        outside = [t for t in seen if not keep[t]]
+        # a token on the very edge of top-p may fall either way in 32-bit; allow the reference's margin
+        assert len(outside) <= max(2, int(0.001 * keep.sum())), f"case {c}: drew {outside} outside the kept set"
+        if c["top_k"] == 1:
+            assert seen == {int(logits[r].argmax())}
+
+
+def test_penalties_match_plain_rule():
+    V = 512
+    logits = torch.randn(4, V, device=DEV) * 3
+    hist = [([1, 5, 9, 5], [9, 9, 20]), ([3], []), ([7, 7, 7], [7, 100]), ([], [2, 4, 6, 4])]
+    rep, freq, pres = [1.5, 1.0, 1.2, 1.0], [0.0, 0.0, 0.3, 0.5], [0.0, 0.0, 0.2, 0.1]
+    ids, cnt, offs = [], [], [0]
+    for p, o in hist:
+        for t in sorted(set(p) | set(o)):
+            ids.append(t)
+            cnt.append(o.count(t))
+        offs.append(len(ids))
+    got = logits.clone()
+    i32 = lambda xs: torch.tensor(xs, device=DEV, dtype=torch.int32)
+    f32 = lambda xs: torch.tensor(xs, device=DEV, dtype=torch.float32)
+    ops().penalties(got, 4, i32(ids), i32(cnt), i32(offs), f32(rep), f32(freq), f32(pres))
+    for r, (p, o) in enumerate(hist):
+        want = plain.apply_penalties(logits[r].cpu().double(), p, o, rep[r], freq[r], pres[r])
+        torch.testing.assert_close(got[r].cpu().double(), want, rtol=1e-6, atol=1e-6)

@@ -29,4 +29,4 @@ CONFIGS = {
 }
 
 # page size used with each configuration in the engine tests
-PAGE = {"A": 16, "B": 8, "C": 4}
+PAGE = {"A": 4, "B": 8, "C": 16}
