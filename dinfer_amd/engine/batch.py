@@ -76,8 +76,13 @@ class StepBatch:
         self.row_owner: list[tuple] = []  # (request index, token index) per logits row
         self._copied = torch.cuda.Event() if pin else None
 
-    def fill(self, entries: list[Entry], cache) -> None:
-        """Writes the step into the pinned buffer from the entries and the cache manager's tables."""
+    def fill(self, entries: list[Entry], cache, pad_to: int | None = None) -> None:
+        """Writes the step into the pinned buffer from the entries and the cache manager's tables.
+
+        pad_to: for a step of single rows that replays a captured graph of that many requests, the
+        batch is filled up with requests of one token at position 0 that write no cache slot
+        (slot -1) and read page 0, which always exists (crates/layers/src/exec.rs:388-426).
+        Their logits rows are computed and ignored."""
         B = len(entries)
         T = sum(len(e.tokens) for e in entries)
         R = sum(len(e.want) for e in entries)
@@ -122,6 +127,22 @@ class StepBatch:
             self.starts.append(e.start)
             self.req_ids.append(e.req_id)
             t += n
+        if pad_to is not None and pad_to > B:
+            if T != B or R != B or pad_to > self.max_reqs or pad_to > self.max_tokens or pad_to > self.max_rows:
+                raise ValueError("only a step of single rows that all want logits can be padded")
+            P = pad_to
+            h["input_ids"][B:P] = 0
+            h["positions"][B:P] = 0
+            h["cu_seqlens"][B + 1:P + 1] = np.arange(B + 1, P + 1, dtype=np.int32)
+            h["seq_lens"][B:P] = 1
+            h["state_slots"][B:P] = 0
+            h["logits_rows"][B:P] = np.arange(B, P, dtype=np.int32)
+            for g in range(len(self.max_blocks)):
+                h["block_table%d" % g][B:P].fill(0)
+                h["slot_mapping%d" % g][B:P] = -1
+            self.q_lens += [1] * (P - B)
+            self.starts += [0] * (P - B)
+            T = B = R = P
         self.num_tokens, self.num_reqs, self.num_rows = T, B, R
         self.max_q_len = max(self.q_lens)
         self.max_seq_len = max(s + n for s, n in zip(self.starts, self.q_lens))

@@ -52,6 +52,11 @@ class ModelRunner:
         self._build_caches()
         self.batch = StepBatch(device, self.max_tokens, options.max_num_seqs, self.max_rows,
                                [self.max_blocks_per_seq] * len(self.group_specs))
+        # batch-size buckets of the decode graphs: powers of two and the largest batch
+        top = min(options.max_num_seqs, self.max_rows, self.max_tokens)
+        self._buckets = sorted({min(1 << i, top) for i in range(top.bit_length() + 1)})
+        self._graphs: dict[int, torch.cuda.CUDAGraph] = {}
+        self._graph_pool = None
 
     # ---- construction --------------------------------------------------------------------------
     @classmethod
@@ -152,6 +157,10 @@ class ModelRunner:
         Returns float32 logits [sum(len(e.want)), vocab] in the order of entries and of want
         (a view of a buffer that the next step overwrites)."""
         b = self.batch
+        n = len(entries)
+        if (self.options.hip_graph and not self.state_tensors and n <= self._buckets[-1]
+                and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)):
+            return self._graph_step(entries)
         b.fill(entries, self.cache)
         b.upload()
         fresh = self.cache.take_fresh_slots()
@@ -160,6 +169,31 @@ class ModelRunner:
             for st in self.state_tensors:
                 st.index_fill_(0, idx, 0)
         return self.model.forward(b, self.cache_views)
+
+    def _graph_step(self, entries: list[Entry]) -> torch.Tensor:
+        """A step of single rows replays a HIP graph captured for its batch-size bucket
+        (crates/layers/src/exec.rs:83-222, models/qwen3/src/executor.rs:995-1014). All step
+        inputs live at fixed addresses; what varies between replays is their content."""
+        b, n = self.batch, len(entries)
+        bucket = next(x for x in self._buckets if x >= n)
+        b.fill(entries, self.cache, pad_to=bucket)
+        b.max_len_bound = self.options.max_model_len  # the graph must hold for every later length
+        b.upload()
+        self.cache.take_fresh_slots()
+        g = self._graphs.get(bucket)
+        if g is None:
+            # once eagerly (first-use initialisation must not happen under capture; it writes the
+            # same cache slots with the same values as the replay will), then capture
+            self.model.forward(b, self.cache_views)
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, pool=self._graph_pool):
+                self.model.forward(b, self.cache_views)
+            if self._graph_pool is None:
+                self._graph_pool = g.pool()
+            self._graphs[bucket] = g
+        g.replay()
+        return self.model.logits[:n]
 
     # ---- request bookkeeping shared by replay and tests ------------------------------------------
     def reserve(self, req_id, start: int, n: int) -> bool:

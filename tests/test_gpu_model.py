@@ -212,3 +212,34 @@ def test_modes_agree_closely_in_32bit(model_dirs):
     for p in range(60):
         assert torch.equal(whole[("x", p)], single[("y", p)]), f"position {p}: token-by-token differs"
         assert torch.equal(whole[("x", p)], parts[("z", p)]), f"position {p}: portions differ"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_decode_graph_replays_equal_eager(model_dirs, dtype):
+    """Decode steps replayed from a captured HIP graph against the same steps run eagerly: every
+    replay is checked, with eager work (prompt portions of other requests) between the replays,
+    and with batches that grow and shrink across the graph's size buckets."""
+    from dinfer_amd.config import EngineOptions
+    from dinfer_amd.engine.runner import ModelRunner
+    name = "B"
+    cfg = CONFIGS[name][0]
+    seqs = {k: tokens_for(name, 60 + 7 * i, 300 + i) for i, k in enumerate("abc")}
+    runners = {}
+    for graph in (False, True):
+        opt = EngineOptions(dtype=dtype, max_model_len=cfg["max_position_embeddings"], max_num_seqs=4,
+                            max_num_batched_tokens=64, block_size=PAGE[name], num_blocks=128, max_logits_rows=64,
+                            decode_exempt_from_budget=False, hip_graph=graph)
+        runners[graph] = ModelRunner.from_dir(model_dirs[name], opt)
+    steps = [([("a", seqs["a"][:20], [19])], [])]
+    steps += [([("a", [seqs["a"][20 + i]], [0])], []) for i in range(3)]                    # bucket 1
+    steps += [([("b", seqs["b"][:33], [32])], [])]                                          # eager in between
+    steps += [([("a", [seqs["a"][23 + i]], [0]), ("b", [seqs["b"][33 + i]], [0])], []) for i in range(4)]  # bucket 2
+    steps += [([("c", seqs["c"][:9], [])], [])]
+    steps += [([(k, [seqs[k][n + i]], [0]) for k, n in (("a", 27), ("b", 37), ("c", 9))], []) for i in range(5)]  # bucket 4
+    steps += [([("b", [seqs["b"][42]], [0])], ["a"])]                                       # back to bucket 1
+    eager, replayed = replay(runners[False], steps), replay(runners[True], steps)
+    assert runners[True]._graphs and not runners[False]._graphs
+    assert eager.keys() == replayed.keys()
+    for k in eager:
+        # same kernels; only the split of the keys differs (the graph splits for the longest possible request)
+        torch.testing.assert_close(replayed[k], eager[k], rtol=1e-3, atol=1e-3, msg=lambda m: f"{k}: {m}")
