@@ -52,17 +52,62 @@ __device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
 
-// One block of 32 keys against NT column tiles. Shared by both kernels.
-//   qf[t][ks]   B operands of the score product (queries or heads), whole head in registers
+// Block-table entries of 64 consecutive pages of one request, one per lane; a lane gets the
+// entry it needs by a cross-lane read, so no key block waits for a table load of its own.
+struct Pages {
+  const int32_t* bt;
+  int max_blocks, base, reg, ps, ps_shift;
+
+  __device__ __forceinline__ void init(const int32_t* table, int max_blocks_, int page_size, int first_key) {
+    bt = table;
+    max_blocks = max_blocks_;
+    ps = page_size;
+    ps_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
+    fetch(page_of(first_key));
+  }
+  __device__ __forceinline__ int page_of(int key) const { return ps_shift >= 0 ? key >> ps_shift : key / ps; }
+  __device__ __forceinline__ int offset_of(int key) const { return ps_shift >= 0 ? key & (ps - 1) : key % ps; }
+  __device__ __forceinline__ void fetch(int first_page) {
+    base = first_page;
+    const int i = base + (int)(threadIdx.x & 63);
+    reg = i < max_blocks ? bt[i] : 0;
+  }
+  // kb is wave-uniform and only grows; afterwards the pages of keys [kb, kb + 32) are on board
+  __device__ __forceinline__ void ensure(int kb) {
+    if (page_of(kb + 31) - base >= 64) fetch(page_of(kb));
+  }
+  // every lane of the wave must call this (it is a cross-lane operation)
+  __device__ __forceinline__ int get(int page) const { return __shfl(reg, page - base, 64); }
+};
+
+template <int DT>
+struct Frags {
+  static constexpr int KS = (DT + 1) / 2;
+  bf16x8 k[2][KS];
+  bf16x8 v[DT];
+};
+
+// NT column tiles (queries, or the heads of a group) against the keys of one request, 32 at a time.
+//   qf[t][ks]   B operands of the score product, the whole head in registers
 //   col_lo/hi   per column tile and lane: the column's visible keys are [col_lo, col_hi)
 //   k_lo, k_hi  the keys this wave may touch at all (held pages, written slots)
+// load() issues the loads of one block, compute() consumes them; walk() keeps the next block's
+// loads in flight while the current one is computed.
 template <int DT, int NT>
 struct Tile {
   static constexpr int KS = (DT + 1) / 2;  // 32-wide steps over the head dimension
   f32x4 o[NT][DT];
   float m[NT], l[NT];
+  Pages pages;
+  const bf16* kc;
+  const bf16* vc;
+  int hk, Hkv, k_lo, k_hi;
+  float scale_log2e;
 
-  __device__ __forceinline__ void init() {
+  __device__ __forceinline__ void init(const bf16* kc_, const bf16* vc_, const int32_t* bt, int max_blocks, int hk_,
+                                       int Hkv_, int ps, int k_lo_, int k_hi_, float scale_log2e_) {
+    kc = kc_; vc = vc_; hk = hk_; Hkv = Hkv_; k_lo = k_lo_; k_hi = k_hi_; scale_log2e = scale_log2e_;
+    pages.init(bt, max_blocks, ps, k_lo_ & ~31);
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       m[t] = -INFINITY;
@@ -72,36 +117,47 @@ struct Tile {
     }
   }
 
-  __device__ __forceinline__ void block(const bf16x8 (&qf)[NT][KS], int kb, int k_lo, int k_hi, const int (&col_lo)[NT],
-                                        const int (&col_hi)[NT], bool need_mask, const bf16* __restrict__ kc,
-                                        const bf16* __restrict__ vc, const int32_t* __restrict__ bt, int hk, int Hkv,
-                                        int D, int ps, float scale_log2e) {
+  __device__ __forceinline__ void load(Frags<DT>& f, int kb) {
+    constexpr int D = DT * 16;
     const int lane = threadIdx.x & 63, i16 = lane & 15, g4 = lane >> 4;
-    // ---- scores ----
-    const int kg_row = kb + 8 * (i16 >> 2);  // the 8-key group of this lane's two K rows (one page: ps % 8 == 0)
+    const int ps = pages.ps;
+    pages.ensure(kb);
+    // K rows of this lane: keys kg_row + (i16 & 3) and + 4, in one page (page size % 8 == 0)
+    const int kg_row = kb + 8 * (i16 >> 2);
     const int key0 = kg_row + (i16 & 3), key1 = key0 + 4;
     const bool v0 = key0 >= k_lo && key0 < k_hi, v1 = key1 >= k_lo && key1 < k_hi;
-    const bf16* krow = kc;
-    if (v0 || v1) {
-      const int pg = bt[kg_row / ps];
-      krow = kc + (((int64_t)pg * Hkv + hk) * ps + (kg_row % ps) + (i16 & 3)) * D;
-    }
-    f32x4 s[NT][2];
-#pragma unroll
-    for (int t = 0; t < NT; ++t) s[t][0] = s[t][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const int pgk = pages.get(pages.page_of(kg_row));
+    const bf16* krow = kc + (((int64_t)pgk * Hkv + hk) * ps + pages.offset_of(kg_row) + (i16 & 3)) * D;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int d = ks * 32 + g4 * 8;
       const bool dv = d < D;  // D % 32 == 16: the upper half of the last step is padding
-      const bf16x8 k0 = (v0 && dv) ? *(const bf16x8*)(krow + d) : zero8();
-      const bf16x8 k1 = (v1 && dv) ? *(const bf16x8*)(krow + 4 * D + d) : zero8();
+      f.k[0][ks] = (v0 && dv) ? *(const bf16x8*)(krow + d) : zero8();
+      f.k[1][ks] = (v1 && dv) ? *(const bf16x8*)(krow + 4 * D + d) : zero8();
+    }
+    // V^T rows of this lane: d = 16 dt + i16, keys kg .. kg + 7
+    const int kg = kb + 8 * g4;
+    const bool vg = kg < k_hi && kg + 8 > k_lo;
+    const int pgv = pages.get(pages.page_of(kg));
+    const bf16* vrow = vc + (((int64_t)pgv * Hkv + hk) * D + i16) * ps + pages.offset_of(kg);
+#pragma unroll
+    for (int d = 0; d < DT; ++d) f.v[d] = vg ? *(const bf16x8*)(vrow + (int64_t)d * 16 * ps) : zero8();
+  }
+
+  __device__ __forceinline__ void compute(const Frags<DT>& f, const bf16x8 (&qf)[NT][KS], int kb,
+                                          const int (&col_lo)[NT], const int (&col_hi)[NT], bool need_mask) {
+    const int lane = threadIdx.x & 63, g4 = lane >> 4;
+    f32x4 s[NT][2];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) s[t][0] = s[t][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
-        s[t][0] = mfma16(k0, qf[t][ks], s[t][0]);
-        s[t][1] = mfma16(k1, qf[t][ks], s[t][1]);
+        s[t][0] = mfma16(f.k[0][ks], qf[t][ks], s[t][0]);
+        s[t][1] = mfma16(f.k[1][ks], qf[t][ks], s[t][1]);
       }
-    }
-    // ---- online softmax per column; this lane holds keys kb + 8 g4 + {0..7} of column i16 ----
+    // online softmax per column; this lane holds keys kb + 8 g4 + {0..7} of column i16
     const int kg = kb + 8 * g4;
     bf16x8 pf[NT];
 #pragma unroll
@@ -137,17 +193,11 @@ struct Tile {
 #pragma unroll
       for (int d = 0; d < DT; ++d) o[t][d] *= alpha;
     }
-    // ---- O^T += V^T . P ----
-    const bool vg = kg < k_hi && kg + 8 > k_lo;
-    const bf16* vrow = vc;
-    if (vg) {
-      const int pg = bt[kg / ps];
-      vrow = vc + (((int64_t)pg * Hkv + hk) * D + i16) * ps + (kg % ps);
-    }
+    // O^T += V^T . P
 #pragma unroll
     for (int d = 0; d < DT; ++d) {
-      bf16x8 vf = vg ? *(const bf16x8*)(vrow + (int64_t)d * 16 * ps) : zero8();
-      if (need_mask && vg) {
+      bf16x8 vf = f.v[d];
+      if (need_mask) {
         // a stale slot may hold anything; its weight is 0, but 0 * inf would poison the sum
 #pragma unroll
         for (int e = 0; e < 8; ++e)
@@ -155,6 +205,27 @@ struct Tile {
       }
 #pragma unroll
       for (int t = 0; t < NT; ++t) o[t][d] = mfma16(vf, pf[t], o[t][d]);
+    }
+  }
+
+  // All key blocks of [k_lo, k_hi); mask(kb) says whether block kb needs per-key masking.
+  template <class MaskFn>
+  __device__ __forceinline__ void walk(const bf16x8 (&qf)[NT][KS], const int (&col_lo)[NT], const int (&col_hi)[NT],
+                                       MaskFn mask) {
+    Frags<DT> f0, f1;
+    int kb = k_lo & ~31;
+    if (kb >= k_hi) return;
+    load(f0, kb);
+    while (true) {
+      const bool more1 = kb + 32 < k_hi;
+      if (more1) load(f1, kb + 32);
+      compute(f0, qf, kb, col_lo, col_hi, mask(kb));
+      if (!more1) break;
+      const bool more2 = kb + 64 < k_hi;
+      if (more2) load(f0, kb + 64);
+      compute(f1, qf, kb + 32, col_lo, col_hi, mask(kb + 32));
+      if (!more2) break;
+      kb += 64;
     }
   }
 
@@ -216,11 +287,10 @@ __global__ void __launch_bounds__(256) attn_flash_kernel(
   const int k_lo = window > 0 ? (p_first - window + 1 > 0 ? p_first - window + 1 : 0) : 0;
 
   Tile<DT, QT> tl;
-  tl.init();
-  for (int kb = k_lo & ~31; kb < k_hi; kb += 32) {
-    const bool need_mask = kb + 31 > p_first || kb < k_lo || (window > 0 && kb < p_last - window + 1);
-    tl.block(qf, kb, k_lo, k_hi, col_lo, col_hi, need_mask, kc, vc, bt, hk, Hkv, D, ps, scale_log2e);
-  }
+  tl.init(kc, vc, bt, (int)max_blocks, hk, Hkv, ps, k_lo, k_hi, scale_log2e);
+  tl.walk(qf, col_lo, col_hi, [&](int kb) {
+    return kb + 31 > p_first || kb < k_lo || (window > 0 && kb < p_last - window + 1);
+  });
 #pragma unroll
   for (int t = 0; t < QT; ++t) {
     const float lt = tl.sum_l(t);
@@ -239,13 +309,25 @@ __global__ void __launch_bounds__(256) attn_flash_kernel(
   }
 }
 
+// The keys a request's row sees, [first, seq), are cut into `splits` equal parts of a multiple of
+// 32 keys; short requests leave the last parts empty. Computed alike by the decode and merge kernels.
+__device__ __forceinline__ void split_range(int seq, int window, int splits, int sp, int* k_lo, int* k_hi, int* kps) {
+  const int first = window > 0 ? (seq - window > 0 ? seq - window : 0) : 0;  // the row's position is seq - 1
+  const int base = first & ~31;
+  const int per = (((seq - base) + splits - 1) / splits + 31) & ~31;
+  const int lo = base + sp * per, hi = lo + per;
+  *k_lo = lo > first ? lo : first;
+  *k_hi = hi < seq ? hi : seq;
+  *kps = per;
+}
+
 // One wave per (split, kv head, request). part: [B, H, splits, D + 4] float = (m in base-2 units, l, -, -, o[D]).
 template <int DT>
 __global__ void __launch_bounds__(64) attn_decode_kernel(
     const bf16* __restrict__ q, int64_t ld_q, float* __restrict__ part, const bf16* __restrict__ kc,
     const bf16* __restrict__ vc, const int32_t* __restrict__ block_table, int64_t max_blocks,
-    const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_lens, int keys_per_split, int splits,
-    float scale_log2e, int window, int H, int Hkv, int ps) {
+    const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_lens, int splits, float scale_log2e,
+    int window, int H, int Hkv, int ps) {
   constexpr int D = DT * 16;
   constexpr int KS = (DT + 1) / 2;
   const int sp = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
@@ -255,11 +337,9 @@ __global__ void __launch_bounds__(64) attn_decode_kernel(
     row = cu_seqlens[b];
     if (cu_seqlens[b + 1] - row != 1) return;  // a longer run of rows belongs to the flash kernel
   }
-  const int seq = seq_lens[b];
-  const int first = window > 0 ? (seq - window > 0 ? seq - window : 0) : 0;  // the row's position is seq - 1
-  const int k_lo = sp * keys_per_split > first ? sp * keys_per_split : first;
-  const int k_hi = (sp + 1) * keys_per_split < seq ? (sp + 1) * keys_per_split : seq;
-  if (k_lo >= k_hi) return;  // a dead split writes nothing; the merge kernel knows which are live
+  int k_lo, k_hi, kps;
+  split_range(seq_lens[b], window, splits, sp, &k_lo, &k_hi, &kps);
+  if (k_lo >= k_hi) return;  // an empty part writes nothing; the merge kernel skips it by the same rule
   const int lane = threadIdx.x & 63, i16 = lane & 15, g4 = lane >> 4;
   const int32_t* bt = block_table + (int64_t)b * max_blocks;
 
@@ -275,11 +355,8 @@ __global__ void __launch_bounds__(64) attn_decode_kernel(
   }
   const int col_lo[1] = {k_lo}, col_hi[1] = {k_hi};
   Tile<DT, 1> tl;
-  tl.init();
-  for (int kb = k_lo & ~31; kb < k_hi; kb += 32) {
-    const bool need_mask = kb < k_lo || kb + 32 > k_hi;
-    tl.block(qf, kb, k_lo, k_hi, col_lo, col_hi, need_mask, kc, vc, bt, hk, Hkv, D, ps, scale_log2e);
-  }
+  tl.init(kc, vc, bt, (int)max_blocks, hk, Hkv, ps, k_lo, k_hi, scale_log2e);
+  tl.walk(qf, col_lo, col_hi, [&](int kb) { return kb < k_lo || kb + 32 > k_hi; });
   const float lt = tl.sum_l(0);
   if (i16 < G) {
     float* pp = part + (((int64_t)b * H + hk * G + i16) * splits + sp) * (D + 4);
@@ -292,34 +369,51 @@ __global__ void __launch_bounds__(64) attn_decode_kernel(
   }
 }
 
-// out[b, h, :] = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s over the live splits.
-__global__ void __launch_bounds__(256) attn_decode_merge_kernel(const float* __restrict__ part, bf16* __restrict__ out,
-                                                                int64_t ld_out, const int32_t* __restrict__ cu_seqlens,
-                                                                const int32_t* __restrict__ seq_lens,
-                                                                int keys_per_split, int splits, int window, int H,
-                                                                int D) {
-  const int h = blockIdx.x, b = blockIdx.y;
+constexpr int MAX_SPLITS = 256;
+
+// out[b, h, :] = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s over the non-empty parts. One wave per (head, request).
+__global__ void __launch_bounds__(64) attn_decode_merge_kernel(const float* __restrict__ part, bf16* __restrict__ out,
+                                                               int64_t ld_out, const int32_t* __restrict__ cu_seqlens,
+                                                               const int32_t* __restrict__ seq_lens, int splits,
+                                                               int window, int H, int D) {
+  __shared__ float wgt[MAX_SPLITS];
+  const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
   int row = b;
   if (cu_seqlens) {
     row = cu_seqlens[b];
     if (cu_seqlens[b + 1] - row != 1) return;
   }
   const int seq = seq_lens[b];
-  const int first = window > 0 ? (seq - window > 0 ? seq - window : 0) : 0;
-  const int s_lo = first / keys_per_split;
-  const int s_hi = (seq + keys_per_split - 1) / keys_per_split;
   const float* pp = part + ((int64_t)b * H + h) * splits * (D + 4);
-  float M = -INFINITY;
-  for (int s = s_lo; s < s_hi; ++s) M = fmaxf(M, pp[(int64_t)s * (D + 4)]);
-  for (int d = threadIdx.x; d < D; d += blockDim.x) {
-    float acc = 0.f, L = 0.f;
-    for (int s = s_lo; s < s_hi; ++s) {
-      const float* ps_ = pp + (int64_t)s * (D + 4);
-      const float a = ps_[0] == -INFINITY ? 0.f : exp2f(ps_[0] - M);
-      acc += a * ps_[4 + d];
-      L += a * ps_[1];
+  float mloc = -INFINITY;
+  for (int s = lane; s < splits; s += 64) {
+    int k_lo, k_hi, kps;
+    split_range(seq, window, splits, s, &k_lo, &k_hi, &kps);
+    const float m = k_lo < k_hi ? pp[(int64_t)s * (D + 4)] : -INFINITY;
+    wgt[s] = m;
+    mloc = fmaxf(mloc, m);
+  }
+  const float M = wave_max(mloc);
+  float lloc = 0.f;
+  for (int s = lane; s < splits; s += 64) {
+    const float m = wgt[s];
+    const float a = m == -INFINITY ? 0.f : exp2f(m - M);
+    wgt[s] = a;
+    const float lv = pp[(int64_t)s * (D + 4) + 1];  // read unconditionally (an empty part holds anything)
+    lloc += a > 0.f ? a * lv : 0.f;
+  }
+  const float L = wave_sum(lloc);
+  __syncthreads();
+  const float inv = L > 0.f ? 1.f / L : 0.f;
+  for (int d = lane; d < D; d += 64) {
+    float acc = 0.f;
+#pragma unroll 8
+    for (int s = 0; s < splits; ++s) {
+      const float a = wgt[s];
+      const float v = pp[(int64_t)s * (D + 4) + 4 + d];  // loads do not wait for the weights
+      acc += a > 0.f ? a * v : 0.f;
     }
-    out[(int64_t)row * ld_out + (int64_t)h * D + d] = (bf16)(L > 0.f ? acc / L : 0.f);
+    out[(int64_t)row * ld_out + (int64_t)h * D + d] = (bf16)(acc * inv);
   }
 }
 
@@ -350,13 +444,13 @@ int launch_flash(const bf16* q, int64_t ld_q, bf16* out, int64_t ld_out, const b
 
 template <int DT>
 int launch_decode(const bf16* q, int64_t ld_q, bf16* out, int64_t ld_out, float* part, const bf16* kc, const bf16* vc,
-                  const int32_t* bt, int64_t max_blocks, const int32_t* cu, const int32_t* sl, int num_reqs, int keys_per_split,
+                  const int32_t* bt, int64_t max_blocks, const int32_t* cu, const int32_t* sl, int num_reqs,
                   int splits, float scale, int window, int H, int Hkv, int ps, hipStream_t stream) {
   attn_decode_kernel<DT><<<dim3((unsigned)splits, (unsigned)Hkv, (unsigned)num_reqs), 64, 0, stream>>>(
-      q, ld_q, part, kc, vc, bt, max_blocks, cu, sl, keys_per_split, splits, scale * LOG2E, window, H, Hkv, ps);
+      q, ld_q, part, kc, vc, bt, max_blocks, cu, sl, splits, scale * LOG2E, window, H, Hkv, ps);
   const int D = DT * 16;
-  attn_decode_merge_kernel<<<dim3((unsigned)H, (unsigned)num_reqs), D <= 64 ? 64 : (D <= 128 ? 128 : 256), 0, stream>>>(
-      part, out, ld_out, cu, sl, keys_per_split, splits, window, H, D);
+  attn_decode_merge_kernel<<<dim3((unsigned)H, (unsigned)num_reqs), 64, 0, stream>>>(part, out, ld_out, cu, sl, splits,
+                                                                                     window, H, D);
   return launch_status();
 }
 
@@ -399,23 +493,21 @@ extern "C" int dinfer_attn_flash(const void* q, int64_t ld_q, void* out, int64_t
 
 // Single-row requests only. cu_seqlens null: every request brings exactly one row (row b belongs to
 // request b). cu_seqlens given: requests with one row are served, the others are left alone.
-// part: float workspace of num_reqs * heads * splits * (head_dim + 4) elements, where
-// splits = ceil(max_len / keys_per_split) and max_len bounds every seq_len.
+// Each request's visible keys are cut into `splits` (1..256) equal parts, one wave each.
+// part: float workspace of num_reqs * heads * splits * (head_dim + 4) elements.
 extern "C" int dinfer_attn_decode(const void* q, int64_t ld_q, void* out, int64_t ld_out, float* part,
                                   int64_t part_elems, const void* k_cache, const void* v_cache,
                                   const int32_t* block_table, int64_t max_blocks, const int32_t* cu_seqlens,
-                                  const int32_t* seq_lens, int num_reqs, int max_len, int keys_per_split, float scale, int window, int heads,
-                                  int kv_heads, int head_dim, int page_size, hipStream_t stream) {
+                                  const int32_t* seq_lens, int num_reqs, int splits, float scale, int window,
+                                  int heads, int kv_heads, int head_dim, int page_size, hipStream_t stream) {
   if (num_reqs <= 0) return OK;
   if (!dinfer_attn_mfma_supports(head_dim, page_size, heads, kv_heads)) return ERR_UNSUPPORTED;
   if (heads / kv_heads > 16) return ERR_UNSUPPORTED;
-  if (window < 0 || max_blocks <= 0 || max_len <= 0 || keys_per_split <= 0 || keys_per_split % 32 || ld_q % 8 ||
-      !aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(part) || num_reqs > 65535 ||
-      kv_heads > 65535)
+  if (window < 0 || max_blocks <= 0 || splits <= 0 || splits > MAX_SPLITS || ld_q % 8 || !aligned16(q) ||
+      !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(part) || num_reqs > 65535 || kv_heads > 65535)
     return ERR_BAD_SHAPE;
-  const int splits = (max_len + keys_per_split - 1) / keys_per_split;
   if ((int64_t)num_reqs * heads * splits * (head_dim + 4) > part_elems) return 5;
   DINFER_DISPATCH_HEAD_DIM(head_dim, return launch_decode<DT>(
       (const bf16*)q, ld_q, (bf16*)out, ld_out, part, (const bf16*)k_cache, (const bf16*)v_cache, block_table,
-      max_blocks, cu_seqlens, seq_lens, num_reqs, keys_per_split, splits, scale, window, heads, kv_heads, page_size, stream));
+      max_blocks, cu_seqlens, seq_lens, num_reqs, splits, scale, window, heads, kv_heads, page_size, stream));
 }

@@ -63,7 +63,31 @@ __device__ int block_argmax(float v, int i, Red& red, float* best_out) {
 __device__ int row_argmax(const float* row, int vocab, Red& red) {
   float best = -INFINITY;
   int besti = 0x7fffffff;
-  for (int i = threadIdx.x; i < vocab; i += BLOCK) better(best, besti, row[i], i);
+  int i0 = 0;
+  if (((uintptr_t)row & 15) == 0) {
+    // 16-byte loads, four in flight per thread; a thread's indices still grow, so ties keep the lowest
+    const f32x4* r4 = (const f32x4*)row;
+    const int n4 = vocab >> 2;
+    int j = threadIdx.x;
+    for (; j + 3 * BLOCK < n4; j += 4 * BLOCK) {
+      const f32x4 a = r4[j], b = r4[j + BLOCK], c = r4[j + 2 * BLOCK], d = r4[j + 3 * BLOCK];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) better(best, besti, a[e], 4 * j + e);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) better(best, besti, b[e], 4 * (j + BLOCK) + e);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) better(best, besti, c[e], 4 * (j + 2 * BLOCK) + e);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) better(best, besti, d[e], 4 * (j + 3 * BLOCK) + e);
+    }
+    for (; j < n4; j += BLOCK) {
+      const f32x4 a = r4[j];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) better(best, besti, a[e], 4 * j + e);
+    }
+    i0 = n4 << 2;
+  }
+  for (int i = i0 + threadIdx.x; i < vocab; i += BLOCK) better(best, besti, row[i], i);
   const int r = block_argmax(best, besti, red, nullptr);
   return r == 0x7fffffff ? 0 : r;
 }

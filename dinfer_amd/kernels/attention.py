@@ -11,8 +11,8 @@ import torch
 
 from . import ops
 
-TARGET_WAVES = 4096   # split-K aims at about this many waves in flight
-MIN_KEYS_PER_SPLIT = 64
+TARGET_WAVES = 1024   # split-K aims at about this many waves (measured: more, shorter waves cost more than they hide)
+MAX_SPLITS = 32
 
 
 class Workspace:
@@ -23,16 +23,15 @@ class Workspace:
         self.mfma = (ctx.dtype == torch.bfloat16 and ops.attn_mfma_supports(head_dim, ctx.page_size, heads, kv_heads))
         self.split_k = self.mfma and heads // kv_heads <= 16
         self.part = None
+        self.kv_heads = kv_heads
         if self.split_k:
-            max_units = TARGET_WAVES + ctx.max_reqs * kv_heads  # (request, kv head, split) triples at most
+            max_units = max(self.splits(n) * n for n in range(1, ctx.max_reqs + 1)) * kv_heads
             elems = max_units * (heads // kv_heads) * (head_dim + 4)
             self.part = ctx.workspace.buffer("attn_partials", elems, dtype=torch.float32, rows=1)
-        self.kv_heads = kv_heads
 
-    def keys_per_split(self, num_reqs: int, max_len: int) -> int:
-        splits = max(1, TARGET_WAVES // (num_reqs * self.kv_heads))
-        kps = -(-max_len // splits)
-        return max(MIN_KEYS_PER_SPLIT, (kps + 31) // 32 * 32)
+    def splits(self, num_reqs: int) -> int:
+        """Parts per request: a function of the batch size only, so a captured graph stays valid."""
+        return max(1, min(MAX_SPLITS, TARGET_WAVES // (num_reqs * self.kv_heads)))
 
 
 def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k_cache, v_cache, batch, group: int, ws: Workspace, *,
@@ -47,10 +46,8 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k_cache, v_cache, batc
     # a few single rows beside long portions are not worth two more launches
     use_decode = singles == B or singles >= 4
     if use_decode:
-        max_len = batch.max_len_bound
-        kps = ws.keys_per_split(B, max_len)
         ops.attn_decode(qkv, out, ws.part, k_cache, v_cache, bt, None if singles == B else batch.cu_seqlens,
-                        batch.seq_lens, B, max_len, kps, **geo)
+                        batch.seq_lens, B, ws.splits(B), **geo)
         if singles == B:
             return out
     return ops.attn_flash(qkv, out, k_cache, v_cache, bt, batch.cu_seqlens, batch.seq_lens, B, T, batch.max_q_len,

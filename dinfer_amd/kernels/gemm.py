@@ -12,6 +12,9 @@ import torch
 from . import ops
 
 
+SMALL_M = 16  # up to this many rows the weight-streaming kernel beats the library (measured on MI355X)
+
+
 def matmul_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int) -> torch.Tensor:
     """out[:m] = a[:m] @ w.T; out has a's dtype, or float32 (logits)."""
     if m <= 0:
@@ -20,7 +23,11 @@ def matmul_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int) -> to
         return ops.gemm_ref(a, w, out, m)
     if not a.is_cuda:
         raise RuntimeError("matrix products run on the GPU only")
+    if m <= SMALL_M and w.shape[1] % 8 == 0:
+        return ops.gemm_small_m(a, w, out, m)
     if out.dtype == torch.float32:
+        if m <= 64 and w.shape[1] % 8 == 0:
+            return ops.gemm_small_m(a, w, out, m)  # float logits straight from the accumulators
         tmp = torch.mm(a[:m], w.t())
         ops.widen(tmp, out, m * w.shape[0]) if out.is_contiguous() else out[:m].copy_(tmp)
         return out

@@ -40,9 +40,10 @@ SIGNATURES = {
     ),
     "dinfer_attn_decode": (
         "attention",
-        [_P, _L, _P, _L, _P, _L, _P, _P, _P, _L, _P, _P, _I, _I, _I, _F, _I, _I, _I, _I, _I, _P],
+        [_P, _L, _P, _L, _P, _L, _P, _P, _P, _L, _P, _P, _I, _I, _F, _I, _I, _I, _I, _I, _P],
     ),
     "dinfer_gemm_ref": ("gemm_ref", [_I, _I, _P, _L, _P, _L, _P, _L, _L, _L, _L, _P]),
+    "dinfer_gemm_small_m": ("gemm", [_I, _P, _L, _P, _L, _P, _L, _L, _L, _L, _I, _I, _P]),
     "dinfer_argmax": ("sampling", [_P, _L, _P, _L, _L, _P]),
     "dinfer_sample": ("sampling", [_P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _P]),
     "dinfer_penalties": ("sampling", [_P, _L, _P, _P, _P, _P, _P, _P, _L, _L, _P]),

@@ -211,18 +211,18 @@ def attn_flash(q, out, k_cache, v_cache, block_table, cu_seqlens, seq_lens, num_
     return out
 
 
-def attn_decode(q, out, part, k_cache, v_cache, block_table, cu_seqlens, seq_lens, num_reqs: int, max_len: int,
-                keys_per_split: int, *, scale: float, window: int, heads: int, kv_heads: int, head_dim: int,
-                page_size: int):
+def attn_decode(q, out, part, k_cache, v_cache, block_table, cu_seqlens, seq_lens, num_reqs: int, splits: int, *,
+                scale: float, window: int, heads: int, kv_heads: int, head_dim: int, page_size: int):
     """Split-K attention for requests that bring one row. cu_seqlens None: row b is request b;
-    given: only the requests with one row are served (mixed batches)."""
+    given: only the requests with one row are served (mixed batches). Each request's keys are cut
+    into `splits` equal parts on the device, so the launch shape does not depend on the lengths."""
     _need_gpu(q, out, part, k_cache, v_cache, block_table, cu_seqlens, seq_lens)
     _check_paged(q, out, k_cache, v_cache, block_table, seq_lens, num_reqs, heads, kv_heads, head_dim, page_size)
     assert part.dtype == torch.float32 and part.is_contiguous()
     lib.call("dinfer_attn_decode", q.data_ptr(), _rows(q), out.data_ptr(), _rows(out), part.data_ptr(),
              part.numel(), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1],
-             _ptr(cu_seqlens), seq_lens.data_ptr(), num_reqs, max_len, keys_per_split, float(scale), int(window),
-             heads, kv_heads, head_dim, page_size, _stream())
+             _ptr(cu_seqlens), seq_lens.data_ptr(), num_reqs, splits, float(scale), int(window), heads, kv_heads,
+             head_dim, page_size, _stream())
     return out
 
 
@@ -237,6 +237,18 @@ def gemm_ref(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int) -> tor
         assert out.dtype == a.dtype
     lib.call("dinfer_gemm_ref", dtype_code(a.dtype), out_f32, a.data_ptr(), _rows(a), w.data_ptr(), _rows(w),
              out.data_ptr(), _rows(out), m, n, k, _stream())
+    return out
+
+
+def gemm_small_m(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, *, row_tiles: int = 0,
+                 waves: int = 0) -> torch.Tensor:
+    """out[:m] = a[:m] @ w.T for m <= 64, bf16 operands, weight streamed once (MFMA, split-K in the workgroup)."""
+    _need_gpu(a, w, out)
+    n, k = w.shape
+    assert a.dtype == w.dtype == torch.bfloat16 and a.shape[1] == k and out.shape[1] == n
+    assert a.shape[0] >= m and out.shape[0] >= m and out.dtype in (torch.bfloat16, torch.float32)
+    lib.call("dinfer_gemm_small_m", 1 if out.dtype == torch.float32 else 0, a.data_ptr(), _rows(a), w.data_ptr(),
+             _rows(w), out.data_ptr(), _rows(out), m, n, k, row_tiles, waves, _stream())
     return out
 
 

@@ -237,14 +237,13 @@ def test_attention_flash(H, Hkv, D, page, window):
 @pytest.mark.parametrize("H,Hkv,D,page", GEOS)
 def test_attention_decode_split_k(H, Hkv, D, page, window):
     # 300 / 70 / 1: several splits, a short one, a single key; then 1..64 at batch 32
-    for hist, kps in (([299, 69, 0, 1000], 64), ([random.Random(7).randrange(64) for _ in range(32)], 256)):
+    for hist, splits in (([299, 69, 0, 1000], 7), ([random.Random(7).randrange(64) for _ in range(32)], 2),
+                         ([5000, 31, 32], 64), ([100, 200], 1)):
         new = [1] * len(hist)
         q, kc, vc, m, outs = paged_case(torch.bfloat16, H, Hkv, D, page, hist, new, seed=5)
         out = torch.zeros(len(hist), H * D, device=DEV, dtype=torch.bfloat16)
-        max_len = max(hist) + 1
-        splits = -(-max_len // kps)
-        part = torch.full((len(hist) * H * splits * (D + 4),), float("nan"), device=DEV)
-        ops().attn_decode(q, out, part, kc, vc, m["bt"], None, m["sl"], len(hist), max_len, kps, scale=D ** -0.5,
+        part = torch.full((len(hist) * H * splits * (D + 4),), float("nan"), device=DEV)  # empty parts stay NaN
+        ops().attn_decode(q, out, part, kc, vc, m["bt"], None, m["sl"], len(hist), splits, scale=D ** -0.5,
                           window=window, heads=H, kv_heads=Hkv, head_dim=D, page_size=page)
         want = expected_attention(outs, hist, D ** -0.5, window)
         torch.testing.assert_close(out.double().cpu().view(-1, H, D), want, rtol=2e-2, atol=2e-2)
@@ -255,10 +254,10 @@ def test_attention_mixed_routes_single_rows_to_split_k():
     hist, new = [500, 0, 64, 900, 33, 10], [1, 40, 1, 1, 20, 1]
     q, kc, vc, m, outs = paged_case(torch.bfloat16, H, Hkv, D, page, hist, new, seed=9)
     out = torch.zeros(sum(new), H * D, device=DEV, dtype=torch.bfloat16)
-    max_len, kps = max(h + n for h, n in zip(hist, new)), 128
-    part = torch.zeros(len(hist) * H * (-(-max_len // kps)) * (D + 4), device=DEV)
+    splits = 5
+    part = torch.zeros(len(hist) * H * splits * (D + 4), device=DEV)
     geo = dict(scale=D ** -0.5, window=0, heads=H, kv_heads=Hkv, head_dim=D, page_size=page)
-    ops().attn_decode(q, out, part, kc, vc, m["bt"], m["cu"], m["sl"], len(hist), max_len, kps, **geo)
+    ops().attn_decode(q, out, part, kc, vc, m["bt"], m["cu"], m["sl"], len(hist), splits, **geo)
     ops().attn_flash(q, out, kc, vc, m["bt"], m["cu"], m["sl"], len(hist), sum(new), max(new), skip_single=True, **geo)
     want = expected_attention(outs, hist, D ** -0.5, 0)
     torch.testing.assert_close(out.double().cpu().view(-1, H, D), want, rtol=2e-2, atol=2e-2)
@@ -279,7 +278,7 @@ def test_attention_finds_one_far_key(kernel):
         ops().attn_flash(q, out, kc, vc, m["bt"], m["cu"], m["sl"], 1, 1, 1, **geo)
     else:
         part = torch.zeros(H * 11 * (D + 4), device=DEV)
-        ops().attn_decode(q, out, part, kc, vc, m["bt"], None, m["sl"], 1, 700, 64, **geo)
+        ops().attn_decode(q, out, part, kc, vc, m["bt"], None, m["sl"], 1, 11, **geo)
     want = expected_attention(outs, hist, D ** -0.5, 0)
     torch.testing.assert_close(out.double().cpu().view(-1, H, D), want, rtol=2e-2, atol=2e-2)
     # the spiked heads (one per kv head) really are dominated by key 5
@@ -394,3 +393,18 @@ def test_penalties_match_plain_rule():
     for r, (p, o) in enumerate(hist):
         want = plain.apply_penalties(logits[r].cpu().double(), p, o, rep[r], freq[r], pres[r])
         torch.testing.assert_close(got[r].cpu().double(), want, rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 33, 64])
+def test_gemm_small_m(M, out_dtype):
+    """Weight-streaming MFMA product against float64, at sizes that are no multiples of its tiles."""
+    for N, K in ((96, 512), (331, 80), (4096, 4096), (1000, 1096), (50, 8)):
+        a = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+        w = (torch.randn(N, K, device=DEV) * 0.05).to(torch.bfloat16)
+        want = a.double() @ w.double().T
+        for rt, waves in ((0, 0), (1, 1), (2, 4), (1, 16), (4, 2) if M <= 32 else (2, 8)):
+            out = torch.full((M, N), float("nan"), device=DEV, dtype=out_dtype)
+            ops().gemm_small_m(a, w, out, M, row_tiles=rt, waves=waves)
+            t = dict(rtol=2e-2, atol=2e-2) if out_dtype == torch.bfloat16 else dict(rtol=1e-4, atol=1e-4)
+            torch.testing.assert_close(out.double(), want, **t, msg=lambda m_: f"M={M} N={N} K={K} rt={rt} waves={waves}: {m_}")
