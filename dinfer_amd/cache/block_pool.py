@@ -1,8 +1,8 @@
 """A pool of cache pages.
 
 ``allocate(n)`` is all-or-nothing and takes pages from the head of the free
-list; ``free(ids)`` puts pages back at the head, so a page that was just given
-back is the next one handed out (crates/core/src/kv/block_pool.rs:128-147,160-182;
+list; ``free(ids)`` puts the pages back at the head in the order given, so pages
+that were just given back are the next ones handed out (crates/core/src/kv/block_pool.rs:128-147,160-182;
 this engine has no prefix cache, so there is no LRU tail).
 A page is held by at most one owner; freeing a page that is not held raises.
 """
@@ -35,11 +35,15 @@ class BlockPool:
         return out
 
     def free(self, ids) -> None:
+        ids = list(ids)
         for b in ids:
             if not (0 <= b < self.num_blocks) or not self._held[b]:
                 raise RuntimeError(f"page {b} is freed but not held")
             self._held[b] = 0
-            self._free.appendleft(b)
+        self._free.extendleft(reversed(ids))
+
+    def free_list(self) -> list[int]:
+        return list(self._free)
 
     def is_held(self, b: int) -> bool:
         return bool(self._held[b])

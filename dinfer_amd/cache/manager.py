@@ -135,8 +135,8 @@ class CacheManager:
         return n
 
     def free(self, req_id) -> None:
-        """Gives back everything the request holds. Pages are freed last-first, so the
-        head of the free list is the request's first page (kv/manager.rs:338-345)."""
+        """Gives back everything the request holds, the last page first, so the tail of a
+        request is what the next allocation takes (kv/manager.rs:338-345)."""
         r = self._reqs.pop(req_id)
         for pool, tab in zip(self.pools, r.tables):
             pool.free([b for b in reversed(tab) if b >= 0])

@@ -1,0 +1,142 @@
+"""The flat batch a step is built into (no GPU), against the exact plans the reference's runner tests
+hold (crates/core/src/runner.rs:1058-1148), and the Engine loop with a stand-in runner."""
+import numpy as np
+import torch
+
+from dinfer_amd.cache import CacheManager, GroupSpec
+from dinfer_amd.config import EngineOptions
+from dinfer_amd.engine.batch import Entry, StepBatch
+from dinfer_amd.engine.request import Request
+from dinfer_amd.engine.scheduler import Scheduler
+from dinfer_amd.sampling import SamplingParams
+
+
+def setup(budget):
+    opt = EngineOptions(max_num_seqs=8, max_num_batched_tokens=budget, block_size=16, max_model_len=4096,
+                        num_blocks=64, decode_exempt_from_budget=False)
+    cache = CacheManager([GroupSpec(16, 64)], 8)
+    return Scheduler(opt, cache, eos_token_ids=[]), StepBatch(torch.device("cpu"), 1024, 8, 8, [4])
+
+
+def run(s, b):
+    """schedule -> fill -> echo executor (token = 1000 + seq_len, runner.rs:888-905) -> update."""
+    out = s.schedule()
+    entries = [Entry(x.request.id, x.request.tokens(x.start, x.num_new), x.start, [x.num_new - 1] if x.samples else [])
+               for x in out.scheduled]
+    b.fill(entries, s.cache)
+    sampled = {x.request.id: 1000 + x.start + x.num_new for x in out.scheduled if x.samples}
+    s.update(out, sampled)
+    return out
+
+
+def test_two_requests_prefill_then_decode_then_finish():
+    s, b = setup(1000)
+    sp = lambda n: SamplingParams(max_tokens=n, temperature=0.0)
+    r1, r2 = Request(1, list(range(20)), sp(3)), Request(2, list(range(5)), sp(2))
+    s.add_request(r1)
+    s.add_request(r2)
+    run(s, b)
+    h = b.h
+    assert b.req_ids == [1, 2] and (b.num_tokens, b.num_reqs, b.num_rows) == (25, 2, 2)
+    assert h["cu_seqlens"][:3].tolist() == [0, 20, 25] and h["logits_rows"][:2].tolist() == [19, 24]
+    assert h["positions"][20:25].tolist() == [0, 1, 2, 3, 4]
+    # request 1 holds pages 0, 1 and request 2 page 2: slot = page * 16 + offset
+    assert h["slot_mapping0"][16] == 16 and h["slot_mapping0"][20] == 32
+    assert h["block_table0"][:2, :2].tolist() == [[0, 1], [2, -1]]
+    assert not b.all_decode and b.max_q_len == 20
+    assert r1.output_ids == [1020] and r2.output_ids == [1005]
+    run(s, b)   # two decode rows
+    assert h["input_ids"][:2].tolist() == [1020, 1005] and h["positions"][:2].tolist() == [20, 5]
+    assert h["seq_lens"][:2].tolist() == [21, 6] and h["slot_mapping0"][:2].tolist() == [20, 37]
+    assert h["logits_rows"][:2].tolist() == [0, 1] and b.all_decode
+    assert r2.finish_reason == "length"
+    run(s, b)
+    assert r1.finish_reason == "length" and r1.num_tokens == 23 and not s.has_unfinished()
+
+
+def test_mixed_and_chunked_batches():
+    s, b = setup(12)
+    sp = SamplingParams(max_tokens=4, temperature=0.0)
+    r1 = Request(1, list(range(20)), sp)
+    s.add_request(r1)
+    out = run(s, b)
+    assert [(x.request.id, x.num_new) for x in out.scheduled] == [(1, 12)]
+    assert b.num_rows == 0 and r1.output_ids == []          # a mid-prompt portion samples nothing
+    r2 = Request(2, list(range(4)), sp)
+    s.add_request(r2)
+    out = run(s, b)
+    assert [(x.request.id, x.num_new) for x in out.scheduled] == [(1, 8), (2, 4)]
+    h = b.h
+    assert h["cu_seqlens"][:3].tolist() == [0, 8, 12] and h["positions"][:8].tolist() == list(range(12, 20))
+    assert h["seq_lens"][:2].tolist() == [20, 4] and h["logits_rows"][:2].tolist() == [7, 11]
+    assert r1.output_ids == [1020] and r2.output_ids == [1004]
+    run(s, b)
+    assert b.all_decode and h["input_ids"][:2].tolist() == [1020, 1004]
+
+
+def test_padding_for_a_graph_bucket():
+    s, b = setup(1000)
+    for i, n in ((1, 20), (2, 5), (3, 7)):
+        s.add_request(Request(i, list(range(n)), SamplingParams(max_tokens=5)))
+    run(s, b)
+    out = s.schedule()
+    entries = [Entry(x.request.id, x.request.tokens(x.start, 1), x.start, [0]) for x in out.scheduled]
+    b.fill(entries, s.cache, pad_to=4)
+    h = b.h
+    assert (b.num_tokens, b.num_reqs, b.num_rows) == (4, 4, 4) and b.q_lens == [1, 1, 1, 1]
+    assert h["cu_seqlens"][:5].tolist() == [0, 1, 2, 3, 4] and h["seq_lens"][:4].tolist() == [21, 6, 8, 1]
+    assert h["slot_mapping0"][3] == -1 and h["block_table0"][3].tolist() == [0, 0, 0, 0]   # writes nothing, reads page 0
+    assert h["logits_rows"][:4].tolist() == [0, 1, 2, 3]
+
+
+def test_limits_are_refused():
+    import pytest
+    s, b = setup(1000)
+    s.cache.admit("x")
+    s.cache.allocate("x", 0, 40)
+    with pytest.raises(ValueError, match="outside its"):
+        b.fill([Entry("x", [1, 2], 0, [2])], s.cache)
+    with pytest.raises(ValueError, match="brings no token"):
+        b.fill([Entry("x", [1], 0, []), Entry("x", [], 1, [])], s.cache)
+    small = StepBatch(torch.device("cpu"), 8, 1, 2, [1])
+    with pytest.raises(ValueError, match="tokens in one step"):
+        small.fill([Entry("x", list(range(9)), 0, [])], s.cache)
+    with pytest.raises(ValueError, match="block table"):
+        small.fill([Entry("x", list(range(8)), 0, [])], s.cache)
+
+
+def test_engine_loop_with_a_stand_in_runner():
+    """Engine.generate over scheduler and sampler seams, with a runner that returns one-hot logits
+    for token (seq_len % vocab): checks ordering of outputs, chunking, finishing and freeing."""
+    from dinfer_amd.engine.engine import Engine
+
+    class FakeModel:
+        class spec:
+            vocab_size = 50
+            eos_token_ids = (49,)
+
+    class FakeRunner:
+        def __init__(self):
+            self.options = EngineOptions(max_num_seqs=3, max_num_batched_tokens=16, block_size=4, max_model_len=64,
+                                         num_blocks=32)
+            self.cache = CacheManager([GroupSpec(4, 32)], 3)
+            self.model, self.device, self.max_rows, self.steps = FakeModel, torch.device("cpu"), 3, []
+
+        def step(self, entries):
+            self.steps.append([(e.req_id, len(e.tokens), e.start) for e in entries])
+            rows = [(e.start + len(e.tokens)) % 50 for e in entries for _ in e.want]
+            return torch.nn.functional.one_hot(torch.tensor(rows, dtype=torch.long), 50).float()
+
+    class FakeSampler:
+        def sample(self, logits, rows):
+            return logits.argmax(-1).tolist()
+
+    eng = Engine(runner=FakeRunner())
+    eng.sampler = FakeSampler()
+    outs = eng.generate([list(range(10)), list(range(30)), [1, 2]], SamplingParams(max_tokens=3, temperature=0.0))
+    assert outs == [[10, 11, 12], [30, 31, 32], [2, 3, 4]]
+    assert eng.runner.steps[0] == [(0, 10, 0), (1, 6, 0)]                   # budget 16: the second prompt is cut
+    assert eng.runner.steps[1] == [(0, 1, 10), (1, 16, 6)]                  # the decode row is exempt: the prompt gets all 16
+    assert eng.runner.cache.num_free() == 32 and not eng.has_unfinished()
+    outs = eng.generate([[5] * 47], SamplingParams(max_tokens=10, temperature=0.0))
+    assert outs == [[47, 48, 49]]                                           # 49 is eos

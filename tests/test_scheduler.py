@@ -1,0 +1,200 @@
+"""The scheduler's decisions (no GPU), driven step by step with made-up sampled tokens. The vectors
+are the ones the reference's own tests hold (crates/core/src/sched/mod.rs:830-1442)."""
+from dinfer_amd.cache import CacheManager, GroupSpec
+from dinfer_amd.config import EngineOptions
+from dinfer_amd.engine.request import LENGTH, PREEMPTED, STOP, Request
+from dinfer_amd.engine.scheduler import Scheduler
+from dinfer_amd.sampling import SamplingParams
+
+
+def mk(max_seqs, budget, blocks, **kw):
+    opt = EngineOptions(max_num_seqs=max_seqs, max_num_batched_tokens=budget, block_size=16, max_model_len=4096,
+                        num_blocks=blocks, decode_exempt_from_budget=False, **kw)
+    cache = CacheManager([GroupSpec(16, blocks)], max_seqs)
+    return Scheduler(opt, cache, eos_token_ids=[2])
+
+
+def req(i, prompt, max_tokens, **kw):
+    base = 100 + i * 10_000
+    return Request(i, list(range(base, base + prompt)), SamplingParams(max_tokens=max_tokens, **kw))
+
+
+def step(s, toks):
+    """One schedule + update; toks: {id: sampled token} for the requests expected to sample."""
+    out = s.schedule()
+    assert {x.request.id for x in out.scheduled if x.samples} == set(toks)
+    res = s.update(out, toks)
+    s.cache.check()
+    return [(x.request.id, x.num_new) for x in out.scheduled], out, res
+
+
+def test_prefill_then_decode_then_finish_by_eos():
+    s = mk(8, 64, 32)
+    s.add_request(req(1, 10, 100))
+    assert step(s, {1: 7})[0] == [(1, 10)]
+    free = s.cache.num_free()
+    assert step(s, {1: 8})[0] == [(1, 1)]
+    assert s.cache.num_free() == free               # a decode inside the last page takes no page
+    sched, _, res = step(s, {1: 2})
+    assert res[0][1:] == (2, STOP) and not s.has_unfinished() and s.cache.num_free() == 32
+
+
+def test_chunked_prefill_splits_by_budget():
+    s = mk(8, 32, 64)
+    s.add_request(req(1, 70, 4))
+    assert step(s, {})[0] == [(1, 32)]
+    assert step(s, {})[0] == [(1, 32)]
+    assert step(s, {1: 9})[0] == [(1, 6)]           # the last portion samples
+    assert step(s, {1: 9})[0] == [(1, 1)]
+
+
+def test_fcfs_second_request_waits_for_budget_then_runs_alongside():
+    s = mk(8, 40, 64)
+    s.add_request(req(1, 30, 10))
+    s.add_request(req(2, 30, 10))
+    assert step(s, {1: 1})[0] == [(1, 30), (2, 10)]
+    assert step(s, {1: 1, 2: 1})[0] == [(1, 1), (2, 20)]
+    assert step(s, {1: 1, 2: 1})[0] == [(1, 1), (2, 1)]
+
+
+def test_preempts_last_running_when_out_of_blocks_and_replays_everything():
+    s = mk(8, 1000, 4)                               # 4 pages = 64 tokens: two 32-token prompts fill it
+    s.add_request(req(1, 32, 2))
+    r2 = req(2, 32, 100)
+    s.add_request(r2)
+    assert len(step(s, {1: 1, 2: 1})[0]) == 2
+    sched, out, _ = step(s, {1: 1})                  # both need a third page: 1 gets it, 2 is preempted
+    assert sched == [(1, 1)] and out.preempted == [2]
+    assert r2.status == PREEMPTED and r2.num_computed == 0 and list(s.waiting) == [r2]
+    assert 1 not in s.requests                       # request 1 reached max_tokens and freed its pages
+    assert step(s, {2: 5})[0] == [(2, 33)]           # replays the prompt and its one output
+    assert r2.output_ids == [1, 5]
+
+
+def test_step_that_preempted_admits_nobody():
+    s = mk(8, 1000, 4)
+    s.add_request(req(1, 32, 100))
+    s.add_request(req(2, 32, 100))
+    step(s, {1: 1, 2: 1})
+    s.add_request(req(3, 4, 100))
+    sched, out, _ = step(s, {1: 1})
+    assert sched == [(1, 1)] and out.preempted == [2] and [r.id for r in s.waiting] == [2, 3]
+
+
+def test_decode_exempt_from_budget_coschedules_decode_and_prefill():
+    s = mk(4, 8, 64)
+    s.opt.decode_exempt_from_budget = True
+    s.add_request(req(1, 4, 16))
+    assert step(s, {1: 1})[0] == [(1, 4)]
+    s.add_request(req(2, 20, 16))
+    assert step(s, {1: 1})[0] == [(1, 1), (2, 8)]    # the decode row is free, the prompt gets all 8
+    s2 = mk(4, 8, 64)
+    s2.add_request(req(1, 4, 16))
+    step(s2, {1: 1})
+    s2.add_request(req(2, 20, 16))
+    assert step(s2, {1: 1})[0] == [(1, 1), (2, 7)]   # charged: only 7 are left
+
+
+def test_sole_request_that_cannot_grow_is_finished_with_length():
+    s = mk(8, 1000, 4)
+    r = req(1, 48, 100)
+    s.add_request(r)
+    assert step(s, {1: 1})[0] == [(1, 48)]
+    forced = []
+    for _ in range(40):
+        out = s.schedule()
+        forced += out.force_finished
+        if not out.scheduled:
+            break
+        s.update(out, {1: 1})
+    assert forced == [(1, LENGTH)] and r.finish_reason == LENGTH and r.num_computed == 64  # 4 pages full
+    assert s.cache.num_free() == 4 and not s.has_unfinished()
+
+
+def test_tail_request_with_others_present_is_skipped_not_finished():
+    s = mk(8, 1000, 6)                               # 6 pages: two 48-token prompts fill them
+    s.add_request(req(1, 48, 2))
+    r2 = req(2, 48, 100)
+    s.add_request(r2)
+    assert len(step(s, {1: 1, 2: 1})[0]) == 2
+    sched, out, _ = step(s, {1: 1})
+    assert sched == [(1, 1)] and r2.status == PREEMPTED and not out.force_finished
+    sched, out, _ = step(s, {2: 1})                  # request 1 is done; 2 comes back and recomputes
+    assert sched[0][0] == 2 and not out.force_finished
+
+
+def test_waiting_request_without_pages_waits():
+    s = mk(8, 1000, 3)
+    s.add_request(req(1, 40, 100))
+    s.add_request(req(2, 20, 100))
+    assert step(s, {1: 1})[0] == [(1, 40)]           # 3 pages taken; request 2 needs 2
+    assert [r.id for r in s.waiting] == [2]
+    assert step(s, {1: 1})[0] == [(1, 1)]
+    s.abort(1)
+    assert step(s, {2: 1})[0] == [(2, 20)]
+
+
+def test_finish_reasons():
+    s = mk(8, 1000, 32)
+    s.add_request(req(1, 4, 2))
+    step(s, {1: 5})
+    assert step(s, {1: 6})[2][0][2] == LENGTH        # max_tokens (mod.rs:1188-1195)
+    s.add_request(req(2, 4, 10, ignore_eos=True))
+    assert step(s, {2: 2})[2][0][2] is None          # eos ignored
+    s.add_request(req(3, 4, 10, stop_token_ids=[77]))
+    res = step(s, {2: 2, 3: 77})[2]
+    assert dict((r.id, why) for r, _, why in res) == {2: None, 3: STOP}
+    s.add_request(req(4, 4, 10, min_tokens=3))
+    assert step(s, {2: 9, 4: 2})[2][-1][2] is None   # eos before min_tokens does not stop
+    step(s, {2: 9, 4: 2})
+    assert step(s, {2: 9, 4: 2})[2][-1][2] == STOP
+
+
+def test_max_model_len_finishes_with_length():
+    s = mk(8, 1000, 32)
+    s.opt.max_model_len = 8
+    s.add_request(req(1, 6, 100))
+    step(s, {1: 5})
+    assert step(s, {1: 5})[2][0][2] == LENGTH        # 8 tokens reached
+    import pytest
+    with pytest.raises(ValueError, match="max_model_len"):
+        s.add_request(req(2, 8, 1))
+
+
+def test_per_request_and_per_step_prompt_caps():
+    s = mk(8, 1000, 64, long_prefill_token_threshold=8)
+    s.add_request(req(1, 30, 4))
+    assert step(s, {1: 1})[0] == [(1, 30)]           # alone: the cap does not apply (mod.rs:343-346)
+    s.add_request(req(2, 30, 4))
+    s.add_request(req(3, 30, 4))
+    assert step(s, {1: 1})[0] == [(1, 1), (2, 8), (3, 8)]
+    s = mk(8, 1000, 64, prefill_tokens_per_step=10)
+    s.add_request(req(1, 6, 4))
+    s.add_request(req(2, 30, 4))
+    assert step(s, {1: 1})[0] == [(1, 6), (2, 4)]    # 10 prompt tokens per step over all requests
+    assert step(s, {1: 1})[0] == [(1, 1), (2, 10)]   # decode rows are outside the quota
+
+
+def test_max_num_seqs_limits_admission():
+    s = mk(2, 1000, 64)
+    for i in (1, 2, 3):
+        s.add_request(req(i, 4, 1))
+    assert [i for i, _ in step(s, {1: 1, 2: 1})[0]] == [1, 2]
+    assert step(s, {3: 1})[0] == [(3, 4)]
+
+
+def test_schedule_and_update_are_cheap_for_many_decode_rows():
+    """The reference gates 1024 decode requests at 200 us in Rust (crates/core/benches/scheduler.rs);
+    this host code is Python, so the gate here only guards against quadratic behaviour."""
+    import time
+    n = 256
+    s = mk(n, 100000, n * 4)
+    for i in range(n):
+        s.add_request(req(i, 17, 1000))
+    out = s.schedule()
+    s.update(out, {i: 1 for i in range(n)})
+    t0 = time.perf_counter()
+    for _ in range(10):
+        out = s.schedule()
+        s.update(out, {i: 1 for i in range(n)})
+    assert (time.perf_counter() - t0) / 10 < 0.02
