@@ -57,6 +57,7 @@ def write_random_model(config, out_dir: str | Path, seed: int = 0, dtype: str = 
     expected, _optional = expected_tensors(spec)
     tensors = {name: draw(seed, name, ts, tdt) for name, ts in expected.items()}
     cfg = config.to_dict()
+    cfg.setdefault("architectures", [config.ARCHITECTURE])  # the key the registry chooses the model by
     cfg["torch_dtype"] = dtype
     (out / "config.json").write_text(json.dumps(cfg, indent=2))
     write_safetensors(out / "model.safetensors", tensors, metadata={"format": "pt", "seed": seed})

@@ -1,0 +1,160 @@
+"""Generation through the Python entry point: greedy against the plain implementation, the workloads
+BASELINE names for the tiny configurations, sampling rules through the whole engine, preemption."""
+import random
+
+import pytest
+import torch
+
+import plain_qwen3 as plain
+from tiny_configs import CONFIGS, PAGE
+
+pytestmark = pytest.mark.gpu
+
+
+def engine(model_dir, name, dtype="float32", **kw):
+    from dinfer_amd import Engine
+    opts = dict(dtype=dtype, max_model_len=CONFIGS[name][0]["max_position_embeddings"], max_num_seqs=4,
+                max_num_batched_tokens=64, block_size=PAGE[name], num_blocks=128)
+    opts.update(kw)
+    return Engine(str(model_dir), **opts)
+
+
+def prompts_for(name, lens, seed):
+    rng = random.Random(seed)
+    V = CONFIGS[name][0]["vocab_size"]
+    return [[rng.randrange(V) for _ in range(n)] for n in lens]
+
+
+def plain_greedy(cfg, w, prompt, n):
+    """(tokens, margins): greedy continuation by the plain model, with the gap between the two best logits."""
+    ids, margins = list(prompt), []
+    for _ in range(n):
+        row = plain.forward(cfg, w, ids)[-1]
+        top = row.topk(2).values
+        margins.append(float(top[0] - top[1]))
+        ids.append(int(row.argmax()))
+    return ids[len(prompt):], margins
+
+
+@pytest.mark.parametrize("name,lens", [("A", [5, 17, 33]), ("B", [1, 9, 40, 70]), ("C", [3, 50])])
+def test_greedy_generation_equals_plain(model_dirs, name, lens):
+    """Tiny A's workload (3 prompts of 5/17/33, 8 greedy tokens) and its like on B and C, in 32-bit,
+    with a budget that cuts prompts into portions beside decoding requests."""
+    from dinfer_amd import SamplingParams
+    cfg, w = plain.load(model_dirs[name])
+    prompts = prompts_for(name, lens, 7)
+    eng = engine(model_dirs[name], name, max_num_batched_tokens=16)
+    got = eng.generate(prompts, SamplingParams(max_tokens=8, temperature=0.0, ignore_eos=True))
+    for p, g in zip(prompts, got):
+        want, margins = plain_greedy(cfg, w, p, 8)
+        for i, (a, b, m) in enumerate(zip(g, want, margins)):
+            assert a == b or m < 1e-4, f"{name}: prompt of {len(p)}, token {i}: {a} != {b} (margin {m})"
+            if a != b:
+                break
+    assert eng.runner.cache.num_free(0) == 128
+    eng.runner.cache.check()
+
+
+def test_bfloat16_generation_follows_plain_until_a_near_tie(model_dirs):
+    from dinfer_amd import SamplingParams
+    name = "B"
+    cfg, w = plain.load(model_dirs[name])
+    prompts = prompts_for(name, [9, 40], 8)
+    got = engine(model_dirs[name], name, dtype="bfloat16").generate(
+        prompts, SamplingParams(max_tokens=8, temperature=0.0, ignore_eos=True))
+    agree = 0
+    for p, g in zip(prompts, got):
+        want, margins = plain_greedy(cfg, w, p, 8)
+        for a, b, m in zip(g, want, margins):
+            if a != b:
+                assert m < 0.05, f"bf16 chose {a}, plain {b}, margin {m}"
+                break
+            agree += 1
+    assert agree >= 8
+
+
+def test_temperature_sampling_with_seed_in_mixed_batches(model_dirs):
+    """Tiny B's workload: prompts of 1/9/40/70 prefilled in portions of 16 beside decoding requests,
+    12 tokens each at temperature 0.7 with a fixed seed. Every sampled token must be the one the plain
+    rule picks from the plain model's logits for (seed, number of outputs so far); and the same
+    request gives the same tokens alone as in the batch."""
+    from dinfer_amd import SamplingParams
+    name = "B"
+    cfg, w = plain.load(model_dirs[name])
+    prompts = prompts_for(name, [1, 9, 40, 70], 9)
+    sps = [SamplingParams(max_tokens=12, temperature=0.7, seed=1000 + i, ignore_eos=True) for i in range(4)]
+    eng = engine(model_dirs[name], name, max_num_batched_tokens=16)
+    got = eng.generate(prompts, sps)
+    judged = 0
+    for p, g, sp in zip(prompts, got, sps):
+        ids = list(p)
+        for i, tok in enumerate(g):
+            row = plain.forward(cfg, w, ids)[-1]
+            want, slack = plain.sample_row(row, 0.7, sp.seed, i)
+            if slack > 2e-5:   # 32-bit logits and sums: anything nearer to an interval's edge may fall either way
+                judged += 1
+                assert tok == want, f"prompt {len(p)}, output {i}: engine {tok}, rule {want}"
+            ids.append(tok)
+    assert judged >= 44
+    alone = engine(model_dirs[name], name).generate([prompts[2]], sps[2])
+    assert alone[0] == got[2]
+
+
+def test_stop_rules_through_the_engine(model_dirs):
+    from dinfer_amd import SamplingParams
+    name = "A"
+    cfg, w = plain.load(model_dirs[name])
+    p = prompts_for(name, [12], 3)[0]
+    want, _ = plain_greedy(cfg, w, p, 8)
+    eng = engine(model_dirs[name], name)
+    stop = want[3]
+    got = eng.generate([p], SamplingParams(max_tokens=8, temperature=0.0, stop_token_ids=[stop], ignore_eos=True))[0]
+    assert got == want[:want.index(stop) + 1]          # ends with the first occurrence of the stop id
+    assert eng.generate([p], SamplingParams(max_tokens=3, temperature=0.0, ignore_eos=True))[0] == want[:3]
+    with pytest.raises(ValueError, match="vocabulary"):
+        eng.add_request([5, 999], SamplingParams())
+    with pytest.raises(ValueError, match="top_p"):
+        eng.add_request([5], SamplingParams(top_p=0.0))
+
+
+def test_preemption_recomputes_and_gives_the_same_tokens(model_dirs):
+    """A pool too small for all requests: the last running one is preempted, later recomputes its prompt
+    and outputs, and still produces the tokens it would have produced alone."""
+    from dinfer_amd import SamplingParams
+    name = "B"
+    prompts = prompts_for(name, [30, 30, 30], 5)
+    sp = SamplingParams(max_tokens=20, temperature=0.0, ignore_eos=True)
+    roomy = engine(model_dirs[name], name).generate(prompts, sp)
+    tight = engine(model_dirs[name], name, num_blocks=15, max_model_len=64)   # 15 pages of 8: 120 tokens for 150
+    got = tight.generate(prompts, sp)
+    assert got == roomy
+    assert tight.runner.cache.num_free(0) == 15
+    tight.runner.cache.check()
+
+
+def test_penalties_and_truncation_through_the_engine(model_dirs):
+    from dinfer_amd import SamplingParams
+    name = "A"
+    cfg, w = plain.load(model_dirs[name])
+    p = prompts_for(name, [10], 4)[0]
+    eng = engine(model_dirs[name], name)
+    sp = SamplingParams(max_tokens=6, temperature=0.0, repetition_penalty=1.8, frequency_penalty=0.7, presence_penalty=0.4,
+                        ignore_eos=True)
+    got = eng.generate([p], sp)[0]
+    ids, out = list(p), []
+    for _ in range(6):
+        row = plain.apply_penalties(plain.forward(cfg, w, ids)[-1], p, out, 1.8, 0.7, 0.4)
+        top = row.topk(2).values
+        tok = int(row.argmax())
+        if float(top[0] - top[1]) < 1e-4:
+            break
+        out.append(tok)
+        ids.append(tok)
+    assert got[:len(out)] == out and len(out) >= 3
+    sp = SamplingParams(max_tokens=30, temperature=1.5, top_k=3, seed=5, ignore_eos=True)
+    got = eng.generate([p], sp)[0]
+    ids = list(p)
+    for tok in got:
+        row = plain.forward(cfg, w, ids)[-1]
+        assert tok in row.topk(4).indices.tolist()         # top-3, with one more allowed at a rounding edge
+        ids.append(tok)

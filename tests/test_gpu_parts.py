@@ -1,0 +1,288 @@
+"""Each part alone against the plain functions, built from parameters only (no model around it);
+and a toy mixer with state of its own, defined here, registered, built and stepped through the
+engine without a change to the framework's files."""
+import random
+from dataclasses import dataclass
+
+import pytest
+import torch
+
+import plain_qwen3 as plain
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda", 0)
+
+
+def context(dtype=torch.float32, page=8, max_tokens=64):
+    from dinfer_amd.parts import BuildContext
+    return BuildContext(DEV, dtype, max_tokens, max_tokens, page, max_reqs=4)
+
+
+def whole_batch(n_tokens_per_req, page=8, groups=1):
+    """A batch of whole prompts starting at position 0, with pages from a real cache manager."""
+    from dinfer_amd.cache import CacheManager, GroupSpec
+    from dinfer_amd.engine.batch import Entry, StepBatch
+    cache = CacheManager([GroupSpec(page, 64)] * groups, 4)
+    entries = []
+    for i, n in enumerate(n_tokens_per_req):
+        cache.admit(i)
+        cache.allocate(i, 0, n)
+        entries.append(Entry(i, [0] * n, 0, []))
+    b = StepBatch(DEV, 64, 4, 64, [16] * groups)
+    b.fill(entries, cache)
+    b.upload()
+    return b
+
+
+def loader(tensors, dtype):
+    return lambda name, compute=False: tensors[name].to(DEV).to(dtype)
+
+
+def tol(dtype):
+    return dict(rtol=3e-2, atol=3e-2) if dtype == torch.bfloat16 else dict(rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_part(dtype):
+    from dinfer_amd.parts import NORMS
+    n = NORMS.get("rmsnorm")(width=80, eps=3e-6)
+    assert n.tensors()["weight"].shape == (80,)
+    w = torch.rand(80) + 0.5
+    n.load(loader({"weight": w}, dtype))
+    x = torch.randn(7, 80, device=DEV).to(dtype)
+    out = torch.empty_like(x)
+    n.forward(x, out, 7)
+    torch.testing.assert_close(out.double().cpu(), plain.rms_norm(x.double().cpu(), w.to(dtype).double(), 3e-6), **tol(dtype))
+
+
+def test_position_part_builds_the_table_from_its_parameters():
+    from dinfer_amd.parts import POSITION_ENCODINGS
+    pe = POSITION_ENCODINGS.get("rotary")(head_dim=48, theta=5e4, max_positions=100, rotary_dim=32)
+    pe.bind(context())
+    t = pe.table().cpu().double()
+    assert t.shape == (100, 32) and pe.rotary_dim == 32 and pe.style == 0
+    ang = plain.rope_angles(list(range(100)), 32, 5e4)
+    torch.testing.assert_close(t, torch.cat([ang.cos(), ang.sin()], 1), rtol=0, atol=1e-6)
+    assert POSITION_ENCODINGS.get("none")(head_dim=48).table() is None
+    with pytest.raises(ValueError):
+        POSITION_ENCODINGS.get("rotary")(head_dim=48, theta=1e4, max_positions=10, rotary_dim=50)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_feed_forward_part(dtype):
+    from dinfer_amd.parts import FEED_FORWARDS
+    ff = FEED_FORWARDS.get("gated_mlp")(hidden=80, intermediate=136)
+    w = {"gate_proj.weight": torch.randn(136, 80) * 0.1, "up_proj.weight": torch.randn(136, 80) * 0.1,
+         "down_proj.weight": torch.randn(80, 136) * 0.1}
+    assert {k: v.shape for k, v in ff.tensors().items()} == {k: tuple(v.shape) for k, v in w.items()}
+    ff.load(loader(w, dtype))
+    ff.bind(context(dtype))
+    b = whole_batch([11])
+    x = torch.randn(64, 80, device=DEV).to(dtype)
+    out = ff.forward(x, b)[:11]
+    wd = {k: v.to(dtype).double() for k, v in w.items()}
+    want = plain.swiglu_mlp(x[:11].double().cpu(), wd["gate_proj.weight"], wd["up_proj.weight"], wd["down_proj.weight"])
+    torch.testing.assert_close(out.double().cpu(), want, **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [None, 5])
+def test_attention_part(dtype, window):
+    """The mixer alone: projections, per-head norm, rotation, cache write, attention, output projection;
+    two requests in one batch; sizes and constants only from its parameters."""
+    from dinfer_amd.parts import MIXERS, CacheView, part
+    H, Hkv, D, Hd, page, theta, eps = 6, 2, 32, 40, 8, 3e4, 2e-5
+    mx = MIXERS.get("attention")(hidden=Hd, heads=H, kv_heads=Hkv, head_dim=D, window=window,
+                                 position=part("rotary", theta=theta, max_positions=64),
+                                 qk_norm=part("rmsnorm", eps=eps))
+    spec = mx.cache_spec()
+    assert (spec.kv_heads, spec.head_dim, spec.window) == (Hkv, D, window)
+    w = {"q_proj.weight": torch.randn(H * D, Hd) * 0.2, "k_proj.weight": torch.randn(Hkv * D, Hd) * 0.2,
+         "v_proj.weight": torch.randn(Hkv * D, Hd) * 0.2, "o_proj.weight": torch.randn(Hd, H * D) * 0.2,
+         "q_norm.weight": torch.rand(D) + 0.5, "k_norm.weight": torch.rand(D) + 0.5}
+    assert {k: v.shape for k, v in mx.tensors().items()} == {k: tuple(v.shape) for k, v in w.items()}
+    mx.load(loader(w, dtype))
+    mx.bind(context(dtype, page=page))
+    lens = [13, 9]
+    b = whole_batch(lens, page=page)
+    kc = torch.zeros(64, Hkv, page, D, device=DEV, dtype=dtype)
+    vc = torch.zeros(64, Hkv, D, page, device=DEV, dtype=dtype)
+    x = torch.randn(64, Hd, device=DEV).to(dtype)
+    out = mx.forward(x, b, CacheView(0, kc, vc, owner=True))[:sum(lens)].double().cpu()
+    cfg = dict(num_attention_heads=H, num_key_value_heads=Hkv, head_dim=D, rms_norm_eps=eps, rope_theta=theta)
+    wd = {"p." + k: v.to(dtype).double() for k, v in w.items()}
+    t0 = 0
+    for n in lens:
+        want = plain.attention_block(x[t0:t0 + n].double().cpu(), list(range(n)), wd, "p.", cfg, window)
+        torch.testing.assert_close(out[t0:t0 + n], want, **tol(dtype))
+        t0 += n
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_block_part(dtype):
+    """The pre-norm arrangement with the deferred residual adds equals the plain layer."""
+    from dinfer_amd.parts import BLOCKS, CacheView, LayerSpec, part
+    Hd, H, Hkv, D, I, page = 48, 3, 1, 16, 56, 8
+    cfg = dict(num_attention_heads=H, num_key_value_heads=Hkv, head_dim=D, rms_norm_eps=1e-5, rope_theta=1e4,
+               use_sliding_window=False)
+    layer = LayerSpec(block=part("prenorm"), norm=part("rmsnorm", eps=1e-5), prefix="model.layers.0.",
+                      mixer=part("attention", heads=H, kv_heads=Hkv, head_dim=D, qk_norm=part("rmsnorm", eps=1e-5),
+                                 position=part("rotary", theta=1e4, max_positions=64)),
+                      feed_forward=part("gated_mlp", intermediate=I))
+    blk = BLOCKS.get("prenorm")(hidden=Hd, layer=layer)
+    g = torch.Generator().manual_seed(1)
+    w = {n: (torch.rand(s.shape, generator=g) + 0.5) if s.init == "gain" else torch.randn(s.shape, generator=g) * 0.2
+         for n, s in blk.tensors().items()}
+    blk.load(loader(w, dtype))
+    blk.bind(context(dtype, page=page))
+    n = 10
+    b = whole_batch([n], page=page)
+    kc = torch.zeros(64, Hkv, page, D, device=DEV, dtype=dtype)
+    vc = torch.zeros(64, Hkv, D, page, device=DEV, dtype=dtype)
+    h0 = torch.randn(64, Hd, device=DEV).to(dtype)
+    prev = torch.randn(64, Hd, device=DEV).to(dtype)       # the previous layer's branch, not yet added
+    hidden = h0.clone()
+    pending = blk.forward(hidden, prev, b, CacheView(0, kc, vc, owner=True))
+    got = (hidden[:n].double() + pending[:n].double()).cpu()
+    wd = {"model.layers.0." + k: v.to(dtype).double() for k, v in w.items()}
+    want = plain.decoder_layer((h0[:n].double() + prev[:n].double()).cpu(), list(range(n)), wd, 0, cfg)
+    if dtype == torch.float32:
+        torch.testing.assert_close(got, want, **tol(dtype))
+    else:
+        # a whole layer chains a dozen bf16 roundings: judge the error against the spread of the output
+        assert float((got - want).abs().max() / want.std()) < 0.03
+
+
+# ---- a toy mixer with state of its own ----------------------------------------------------------------
+def register_toy():
+    from dinfer_amd.config import ModelConfig, key, register_architecture
+    from dinfer_amd.parts import MIXERS, LayerSpec, Mixer, ModelSpec, RunEntry, StateSpec, TensorSpec, part
+
+    class DecayMixer(Mixer):
+        """s_t = decay * s_{t-1} + x_t (per request, float32 state in its slot); y_t = s_t W^T."""
+
+        def __init__(self, hidden, decay):
+            self.hidden, self.decay = hidden, decay
+
+        def cache_spec(self):
+            return StateSpec((self.hidden,), "float32")
+
+        def tensors(self):
+            return {"mix.weight": TensorSpec((self.hidden, self.hidden))}
+
+        def load(self, get):
+            self.w = get("mix.weight", compute=True)
+
+        def bind(self, ctx):
+            self.out = ctx.workspace.buffer("toy_out", self.hidden)
+
+        def forward(self, x, batch, cache):
+            slots = batch.state_slots[:batch.num_reqs].tolist()
+            t = 0
+            for slot, n in zip(slots, batch.q_lens):
+                s = cache.state[slot]
+                for i in range(n):
+                    s.mul_(self.decay).add_(x[t + i].float())
+                    self.out[t + i] = (s @ self.w.float().T).to(self.out.dtype)
+                t += n
+            return self.out
+
+    @dataclass(frozen=True)
+    class ToyConfig(ModelConfig):
+        vocab_size: int = key(int)
+        hidden_size: int = key(int)
+        decay: float = key(float)
+        ARCHITECTURE = "ToyStateLM"
+
+    def build_spec(c):
+        norm = part("rmsnorm", eps=1e-6)
+        ff = part("gated_mlp", intermediate=2 * c.hidden_size)
+        attn = part("attention", heads=2, kv_heads=1, head_dim=16, position=part("rotary", theta=1e4, max_positions=256))
+        layers = [LayerSpec(part("prenorm", mixer_prefix="toy."), part("toy_decay", decay=c.decay), ff, norm, "layers.0."),
+                  LayerSpec(part("prenorm"), attn, ff, norm, "layers.1.")]
+        # the stateful layer runs twice (shared weights, a state of its own each time), around the attention layer
+        return ModelSpec("ToyStateLM", c.vocab_size, c.hidden_size, 256, layers, [RunEntry(0), RunEntry(1), RunEntry(0)],
+                         norm, "norm.", "embed.weight", "head.weight", tie_embeddings=True)
+
+    if "toy_decay" not in MIXERS:
+        MIXERS.register("toy_decay", DecayMixer)
+    register_architecture("ToyStateLM", ToyConfig, build_spec)
+    return ToyConfig
+
+
+def toy_plain(w, ids, decay, dtype):
+    """The toy model for one whole sequence, straight torch in float64."""
+    Hd = w["embed.weight"].shape[1]
+    W = {k: v.double() for k, v in w.items()}
+    h = W["embed.weight"][ids]
+
+    def ffn(p, x):
+        return plain.swiglu_mlp(x, W[p + "mlp.gate_proj.weight"], W[p + "mlp.up_proj.weight"], W[p + "mlp.down_proj.weight"])
+
+    def toy_layer(h):
+        p = "layers.0."
+        x = plain.rms_norm(h, W[p + "input_layernorm.weight"], 1e-6)
+        s, ys = torch.zeros(Hd, dtype=torch.float64), []
+        for t in range(len(ids)):
+            s = decay * s + x[t]
+            ys.append(s @ W[p + "toy.mix.weight"].T)
+        h = h + torch.stack(ys)
+        return h + ffn(p, plain.rms_norm(h, W[p + "post_attention_layernorm.weight"], 1e-6))
+
+    def attn_layer(h):
+        p = "layers.1."
+        x = plain.rms_norm(h, W[p + "input_layernorm.weight"], 1e-6)
+        T = len(ids)
+        q = (x @ W[p + "self_attn.q_proj.weight"].T).view(T, 2, 16)
+        k = (x @ W[p + "self_attn.k_proj.weight"].T).view(T, 1, 16)
+        v = (x @ W[p + "self_attn.v_proj.weight"].T).view(T, 1, 16)
+        ang = plain.rope_angles(list(range(T)), 16, 1e4)
+        o = plain.causal_attention(plain.rope_neox(q, ang), plain.rope_neox(k, ang), v, 16 ** -0.5)
+        h = h + o.reshape(T, 32) @ W[p + "self_attn.o_proj.weight"].T
+        return h + ffn(p, plain.rms_norm(h, W[p + "post_attention_layernorm.weight"], 1e-6))
+
+    h = toy_layer(attn_layer(toy_layer(h)))
+    return plain.rms_norm(h, W["norm.weight"], 1e-6) @ W["embed.weight"].T
+
+
+def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
+    from safetensors.torch import load_file
+    from dinfer_amd.config import EngineOptions, unregister_architecture
+    from dinfer_amd.engine.batch import Entry
+    from dinfer_amd.engine.runner import ModelRunner
+    from dinfer_amd.parts import MIXERS
+    from dinfer_amd.weights import write_random_model
+    ToyConfig = register_toy()
+    try:
+        cfg = ToyConfig.from_dict(dict(vocab_size=97, hidden_size=24, decay=0.8, architectures=["ToyStateLM"]))
+        write_random_model(cfg, tmp_path, seed=4, dtype="float32")
+        w = load_file(str(tmp_path / "model.safetensors"))
+        assert "layers.0.toy.mix.weight" in w and "layers.1.self_attn.q_proj.weight" in w
+        opt = EngineOptions(dtype="float32", max_model_len=128, max_num_seqs=3, max_num_batched_tokens=64,
+                            block_size=8, num_blocks=32, max_logits_rows=64, decode_exempt_from_budget=False)
+        r = ModelRunner.from_dir(tmp_path, opt)
+        assert len(r.state_tensors) == 2 and len(r.group_specs) == 1      # two state entries, one page group
+        rng = random.Random(1)
+        seqs = {k: [rng.randrange(97) for _ in range(n)] for k, n in (("a", 21), ("b", 30), ("c", 9), ("d", 14))}
+        want = {k: toy_plain(w, v, 0.8, torch.float64) for k, v in seqs.items()}
+        # a and b interleaved in portions; c afterwards in a's slot (its state must start from zero); d whole
+        plan = [[("a", 5), ("b", 2)], [("b", 11)], [("a", 16), ("b", 1)], [("b", 16), ("c", 9)], [("d", 14)]]
+        fed = {k: 0 for k in seqs}
+        for st in plan:
+            entries = []
+            for k, n in st:
+                assert r.reserve(k, fed[k], n)
+                entries.append(Entry(k, seqs[k][fed[k]:fed[k] + n], fed[k], list(range(n))))
+            logits = r.step(entries).double().cpu()
+            i = 0
+            for e in entries:
+                n = len(e.tokens)
+                torch.testing.assert_close(logits[i:i + n], want[e.req_id][e.start:e.start + n], rtol=1e-4, atol=1e-5)
+                i += n
+                fed[e.req_id] += n
+                if fed[e.req_id] == len(seqs[e.req_id]):
+                    r.finish(e.req_id)
+        r.cache.check()
+    finally:
+        unregister_architecture("ToyStateLM")
+        MIXERS.unregister("toy_decay")
