@@ -7,7 +7,7 @@
 // loads 32 contiguous bytes W[n0 + i][kk + 16 g .. + 16] and feeds them to two
 // MFMAs; the activations are loaded with the same k mapping, so a wave reads
 // 128 contiguous bytes of each of its 16 rows per step, and the waves of a
-// workgroup take adjacent 128-byte pieces of the same rows (split-K inside the
+// workgroup take consecutive runs of k of the same rows (split-K inside the
 // workgroup). Partial sums meet in LDS and are added in wave order, then stored
 // once. No atomics: the result of a given launch shape is reproducible.
 //
@@ -43,22 +43,27 @@ __device__ __forceinline__ void store4<bf16>(bf16* p, f32x4 v) {
 }
 
 
-template <int MT, int RT, class O>
+// GATED (RT == 2): W is [2N, K], rows [0, N) the gate and [N, 2N) the up projection; the workgroup's
+// two row tiles are gate rows n0.. and up rows N + n0.., and the epilogue stores
+// silu(gate) * up into C [M, N]: the activation costs no pass of its own.
+template <int MT, int RT, class O, bool GATED = false>
 __global__ void __launch_bounds__(1024) gemm_small_m_kernel(const bf16* __restrict__ A, int64_t lda,
                                                             const bf16* __restrict__ W, int64_t ldw,
                                                             O* __restrict__ C, int64_t ldc, int M, int N, int K) {
+  static_assert(!GATED || RT == 2, "the gated form pairs one gate tile with one up tile");
   // 64-wide k steps in flight per wave: as many as the register file takes at 16 waves a workgroup
   constexpr int UNROLL = MT <= 2 ? (4 / RT > 0 ? 4 / RT : 1) : (2 / RT > 0 ? 2 / RT : 1);
   extern __shared__ float red[];  // [waves][RT * MT][64 lanes][4]
   const int nw = blockDim.x >> 6;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, i16 = lane & 15, g4 = lane >> 4;
-  const int n0 = blockIdx.x * 16 * RT;
+  const int n0 = GATED ? blockIdx.x * 16 : blockIdx.x * 16 * RT;
 
   const bf16* wp[RT];
 #pragma unroll
   for (int r = 0; r < RT; ++r) {
-    int n = n0 + r * 16 + i16;
+    int n = GATED ? n0 + i16 : n0 + r * 16 + i16;
     if (n >= N) n = N - 1;  // rows past the end are computed and dropped
+    if (GATED && r == 1) n += N;
     wp[r] = W + (int64_t)n * ldw + 16 * g4;
   }
   const bf16* ap[MT];
@@ -75,14 +80,18 @@ __global__ void __launch_bounds__(1024) gemm_small_m_kernel(const bf16* __restri
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[r][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  const int steps = (K + 63) / 64;  // k steps of 64; wave w takes steps w, w + nw, ...
-  for (int s0 = wave; s0 < steps; s0 += nw * UNROLL) {
+  // k steps of 64; wave w takes a contiguous run of them, so its loads walk each row in long pieces
+  const int steps = (K + 63) / 64;
+  const int per_wave = (steps + nw - 1) / nw;
+  const int s_begin = wave * per_wave;
+  const int s_end = s_begin + per_wave < steps ? s_begin + per_wave : steps;
+  for (int s0 = s_begin; s0 < s_end; s0 += UNROLL) {
     bf16x8 wf[UNROLL][RT][2], af[UNROLL][MT][2];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
-      const int kk = (s0 + u * nw) * 64;
+      const int kk = (s0 + u) * 64;
       const int k = kk + 16 * g4;
-      const bool ok0 = k < K && (s0 + u * nw) < steps, ok1 = k + 8 < K && (s0 + u * nw) < steps;
+      const bool ok0 = k < K && (s0 + u) < s_end, ok1 = k + 8 < K && (s0 + u) < s_end;
 #pragma unroll
       for (int r = 0; r < RT; ++r) {
         wf[u][r][0] = ok0 ? *(const bf16x8*)(wp[r] + kk) : zero8();
@@ -113,11 +122,20 @@ __global__ void __launch_bounds__(1024) gemm_small_m_kernel(const bf16* __restri
     for (int t = 0; t < MT; ++t) slot[(r * MT + t) * 64] = acc[r][t];
   __syncthreads();
   // thread x sums slot x of every wave, in wave order; slot = (tile, lane): 4 consecutive n of one token
-  for (int x = threadIdx.x; x < RT * MT * 64; x += blockDim.x) {
+  for (int x = threadIdx.x; x < (GATED ? 1 : RT) * MT * 64; x += blockDim.x) {
     f32x4 s = ((const f32x4*)red)[x];
     for (int w = 1; w < nw; ++w) {
       const f32x4 v = ((const f32x4*)red)[(int64_t)w * RT * MT * 64 + x];
       s[0] += v[0]; s[1] += v[1]; s[2] += v[2]; s[3] += v[3];
+    }
+    if (GATED) {  // slot x of the up tile lies MT * 64 slots further on
+      f32x4 u = ((const f32x4*)red)[MT * 64 + x];
+      for (int w = 1; w < nw; ++w) {
+        const f32x4 v = ((const f32x4*)red)[(int64_t)w * RT * MT * 64 + MT * 64 + x];
+        u[0] += v[0]; u[1] += v[1]; u[2] += v[2]; u[3] += v[3];
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) s[e] = (s[e] / (1.f + expf(-s[e]))) * u[e];
     }
     const int tile = x >> 6, ln = x & 63;
     const int r = tile / MT, t = tile % MT;
@@ -140,6 +158,15 @@ int launch(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, O* C, int64_t
   const int row_tiles = (N + 16 * RT - 1) / (16 * RT);
   const size_t lds = (size_t)waves * RT * MT * 64 * sizeof(f32x4);
   gemm_small_m_kernel<MT, RT, O><<<(unsigned)row_tiles, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
+  return launch_status();
+}
+
+template <int MT>
+int launch_gated(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, bf16* C, int64_t ldc, int M, int N, int K,
+                 int waves, hipStream_t stream) {
+  const int col_tiles = (N + 15) / 16;
+  const size_t lds = (size_t)waves * 2 * MT * 64 * sizeof(f32x4);
+  gemm_small_m_kernel<MT, 2, bf16, true><<<(unsigned)col_tiles, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
   return launch_status();
 }
 
@@ -170,12 +197,12 @@ extern "C" int dinfer_gemm_small_m(int out_f32, const void* A, int64_t lda, cons
     return ERR_BAD_SHAPE;
   const int mt = (int)(M + 15) / 16;
   int rt = row_tiles_per_block, nw = waves;
-  if (rt == 0) rt = mt >= 2 ? 2 : ((N >= 16384 && M > 4) ? 2 : 1);
+  if (rt == 0) rt = mt >= 2 ? 2 : ((N >= 6144 && M > 4) ? 2 : 1);  // measured on MI355X
   if (nw == 0) {
     // about 2048 waves in flight, each with at least two k steps
     const int64_t tiles = (N + 16 * rt - 1) / (16 * rt);
     nw = 4;
-    while (nw < 16 && tiles * nw < 2048) nw *= 2;
+    while (nw < 16 && tiles * nw < (rt == 1 ? 2048 : 768)) nw *= 2;
     const int64_t steps = (K + 63) / 64;
     while (nw > 1 && steps < 2 * nw) nw /= 2;
   }
@@ -187,4 +214,29 @@ extern "C" int dinfer_gemm_small_m(int out_f32, const void* A, int64_t lda, cons
                            stream);
   return dispatch<bf16>((const bf16*)A, lda, (const bf16*)W, ldw, (bf16*)C, ldc, (int)M, (int)N, (int)K, rt, nw,
                         stream);
+}
+
+
+// out[:M] = silu(A . Wg^T) * (A . Wu^T) with W = [Wg; Wu] stacked [2N, K], M <= 32, bf16 in and out:
+// the two projections of a gated feed-forward and its activation in one weight-streaming kernel.
+extern "C" int dinfer_gemm_small_m_gated(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc,
+                                         int64_t M, int64_t N, int64_t K, int waves, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return OK;
+  if (M > 32) return ERR_UNSUPPORTED;
+  if (K <= 0 || K % 8 || lda < K || ldw < K || ldc < N || lda % 8 || ldw % 8 || N > 0x3fffffff || K > 0x7fffffff ||
+      ((uintptr_t)A % 16) || ((uintptr_t)W % 16))
+    return ERR_BAD_SHAPE;
+  const int mt = (int)(M + 15) / 16;
+  int nw = waves;
+  if (nw == 0) {
+    const int64_t tiles = (N + 15) / 16;
+    nw = 4;
+    while (nw < 16 && tiles * nw < 768) nw *= 2;
+    const int64_t steps = (K + 63) / 64;
+    while (nw > 1 && steps < 2 * nw) nw /= 2;
+  }
+  if (nw < 1 || nw > 16 || (size_t)nw * 2 * mt * 64 * sizeof(f32x4) > 64 * 1024) return ERR_BAD_SHAPE;
+  if (mt == 1)
+    return launch_gated<1>((const bf16*)A, lda, (const bf16*)W, ldw, (bf16*)C, ldc, (int)M, (int)N, (int)K, nw, stream);
+  return launch_gated<2>((const bf16*)A, lda, (const bf16*)W, ldw, (bf16*)C, ldc, (int)M, (int)N, (int)K, nw, stream);
 }

@@ -15,6 +15,11 @@ from . import ops
 SMALL_M = 16  # up to this many rows the weight-streaming kernel beats the library (measured on MI355X)
 
 
+def fuses_gated_act(a: torch.Tensor, w: torch.Tensor, m: int, act: str) -> bool:
+    """Whether the gate/up projections and the activation of a gated feed-forward run as one kernel."""
+    return a.dtype == torch.bfloat16 and act == "silu" and 0 < m <= SMALL_M and w.shape[1] % 8 == 0
+
+
 def matmul_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int) -> torch.Tensor:
     """out[:m] = a[:m] @ w.T; out has a's dtype, or float32 (logits)."""
     if m <= 0:

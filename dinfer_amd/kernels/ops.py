@@ -252,6 +252,19 @@ def gemm_small_m(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, *,
     return out
 
 
+def gemm_small_m_gated(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, *, waves: int = 0) -> torch.Tensor:
+    """out[:m] = silu(a @ wg.T) * (a @ wu.T) for w = [wg; wu] stacked [2N, K], m <= 32, bf16: both
+    projections of a gated feed-forward and the activation in one weight-streaming kernel."""
+    _need_gpu(a, w, out)
+    k = w.shape[1]
+    n = w.shape[0] // 2
+    assert w.shape[0] == 2 * n and a.dtype == w.dtype == out.dtype == torch.bfloat16
+    assert a.shape[1] == k and out.shape[1] == n and a.shape[0] >= m and out.shape[0] >= m
+    lib.call("dinfer_gemm_small_m_gated", a.data_ptr(), _rows(a), w.data_ptr(), _rows(w), out.data_ptr(), _rows(out),
+             m, n, k, waves, _stream())
+    return out
+
+
 def argmax(logits: torch.Tensor, out: torch.Tensor, rows: int) -> torch.Tensor:
     _need_gpu(logits, out)
     assert logits.dtype == torch.float32 and out.dtype == torch.int32 and out.numel() >= rows

@@ -4,7 +4,7 @@ from __future__ import annotations
 
 import torch
 
-from ..kernels import ops
+from ..kernels import gemm, ops
 from .base import FeedForward
 from .linear import Linear
 from .registry import FEED_FORWARDS
@@ -38,6 +38,10 @@ class GatedMLP(FeedForward):
 
     def forward(self, x, batch):
         T = batch.num_tokens
-        self.gate_up.forward(x, self.gu_buf, T)
-        ops.gated_act(self.gu_buf, self.act_buf, T, self.act)
+        if gemm.fuses_gated_act(x, self.gate_up.weight, T, self.act):
+            # decode-sized steps: both projections and the activation in one weight-streaming kernel
+            ops.gemm_small_m_gated(x, self.gate_up.weight, self.act_buf, T)
+        else:
+            self.gate_up.forward(x, self.gu_buf, T)
+            ops.gated_act(self.gu_buf, self.act_buf, T, self.act)
         return self.down.forward(self.act_buf, self.out_buf, T)

@@ -408,3 +408,19 @@ def test_gemm_small_m(M, out_dtype):
             ops().gemm_small_m(a, w, out, M, row_tiles=rt, waves=waves)
             t = dict(rtol=2e-2, atol=2e-2) if out_dtype == torch.bfloat16 else dict(rtol=1e-4, atol=1e-4)
             torch.testing.assert_close(out.double(), want, **t, msg=lambda m_: f"M={M} N={N} K={K} rt={rt} waves={waves}: {m_}")
+
+
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 32])
+def test_gemm_small_m_gated(M):
+    """Both projections of a gated feed-forward and silu(gate) * up in one kernel, against float64."""
+    for N, K in ((136, 4096), (1000, 1096), (12288, 512), (20, 8)):
+        a = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+        w = (torch.randn(2 * N, K, device=DEV) * 0.05).to(torch.bfloat16)
+        z = a.double() @ w.double().T
+        want = plain.silu(z[:, :N]) * z[:, N:]
+        for waves in (0, 1, 8):
+            out = torch.full((M, N), float("nan"), device=DEV, dtype=torch.bfloat16)
+            ops().gemm_small_m_gated(a, w, out, M, waves=waves)
+            # one rounding of the result; the operands are exact here, so the sums are exact to float
+            err = (out.double() - want).abs()
+            assert bool((err <= 1e-2 * want.abs() + 1e-3 * want.std()).all()), f"M={M} N={N} K={K}: {float(err.max())}"
