@@ -1,0 +1,70 @@
+"""One layer with the layer sizes of Qwen3-8B, 14B and 32B (group sizes 4, 5 and 8; H * D equal to,
+and larger than, the hidden size), random weights, against the plain implementation in 32-bit and
+in bfloat16: whole prompt, then decoding, then a second request beside it. The vocabulary is cut to
+2048 rows, which is no layer size."""
+import random
+
+import pytest
+import torch
+
+import plain_qwen3 as plain
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = {
+    "8B": dict(hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, intermediate_size=12288),
+    "14B": dict(hidden_size=5120, num_attention_heads=40, num_key_value_heads=8, intermediate_size=17408),
+    "32B": dict(hidden_size=5120, num_attention_heads=64, num_key_value_heads=8, intermediate_size=25600),
+}
+
+
+@pytest.fixture(scope="module")
+def big_models(tmp_path_factory):
+    from dinfer_amd.config.qwen3 import Qwen3Config
+    from dinfer_amd.weights import write_random_model
+    out = {}
+    for name, sizes in SHAPES.items():
+        cfg = dict(architectures=["Qwen3ForCausalLM"], vocab_size=2048, head_dim=128, num_hidden_layers=1,
+                   rms_norm_eps=1e-6, rope_theta=1e6, max_position_embeddings=512, tie_word_embeddings=False, **sizes)
+        d = tmp_path_factory.mktemp(f"big_{name}")
+        write_random_model(Qwen3Config.from_dict(cfg), d, seed=len(name))
+        out[name] = d
+    return out
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(SHAPES))
+def test_layer_sizes_of_the_large_models(big_models, name, dtype):
+    from dinfer_amd.config import EngineOptions
+    from dinfer_amd.engine.batch import Entry
+    from dinfer_amd.engine.runner import ModelRunner
+    cfg, w = plain.load(big_models[name], dtype=torch.float32)
+    opt = EngineOptions(dtype=dtype, max_model_len=512, max_num_seqs=4, max_num_batched_tokens=256, block_size=16,
+                        num_blocks=64, max_logits_rows=256, decode_exempt_from_budget=False)
+    r = ModelRunner.from_dir(big_models[name], opt)
+    rng = random.Random(1)
+    a = [rng.randrange(2048) for _ in range(100)]
+    b = [rng.randrange(2048) for _ in range(37)]
+    want = {"a": plain.forward(cfg, w, a).double(), "b": plain.forward(cfg, w, b).double()}
+    steps = [[("a", a[:90], list(range(90)))]]
+    steps += [[("a", [a[90 + i]], [0])] for i in range(4)]
+    steps += [[("a", a[94:], list(range(6))), ("b", b[:30], list(range(30)))], [("b", b[30:], list(range(7)))]]
+    fed = {"a": 0, "b": 0}
+    for st in steps:
+        entries = []
+        for rid, toks, wants in st:
+            assert r.reserve(rid, fed[rid], len(toks))
+            entries.append(Entry(rid, toks, fed[rid], wants))
+        got = r.step(entries).double().cpu()
+        i = 0
+        for e in entries:
+            ref = want[e.req_id][e.start:e.start + len(e.tokens)]
+            g = got[i:i + len(e.tokens)]
+            if dtype == "float32":
+                # the plain model runs in float32 here (float64 of these sizes is slow): both sides round
+                torch.testing.assert_close(g, ref, rtol=2e-3, atol=2e-4)
+            else:
+                err = ((g - ref).abs() / ref.std(-1, keepdim=True)).max().item()
+                assert err < 0.08, f"{name} {e.req_id}@{e.start}: {err:.3f} row-sigmas"
+            i += len(e.tokens)
+            fed[e.req_id] += len(e.tokens)
