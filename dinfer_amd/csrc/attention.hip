@@ -117,31 +117,39 @@ struct Tile {
     }
   }
 
+  // Loads are unconditional: a key outside [k_lo, k_hi) is replaced by the nearest key inside, which
+  // lies in a page the request holds, so straight-line code with all loads in flight at once. What
+  // was loaded for such a key never counts: its score is masked, and compute() zeroes its value.
   __device__ __forceinline__ void load(Frags<DT>& f, int kb) {
     constexpr int D = DT * 16;
     const int lane = threadIdx.x & 63, i16 = lane & 15, g4 = lane >> 4;
     const int ps = pages.ps;
     pages.ensure(kb);
+    const int last = k_hi - 1;
     // K rows of this lane: keys kg_row + (i16 & 3) and + 4, in one page (page size % 8 == 0)
-    const int kg_row = kb + 8 * (i16 >> 2);
-    const int key0 = kg_row + (i16 & 3), key1 = key0 + 4;
-    const bool v0 = key0 >= k_lo && key0 < k_hi, v1 = key1 >= k_lo && key1 < k_hi;
-    const int pgk = pages.get(pages.page_of(kg_row));
-    const bf16* krow = kc + (((int64_t)pgk * Hkv + hk) * ps + pages.offset_of(kg_row) + (i16 & 3)) * D;
+    int key0 = kb + 8 * (i16 >> 2) + (i16 & 3), key1 = key0 + 4;
+    key0 = key0 < k_lo ? k_lo : (key0 > last ? last : key0);
+    key1 = key1 < k_lo ? k_lo : (key1 > last ? last : key1);
+    const int pg0 = pages.get(pages.page_of(key0)), pg1 = pages.get(pages.page_of(key1));
+    const bf16* kr0 = kc + (((int64_t)pg0 * Hkv + hk) * ps + pages.offset_of(key0)) * D;
+    const bf16* kr1 = kc + (((int64_t)pg1 * Hkv + hk) * ps + pages.offset_of(key1)) * D;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      const int d = ks * 32 + g4 * 8;
+      int d = ks * 32 + g4 * 8;
       const bool dv = d < D;  // D % 32 == 16: the upper half of the last step is padding
-      f.k[0][ks] = (v0 && dv) ? *(const bf16x8*)(krow + d) : zero8();
-      f.k[1][ks] = (v1 && dv) ? *(const bf16x8*)(krow + 4 * D + d) : zero8();
+      if (!dv) d = 0;
+      f.k[0][ks] = *(const bf16x8*)(kr0 + d);
+      f.k[1][ks] = *(const bf16x8*)(kr1 + d);
+      if (DT % 2 == 1 && ks == KS - 1 && !dv) f.k[0][ks] = f.k[1][ks] = zero8();
     }
-    // V^T rows of this lane: d = 16 dt + i16, keys kg .. kg + 7
-    const int kg = kb + 8 * g4;
-    const bool vg = kg < k_hi && kg + 8 > k_lo;
+    // V^T rows of this lane: d = 16 dt + i16, keys kg .. kg + 7 (one page)
+    int kg = kb + 8 * g4;
+    const int g_lo = k_lo & ~7, g_hi = last & ~7;
+    kg = kg < g_lo ? g_lo : (kg > g_hi ? g_hi : kg);
     const int pgv = pages.get(pages.page_of(kg));
     const bf16* vrow = vc + (((int64_t)pgv * Hkv + hk) * D + i16) * ps + pages.offset_of(kg);
 #pragma unroll
-    for (int d = 0; d < DT; ++d) f.v[d] = vg ? *(const bf16x8*)(vrow + (int64_t)d * 16 * ps) : zero8();
+    for (int d = 0; d < DT; ++d) f.v[d] = *(const bf16x8*)(vrow + (int64_t)d * 16 * ps);
   }
 
   __device__ __forceinline__ void compute(const Frags<DT>& f, const bf16x8 (&qf)[NT][KS], int kb,
@@ -209,12 +217,22 @@ struct Tile {
   }
 
   // All key blocks of [k_lo, k_hi); mask(kb) says whether block kb needs per-key masking.
-  template <class MaskFn>
+  // PREFETCH: the next block's loads are issued before the current block is computed (two sets of
+  // fragments in registers); without it one set, and latency is hidden by more waves per SIMD.
+  template <bool PREFETCH, class MaskFn>
   __device__ __forceinline__ void walk(const bf16x8 (&qf)[NT][KS], const int (&col_lo)[NT], const int (&col_hi)[NT],
                                        MaskFn mask) {
-    Frags<DT> f0, f1;
     int kb = k_lo & ~31;
     if (kb >= k_hi) return;
+    if (!PREFETCH) {
+      for (; kb < k_hi; kb += 32) {
+        Frags<DT> f;
+        load(f, kb);
+        compute(f, qf, kb, col_lo, col_hi, mask(kb));
+      }
+      return;
+    }
+    Frags<DT> f0, f1;
     load(f0, kb);
     while (true) {
       const bool more1 = kb + 32 < k_hi;
@@ -238,8 +256,13 @@ struct Tile {
   }
 };
 
+// Measured on MI355X at head size 128 (2,048-token prompt): one set of fragments with two waves per
+// SIMD beats prefetching with one wave (123 us against 132 us a layer), and 32 query rows per wave
+// beat 16 (more waves, 168 us) and 64 (one wave per SIMD, 182 us).
+constexpr bool FLASH_PREFETCH = false;
+
 template <int DT, int QT>
-__global__ void __launch_bounds__(256) attn_flash_kernel(
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) attn_flash_kernel(
     const bf16* __restrict__ q, int64_t ld_q, bf16* __restrict__ out, int64_t ld_out, const bf16* __restrict__ kc,
     const bf16* __restrict__ vc, const int32_t* __restrict__ block_table, int64_t max_blocks,
     const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_lens, int tiles_x, float scale_log2e,
@@ -288,7 +311,7 @@ __global__ void __launch_bounds__(256) attn_flash_kernel(
 
   Tile<DT, QT> tl;
   tl.init(kc, vc, bt, (int)max_blocks, hk, Hkv, ps, k_lo, k_hi, scale_log2e);
-  tl.walk(qf, col_lo, col_hi, [&](int kb) {
+  tl.template walk<FLASH_PREFETCH>(qf, col_lo, col_hi, [&](int kb) {
     return kb + 31 > p_first || kb < k_lo || (window > 0 && kb < p_last - window + 1);
   });
 #pragma unroll
@@ -323,7 +346,7 @@ __device__ __forceinline__ void split_range(int seq, int window, int splits, int
 
 // One wave per (split, kv head, request). part: [B, H, splits, D + 4] float = (m in base-2 units, l, -, -, o[D]).
 template <int DT>
-__global__ void __launch_bounds__(64) attn_decode_kernel(
+__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 8))) attn_decode_kernel(
     const bf16* __restrict__ q, int64_t ld_q, float* __restrict__ part, const bf16* __restrict__ kc,
     const bf16* __restrict__ vc, const int32_t* __restrict__ block_table, int64_t max_blocks,
     const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_lens, int splits, float scale_log2e,
@@ -356,7 +379,7 @@ __global__ void __launch_bounds__(64) attn_decode_kernel(
   const int col_lo[1] = {k_lo}, col_hi[1] = {k_hi};
   Tile<DT, 1> tl;
   tl.init(kc, vc, bt, (int)max_blocks, hk, Hkv, ps, k_lo, k_hi, scale_log2e);
-  tl.walk(qf, col_lo, col_hi, [&](int kb) { return kb < k_lo || kb + 32 > k_hi; });
+  tl.template walk<false>(qf, col_lo, col_hi, [&](int kb) { return kb < k_lo || kb + 32 > k_hi; });
   const float lt = tl.sum_l(0);
   if (i16 < G) {
     float* pp = part + (((int64_t)b * H + hk * G + i16) * splits + sp) * (D + 4);

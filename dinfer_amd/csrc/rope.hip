@@ -105,6 +105,76 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_kernel(
   }
 }
 
+// The common case (pairs (i, i + D/2), the whole head rotated): both elements of a pair live in one
+// lane, so there is no exchange through LDS and no barrier, and every load of a head (values, gains,
+// angles) is issued before the first use. NP pairs per lane cover D <= 128 * NP.
+template <class S, int NP>
+__global__ void __launch_bounds__(WAVES * 64) qkv_post_neox_kernel(
+    S* __restrict__ qkv, int64_t ld, int64_t q_off, int64_t k_off, int64_t v_off, const void* __restrict__ wq,
+    const void* __restrict__ wk, int wf32, float eps, float w_offset, const int32_t* __restrict__ pos,
+    const float* __restrict__ cos_sin, S* __restrict__ k_cache, S* __restrict__ v_cache,
+    const int64_t* __restrict__ slots, int H, int Hkv, int D, int page) {
+  const int64_t t = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int item = blockIdx.y * WAVES + wave;
+  if (item >= H + 2 * Hkv) return;
+  S* row = qkv + t * ld;
+  const int64_t slot = slots ? slots[t] : -1;
+  const int64_t blk = slot >= 0 ? slot / page : 0;
+  const int off = slot >= 0 ? (int)(slot % page) : 0;
+  if (item >= H + Hkv) {
+    if (slot < 0) return;
+    const int hk = item - H - Hkv;
+    const S* vs = row + v_off + (int64_t)hk * D;
+    S* vd = v_cache + ((blk * Hkv + hk) * (int64_t)D) * page + off;
+    for (int d = lane; d < D; d += 64) vd[(int64_t)d * page] = vs[d];
+    return;
+  }
+  const bool is_q = item < H;
+  const int hk = item - H;
+  S* base = is_q ? row + q_off + (int64_t)item * D : row + k_off + (int64_t)hk * D;
+  const void* w = is_q ? wq : wk;
+  const int half = D / 2;
+  const float* cs = cos_sin ? cos_sin + (int64_t)pos[t] * D : nullptr;
+  float x1[NP], x2[NP], g1[NP], g2[NP], c[NP], sn[NP];
+#pragma unroll
+  for (int p = 0; p < NP; ++p) {
+    const int i = lane + 64 * p;
+    const bool ok = i < half;
+    x1[p] = ok ? to_f32(base[i]) : 0.f;
+    x2[p] = ok ? to_f32(base[i + half]) : 0.f;
+    g1[p] = (ok && w) ? ld_param<S>(w, i, wf32) + w_offset : 1.f;
+    g2[p] = (ok && w) ? ld_param<S>(w, i + half, wf32) + w_offset : 1.f;
+    c[p] = (ok && cs) ? cs[i] : 1.f;
+    sn[p] = (ok && cs) ? cs[half + i] : 0.f;
+  }
+  float inv = 1.f;
+  if (w) {
+    float ss = 0.f;
+#pragma unroll
+    for (int p = 0; p < NP; ++p) ss += x1[p] * x1[p] + x2[p] * x2[p];
+    ss = wave_sum(ss);
+    inv = 1.f / sqrtf(ss / (float)D + eps);
+  }
+  S* kd = (!is_q && slot >= 0) ? k_cache + ((blk * Hkv + hk) * (int64_t)page + off) * D : nullptr;
+#pragma unroll
+  for (int p = 0; p < NP; ++p) {
+    const int i = lane + 64 * p;
+    if (i < half) {
+      const float y1 = w ? x1[p] * inv * g1[p] : x1[p], y2 = w ? x2[p] * inv * g2[p] : x2[p];
+      const S r1 = from_f32<S>(y1 * c[p] - y2 * sn[p]), r2 = from_f32<S>(y2 * c[p] + y1 * sn[p]);
+      if (is_q) {
+        base[i] = r1;
+        base[i + half] = r2;
+      }
+      if (kd) {
+        kd[i] = r1;
+        kd[i + half] = r2;
+      }
+    }
+  }
+}
+
 }  // namespace
 
 extern "C" int dinfer_qkv_post(int dtype, void* qkv, int64_t tokens, int64_t ld, int64_t q_off, int64_t k_off,
@@ -120,6 +190,24 @@ extern "C" int dinfer_qkv_post(int dtype, void* qkv, int64_t tokens, int64_t ld,
   if ((q_gain == nullptr) != (k_gain == nullptr)) return ERR_BAD_SHAPE;
   const int items = heads + 2 * kv_heads;
   const dim3 grid((unsigned)tokens, (unsigned)((items + WAVES - 1) / WAVES));
+  const bool whole_head_neox = style == 0 && head_dim % 2 == 0 && (!cos_sin || rotary_dim == head_dim);
+  if (whole_head_neox) {
+    DINFER_DISPATCH_DTYPE(dtype, {
+      if (head_dim <= 128)
+        qkv_post_neox_kernel<S, 1><<<grid, WAVES * 64, 0, stream>>>(
+            (S*)qkv, ld, q_off, k_off, v_off, q_gain, k_gain, w_f32, eps, w_offset, positions, cos_sin, (S*)k_cache,
+            (S*)v_cache, slot_mapping, heads, kv_heads, head_dim, page_size);
+      else if (head_dim <= 256)
+        qkv_post_neox_kernel<S, 2><<<grid, WAVES * 64, 0, stream>>>(
+            (S*)qkv, ld, q_off, k_off, v_off, q_gain, k_gain, w_f32, eps, w_offset, positions, cos_sin, (S*)k_cache,
+            (S*)v_cache, slot_mapping, heads, kv_heads, head_dim, page_size);
+      else
+        qkv_post_neox_kernel<S, 4><<<grid, WAVES * 64, 0, stream>>>(
+            (S*)qkv, ld, q_off, k_off, v_off, q_gain, k_gain, w_f32, eps, w_offset, positions, cos_sin, (S*)k_cache,
+            (S*)v_cache, slot_mapping, heads, kv_heads, head_dim, page_size);
+    });
+    return launch_status();
+  }
   DINFER_DISPATCH_DTYPE(dtype, {
     qkv_post_kernel<S><<<grid, WAVES * 64, 0, stream>>>((S*)qkv, ld, q_off, k_off, v_off, q_gain, k_gain, w_f32, eps,
                                                         w_offset, positions, cos_sin, rotary_dim, style, (S*)k_cache,
