@@ -30,6 +30,13 @@ namespace {
 constexpr int MAX_D = 512;
 constexpr int WAVES = 4;
 
+__device__ __forceinline__ bf16x8 zero8() {
+  bf16x8 z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = (bf16)0.f;
+  return z;
+}
+
 template <class S>
 __global__ void __launch_bounds__(WAVES * 64) qkv_post_kernel(
     S* __restrict__ qkv, int64_t ld, int64_t q_off, int64_t k_off, int64_t v_off, const void* __restrict__ wq,
@@ -106,8 +113,11 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_kernel(
 }
 
 // The common case (pairs (i, i + D/2), the whole head rotated): both elements of a pair live in one
-// lane, so there is no exchange through LDS and no barrier, and every load of a head (values, gains,
-// angles) is issued before the first use. NP pairs per lane cover D <= 128 * NP.
+// lane, so there is no exchange through LDS and no barrier. A wave takes IPW heads of one token and
+// issues every load of all of them (values, gains, angles) before the first use; fewer, fatter waves
+// also keep the kernel off the wave-launch limit. NP pairs per lane cover D <= 128 * NP.
+constexpr int IPW = 4;  // head items per wave
+
 template <class S, int NP>
 __global__ void __launch_bounds__(WAVES * 64) qkv_post_neox_kernel(
     S* __restrict__ qkv, int64_t ld, int64_t q_off, int64_t k_off, int64_t v_off, const void* __restrict__ wq,
@@ -116,60 +126,229 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_neox_kernel(
     const int64_t* __restrict__ slots, int H, int Hkv, int D, int page) {
   const int64_t t = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int item = blockIdx.y * WAVES + wave;
-  if (item >= H + 2 * Hkv) return;
+  const int item0 = (blockIdx.y * WAVES + wave) * IPW;
+  const int items = H + 2 * Hkv;
+  if (item0 >= items) return;
   S* row = qkv + t * ld;
   const int64_t slot = slots ? slots[t] : -1;
   const int64_t blk = slot >= 0 ? slot / page : 0;
   const int off = slot >= 0 ? (int)(slot % page) : 0;
-  if (item >= H + Hkv) {
-    if (slot < 0) return;
-    const int hk = item - H - Hkv;
-    const S* vs = row + v_off + (int64_t)hk * D;
-    S* vd = v_cache + ((blk * Hkv + hk) * (int64_t)D) * page + off;
-    for (int d = lane; d < D; d += 64) vd[(int64_t)d * page] = vs[d];
-    return;
-  }
-  const bool is_q = item < H;
-  const int hk = item - H;
-  S* base = is_q ? row + q_off + (int64_t)item * D : row + k_off + (int64_t)hk * D;
-  const void* w = is_q ? wq : wk;
   const int half = D / 2;
   const float* cs = cos_sin ? cos_sin + (int64_t)pos[t] * D : nullptr;
-  float x1[NP], x2[NP], g1[NP], g2[NP], c[NP], sn[NP];
+
+  float x1[IPW][NP], x2[IPW][NP];
+  float g1q[NP], g2q[NP], g1k[NP], g2k[NP], c[NP], sn[NP];
 #pragma unroll
   for (int p = 0; p < NP; ++p) {
     const int i = lane + 64 * p;
     const bool ok = i < half;
-    x1[p] = ok ? to_f32(base[i]) : 0.f;
-    x2[p] = ok ? to_f32(base[i + half]) : 0.f;
-    g1[p] = (ok && w) ? ld_param<S>(w, i, wf32) + w_offset : 1.f;
-    g2[p] = (ok && w) ? ld_param<S>(w, i + half, wf32) + w_offset : 1.f;
+    g1q[p] = (ok && wq) ? ld_param<S>(wq, i, wf32) + w_offset : 1.f;
+    g2q[p] = (ok && wq) ? ld_param<S>(wq, i + half, wf32) + w_offset : 1.f;
+    g1k[p] = (ok && wk) ? ld_param<S>(wk, i, wf32) + w_offset : 1.f;
+    g2k[p] = (ok && wk) ? ld_param<S>(wk, i + half, wf32) + w_offset : 1.f;
     c[p] = (ok && cs) ? cs[i] : 1.f;
     sn[p] = (ok && cs) ? cs[half + i] : 0.f;
   }
-  float inv = 1.f;
-  if (w) {
-    float ss = 0.f;
 #pragma unroll
-    for (int p = 0; p < NP; ++p) ss += x1[p] * x1[p] + x2[p] * x2[p];
-    ss = wave_sum(ss);
-    inv = 1.f / sqrtf(ss / (float)D + eps);
+  for (int u = 0; u < IPW; ++u) {
+    const int item = item0 + u;
+    // q heads, then k heads, then v heads lie one after the other in the row when the offsets say so;
+    // in general each kind has its own offset
+    const S* src = item < H ? row + q_off + (int64_t)item * D
+                 : item < H + Hkv ? row + k_off + (int64_t)(item - H) * D
+                                  : row + v_off + (int64_t)(item - H - Hkv) * D;
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+      const int i = lane + 64 * p;
+      const bool ok = i < half && item < items;
+      x1[u][p] = ok ? to_f32(src[i]) : 0.f;
+      x2[u][p] = ok ? to_f32(src[i + half]) : 0.f;
+    }
   }
-  S* kd = (!is_q && slot >= 0) ? k_cache + ((blk * Hkv + hk) * (int64_t)page + off) * D : nullptr;
 #pragma unroll
-  for (int p = 0; p < NP; ++p) {
-    const int i = lane + 64 * p;
-    if (i < half) {
-      const float y1 = w ? x1[p] * inv * g1[p] : x1[p], y2 = w ? x2[p] * inv * g2[p] : x2[p];
-      const S r1 = from_f32<S>(y1 * c[p] - y2 * sn[p]), r2 = from_f32<S>(y2 * c[p] + y1 * sn[p]);
-      if (is_q) {
-        base[i] = r1;
-        base[i + half] = r2;
+  for (int u = 0; u < IPW; ++u) {
+    const int item = item0 + u;
+    if (item >= items) break;
+    if (item >= H + Hkv) {  // a v head: cache copy only
+      if (slot < 0) continue;
+      const int hk = item - H - Hkv;
+      S* vd = v_cache + ((blk * Hkv + hk) * (int64_t)D) * page + off;
+#pragma unroll
+      for (int p = 0; p < NP; ++p) {
+        const int i = lane + 64 * p;
+        if (i < half) {
+          vd[(int64_t)i * page] = from_f32<S>(x1[u][p]);  // the value came from S: the round trip is exact
+          vd[(int64_t)(i + half) * page] = from_f32<S>(x2[u][p]);
+        }
       }
-      if (kd) {
-        kd[i] = r1;
-        kd[i + half] = r2;
+      continue;
+    }
+    const bool is_q = item < H;
+    const bool normed = is_q ? wq != nullptr : wk != nullptr;
+    float inv = 1.f;
+    if (normed) {
+      float ss = 0.f;
+#pragma unroll
+      for (int p = 0; p < NP; ++p) ss += x1[u][p] * x1[u][p] + x2[u][p] * x2[u][p];
+      ss = wave_sum(ss);
+      inv = 1.f / sqrtf(ss / (float)D + eps);
+    }
+    const int hk = item - H;
+    S* base = is_q ? row + q_off + (int64_t)item * D : nullptr;
+    S* kd = (!is_q && slot >= 0) ? k_cache + ((blk * Hkv + hk) * (int64_t)page + off) * D : nullptr;
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+      const int i = lane + 64 * p;
+      if (i < half) {
+        const float y1 = normed ? x1[u][p] * inv * (is_q ? g1q[p] : g1k[p]) : x1[u][p];
+        const float y2 = normed ? x2[u][p] * inv * (is_q ? g2q[p] : g2k[p]) : x2[u][p];
+        const S r1 = from_f32<S>(y1 * c[p] - y2 * sn[p]), r2 = from_f32<S>(y2 * c[p] + y1 * sn[p]);
+        if (base) {
+          base[i] = r1;
+          base[i + half] = r2;
+        }
+        if (kd) {
+          kd[i] = r1;
+          kd[i + half] = r2;
+        }
+      }
+    }
+  }
+}
+
+// bf16, whole-head neox rotation, D in {64, 128, 256}: LPH = D / 8 lanes share a head, each with 8
+// consecutive dims in one 16-byte load; the partner of a pair sits LPH / 2 lanes away and comes by a
+// cross-lane read. A wave covers 64 / LPH heads of one token per instruction, an order of magnitude
+// fewer memory instructions than 2-byte accesses.
+template <int LPH>
+__global__ void __launch_bounds__(WAVES * 64) qkv_post_vec_kernel(
+    bf16* __restrict__ qkv, int64_t ld, int64_t q_off, int64_t k_off, int64_t v_off, const void* __restrict__ wq,
+    const void* __restrict__ wk, int wf32, float eps, float w_offset, const int32_t* __restrict__ pos,
+    const float* __restrict__ cos_sin, bf16* __restrict__ k_cache, bf16* __restrict__ v_cache,
+    const int64_t* __restrict__ slots, int H, int Hkv, int page, int skip_v) {
+  constexpr int D = LPH * 8, HALF = D / 2, HPW = 64 / LPH;  // heads per wave
+  const int64_t t = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int sub = lane / LPH, l = lane % LPH;  // which head of the wave, which 8 dims of it
+  const int item = (blockIdx.y * WAVES + wave) * HPW + sub;
+  const int items = H + 2 * Hkv;
+  const bool live = item < items;
+  const bool is_v = live && item >= H + Hkv, is_q = live && item < H, is_k = live && !is_q && !is_v;
+  bf16* row = qkv + t * ld;
+  const int64_t slot = slots ? slots[t] : -1;
+  const int64_t blk = slot >= 0 ? slot / page : 0;
+  const int off = slot >= 0 ? (int)(slot % page) : 0;
+  const int d0 = 8 * l;
+  bf16* src = is_q ? row + q_off + (int64_t)item * D
+            : is_k ? row + k_off + (int64_t)(item - H) * D
+                   : row + v_off + (int64_t)(item - H - Hkv) * D;
+  const void* w = is_q ? wq : wk;
+  bf16x8 xv = zero8();
+  if (live) xv = *(const bf16x8*)(src + d0);
+  if (is_v) {
+    if (slot >= 0 && !skip_v) {
+      bf16* vd = v_cache + ((blk * Hkv + (item - H - Hkv)) * (int64_t)D + d0) * page + off;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) vd[(int64_t)e * page] = xv[e];
+    }
+  }
+  const bool qk = is_q || is_k;
+  // gains and angles of this lane's dims: the pair index of dim d is d mod D/2
+  float g[8], c[8], sn[8];
+  const int pi = d0 % HALF;
+  if (qk && w) {
+    if (wf32) {
+      const f32x4 a = *(const f32x4*)((const float*)w + d0), b = *(const f32x4*)((const float*)w + d0 + 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { g[e] = a[e] + w_offset; g[4 + e] = b[e] + w_offset; }
+    } else {
+      const bf16x8 gv = *(const bf16x8*)((const bf16*)w + d0);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) g[e] = (float)gv[e] + w_offset;
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) g[e] = 1.f;
+  }
+  if (qk && cos_sin) {
+    const float* cs = cos_sin + (int64_t)pos[t] * D;
+    const f32x4 c0 = *(const f32x4*)(cs + pi), c1 = *(const f32x4*)(cs + pi + 4);
+    const f32x4 s0 = *(const f32x4*)(cs + HALF + pi), s1 = *(const f32x4*)(cs + HALF + pi + 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { c[e] = c0[e]; c[4 + e] = c1[e]; sn[e] = s0[e]; sn[4 + e] = s1[e]; }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { c[e] = 1.f; sn[e] = 0.f; }
+  }
+  float x[8], ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    x[e] = (float)xv[e];
+    ss += x[e] * x[e];
+  }
+  // every lane takes part in the cross-lane steps, whatever its head is
+#pragma unroll
+  for (int o = LPH / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+  const float inv = (qk && w) ? 1.f / sqrtf(ss / (float)D + eps) : 1.f;
+  float y[8], other[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) y[e] = (qk && w) ? x[e] * inv * g[e] : x[e];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) other[e] = __shfl_xor(y[e], LPH / 2, 64);
+  if (!qk) return;
+  const bool first = l < LPH / 2;  // this lane holds the first elements of its pairs
+  bf16x8 r;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) r[e] = (bf16)(first ? y[e] * c[e] - other[e] * sn[e] : y[e] * c[e] + other[e] * sn[e]);
+  if (is_q) {
+    *(bf16x8*)(src + d0) = r;
+  } else if (slot >= 0) {
+    *(bf16x8*)(k_cache + ((blk * Hkv + (item - H)) * (int64_t)page + off) * D + d0) = r;
+  }
+}
+
+// V into its transposed pages for many tokens: one wave takes 8 consecutive tokens of one kv head.
+// When their slots are 8 consecutive slots starting at a multiple of 8 (a prompt portion that starts
+// on such a boundary), a lane gathers two dims of the 8 tokens and stores them as two 16-byte rows
+// of V^T; otherwise it falls back to one 2-byte store per element.
+__global__ void __launch_bounds__(WAVES * 64) v_write_transposed_kernel(const bf16* __restrict__ qkv, int64_t ld,
+                                                                        int64_t v_off, bf16* __restrict__ v_cache,
+                                                                        const int64_t* __restrict__ slots, int T,
+                                                                        int Hkv, int D, int page) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t0 = (blockIdx.x * WAVES + wave) * 8, hk = blockIdx.y;
+  if (t0 >= T) return;
+  const int n = T - t0 < 8 ? T - t0 : 8;
+  const int64_t s0 = slots[t0];
+  bool aligned = n == 8 && s0 >= 0 && (s0 & 7) == 0;
+  for (int j = 1; j < n && aligned; ++j) aligned = slots[t0 + j] == s0 + j;
+  const bf16* src = qkv + (int64_t)t0 * ld + v_off + (int64_t)hk * D;
+  for (int d2 = lane; d2 < D / 2; d2 += 64) {
+    bf16x2 v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (j < n) v[j] = *(const bf16x2*)(src + (int64_t)j * ld + 2 * d2);
+    if (aligned) {
+      const int64_t blk = s0 / page;
+      const int off = (int)(s0 % page);
+      bf16* vd = v_cache + ((blk * Hkv + hk) * (int64_t)D + 2 * d2) * page + off;
+      bf16x8 a, b;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        a[j] = v[j][0];
+        b[j] = v[j][1];
+      }
+      *(bf16x8*)vd = a;
+      *(bf16x8*)(vd + page) = b;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        if (j >= n) break;
+        const int64_t sl = slots[t0 + j];
+        if (sl < 0) continue;
+        bf16* vd = v_cache + (((sl / page) * Hkv + hk) * (int64_t)D + 2 * d2) * page + sl % page;
+        vd[0] = v[j][0];
+        vd[page] = v[j][1];
       }
     }
   }
@@ -191,7 +370,31 @@ extern "C" int dinfer_qkv_post(int dtype, void* qkv, int64_t tokens, int64_t ld,
   const int items = heads + 2 * kv_heads;
   const dim3 grid((unsigned)tokens, (unsigned)((items + WAVES - 1) / WAVES));
   const bool whole_head_neox = style == 0 && head_dim % 2 == 0 && (!cos_sin || rotary_dim == head_dim);
+  const bool vec_ok = dtype == DT_BF16 && (head_dim == 64 || head_dim == 128 || head_dim == 256) && ld % 8 == 0 &&
+                      q_off % 8 == 0 && k_off % 8 == 0 && v_off % 8 == 0 && ((uintptr_t)qkv % 16) == 0 &&
+                      ((uintptr_t)q_gain % 16) == 0 && ((uintptr_t)k_gain % 16) == 0 && ((uintptr_t)cos_sin % 16) == 0 &&
+                      ((uintptr_t)k_cache % 16) == 0;
+  if (whole_head_neox && vec_ok) {
+    const int lph = head_dim / 8, hpw = 64 / lph;
+    const dim3 vgrid((unsigned)tokens, (unsigned)((items + WAVES * hpw - 1) / (WAVES * hpw)));
+    // many tokens: V goes to its transposed pages through the gathering kernel (16-byte stores)
+    const int skip_v = (slot_mapping && tokens >= 64 && page_size % 8 == 0 && ((uintptr_t)v_cache % 16) == 0) ? 1 : 0;
+    if (skip_v)
+      v_write_transposed_kernel<<<dim3((unsigned)((tokens + 8 * WAVES - 1) / (8 * WAVES)), (unsigned)kv_heads), WAVES * 64,
+                                  0, stream>>>((const bf16*)qkv, ld, v_off, (bf16*)v_cache, slot_mapping, (int)tokens,
+                                               kv_heads, head_dim, page_size);
+#define DINFER_QKV_VEC(LPH_)                                                                                          \
+  qkv_post_vec_kernel<LPH_><<<vgrid, WAVES * 64, 0, stream>>>(                                                         \
+      (bf16*)qkv, ld, q_off, k_off, v_off, q_gain, k_gain, w_f32, eps, w_offset, positions, cos_sin, (bf16*)k_cache, \
+      (bf16*)v_cache, slot_mapping, heads, kv_heads, page_size, skip_v)
+    if (lph == 8) DINFER_QKV_VEC(8);
+    else if (lph == 16) DINFER_QKV_VEC(16);
+    else DINFER_QKV_VEC(32);
+#undef DINFER_QKV_VEC
+    return launch_status();
+  }
   if (whole_head_neox) {
+    const dim3 grid((unsigned)tokens, (unsigned)((items + WAVES * IPW - 1) / (WAVES * IPW)));
     DINFER_DISPATCH_DTYPE(dtype, {
       if (head_dim <= 128)
         qkv_post_neox_kernel<S, 1><<<grid, WAVES * 64, 0, stream>>>(

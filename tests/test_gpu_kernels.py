@@ -92,7 +92,8 @@ def rope_table(max_pos, rd, theta):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,Hkv,D,page", [(16, 8, 128, 16), (6, 2, 48, 4), (5, 5, 80, 8), (4, 1, 256, 32)])
+@pytest.mark.parametrize("H,Hkv,D,page", [(16, 8, 128, 16), (6, 2, 48, 4), (5, 5, 80, 8), (4, 1, 256, 32), (7, 1, 64, 8),
+                                         (3, 3, 320, 8)])
 def test_qkv_post(dtype, H, Hkv, D, page):
     T, theta, eps, nblocks = 6, 1e6, 1e-6, 4
     width = (H + 2 * Hkv) * D
@@ -424,3 +425,35 @@ def test_gemm_small_m_gated(M):
             # one rounding of the result; the operands are exact here, so the sums are exact to float
             err = (out.double() - want).abs()
             assert bool((err <= 1e-2 * want.abs() + 1e-3 * want.std()).all()), f"M={M} N={N} K={K}: {float(err.max())}"
+
+
+@pytest.mark.parametrize("start", [0, 8, 3])
+def test_qkv_post_many_tokens_writes_v_transposed(start):
+    """From 64 tokens on, V is written by the gathering kernel: slots that start on a multiple of 8
+    (16-byte rows of V^T), slots that do not (element stores), pages in shuffled order, a ragged tail
+    and a token without a slot."""
+    H, Hkv, D, page, T = 8, 2, 128, 16, 77
+    qkv_in = torch.randn(T, (H + 2 * Hkv) * D, device=DEV).to(torch.bfloat16)
+    pos = torch.arange(start, start + T, device=DEV, dtype=torch.int32)
+    nblocks = 8
+    order = [5, 2, 7, 0, 3, 6, 1, 4]
+    slots = [order[p // page] * page + p % page for p in range(start, start + T)]
+    slots[40] = -1
+    slots_t = torch.tensor(slots, device=DEV, dtype=torch.int64)
+    table = rope_table(128, D, 1e6).to(DEV)
+    kc = torch.zeros(nblocks, Hkv, page, D, device=DEV, dtype=torch.bfloat16)
+    vc = torch.zeros(nblocks, Hkv, D, page, device=DEV, dtype=torch.bfloat16)
+    qkv = qkv_in.clone()
+    ops().qkv_post(qkv, T, heads=H, kv_heads=Hkv, head_dim=D, q_off=0, k_off=H * D, v_off=(H + Hkv) * D, q_gain=None,
+                   k_gain=None, eps=0.0, gain_offset=0.0, positions=pos, cos_sin=table, rotary_dim=D, rope_style=0,
+                   k_cache=kc, v_cache=vc, slot_mapping=slots_t, page_size=page)
+    v = qkv_in[:, (H + Hkv) * D:].view(T, Hkv, D)
+    want_v = torch.zeros_like(vc)
+    for t, s in enumerate(slots):
+        if s >= 0:
+            want_v[s // page, :, :, s % page] = v[t]
+    assert torch.equal(vc, want_v)
+    k = plain.rope_neox(qkv_in[:, H * D:(H + Hkv) * D].double().cpu().view(T, Hkv, D), plain.rope_angles(pos.tolist(), D, 1e6))
+    for t, s in enumerate(slots):
+        if s >= 0:
+            torch.testing.assert_close(kc[s // page, :, s % page, :].double().cpu(), k[t], rtol=2e-2, atol=2e-2)
