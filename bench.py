@@ -55,6 +55,7 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     ap.add_argument("--no-hip-graph", action="store_true")
+    ap.add_argument("--skip-prefill", action="store_true", help="do not time the 2,048-token prefill (profiling decode)")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py measures one GPU only (this engine does not use a second one); got --gpus {a.gpus}")
@@ -98,12 +99,14 @@ def main() -> int:
         eng.abort(rid)
         return dt
 
-    time_prefill()  # warm-up: library initialisation, first-use allocations
-    pre = min(time_prefill() for _ in range(3))
-    attn_flops = sizes["num_hidden_layers"] * 2 * PROMPT * PROMPT * cfg.head_dim * cfg.num_attention_heads
-    pre_flops = 2 * PROMPT * nums["linear_params"] + attn_flops + 2 * nums["head_params"]
-    prefill = {"value": round(PROMPT / pre, 1), "tokens": PROMPT, "ms": round(pre * 1e3, 3),
-               "frac": round(pre_flops / pre / MFMA_PEAK[a.dtype], 4)}
+    prefill = None
+    if not a.skip_prefill:
+        time_prefill()  # warm-up: library initialisation, first-use allocations
+        pre = min(time_prefill() for _ in range(3))
+        attn_flops = sizes["num_hidden_layers"] * 2 * PROMPT * PROMPT * cfg.head_dim * cfg.num_attention_heads
+        pre_flops = 2 * PROMPT * nums["linear_params"] + attn_flops + 2 * nums["head_params"]
+        prefill = {"value": round(PROMPT / pre, 1), "tokens": PROMPT, "ms": round(pre * 1e3, 3),
+                   "frac": round(pre_flops / pre / MFMA_PEAK[a.dtype], 4)}
 
     # ---- decode at a batch: B requests prefilled to 2,048 tokens, then timed decode steps
     def decode(batch, steps, warmup):
