@@ -158,3 +158,28 @@ def test_penalties_and_truncation_through_the_engine(model_dirs):
         row = plain.forward(cfg, w, ids)[-1]
         assert tok in row.topk(4).indices.tolist()         # top-3, with one more allowed at a rounding edge
         ids.append(tok)
+
+
+def test_command_line_generate(model_dirs, tmp_path):
+    """bin/dinfer generate: token ids in, token ids out, equal to the Python entry point."""
+    import json
+    import subprocess
+    import sys
+    from pathlib import Path
+    from dinfer_amd import SamplingParams
+    root = Path(__file__).resolve().parent.parent
+    name = "A"
+    prompts = prompts_for(name, [6, 11], 12)
+    f = tmp_path / "prompts.jsonl"
+    f.write_text(json.dumps(prompts[1]) + "\n")
+    p = subprocess.run([sys.executable, str(root / "bin" / "dinfer"), "generate", "--model", str(model_dirs[name]),
+                        "--dtype", "float32", "--max-model-len", "128", "--max-num-seqs", "4", "--block-size", "4",
+                        "--num-blocks", "64", "--max-num-batched-tokens", "32", "--prompt-ids",
+                        ",".join(map(str, prompts[0])), "--prompts-file", str(f), "--max-tokens", "5", "--temperature", "0",
+                        "--ignore-eos"], capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    got = [json.loads(l) for l in p.stdout.splitlines() if l.startswith("{")]
+    want = engine(model_dirs[name], name).generate(prompts, SamplingParams(max_tokens=5, temperature=0.0, ignore_eos=True))
+    assert [g["prompt_ids"] for g in got] == prompts and [g["output_ids"] for g in got] == want
+    p = subprocess.run([sys.executable, str(root / "bin" / "dinfer"), "device-info"], capture_output=True, text=True, timeout=120)
+    assert p.returncode == 0 and "gfx950" in json.loads(p.stdout)["arch"]

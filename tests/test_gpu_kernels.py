@@ -457,3 +457,17 @@ def test_qkv_post_many_tokens_writes_v_transposed(start):
     for t, s in enumerate(slots):
         if s >= 0:
             torch.testing.assert_close(kc[s // page, :, s % page, :].double().cpu(), k[t], rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_add_widen_fill(dtype):
+    a = torch.randn(5, 331, device=DEV).to(dtype)
+    b = torch.randn(5, 331, device=DEV).to(dtype)
+    want = (a.float() + b.float()).to(dtype)            # summed in float, one rounding
+    ops().add_inplace(a, b)
+    assert torch.equal(a, want)
+    wide = torch.empty(5, 331, device=DEV)
+    ops().widen(b, wide)
+    assert torch.equal(wide, b.float())
+    ops().fill_zero(wide)
+    assert not wide.any()
