@@ -170,11 +170,13 @@ struct Tile {
     bf16x8 pf[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
+      // raw scores; the running maximum m is kept in raw units too, and the scale is folded into
+      // one fused multiply-add per score: p = 2^(c s - c m), c = scale * log2(e) > 0
       float x[8];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        x[r] = s[t][0][r] * scale_log2e;
-        x[4 + r] = s[t][1][r] * scale_log2e;
+        x[r] = s[t][0][r];
+        x[4 + r] = s[t][1][r];
       }
       if (need_mask) {
 #pragma unroll
@@ -188,18 +190,24 @@ struct Tile {
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
       const float m_new = fmaxf(m[t], mx);
       const float m_use = m_new == -INFINITY ? 0.f : m_new;  // nothing visible yet: keep everything zero
-      const float alpha = exp2f(m[t] - m_use);
-      m[t] = m_new;
+      const float mc = m_use * scale_log2e;
       float ps_ = 0.f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float p = exp2f(x[e] - m_use);
+        const float p = exp2f(fmaf(x[e], scale_log2e, -mc));
         ps_ += p;
         pf[t][e] = (bf16)p;
       }
-      l[t] = l[t] * alpha + ps_;  // partial over this lane's keys; lane groups are summed at the end
+      // the maximum rarely moves after the first blocks; the output is rescaled only when it did for
+      // some column of the wave (a uniform branch)
+      if (__any(m_new > m[t])) {
+        const float alpha = exp2f(fmaf(m[t], scale_log2e, -mc));  // m = -inf: 0
+        l[t] *= alpha;
 #pragma unroll
-      for (int d = 0; d < DT; ++d) o[t][d] *= alpha;
+        for (int d = 0; d < DT; ++d) o[t][d] *= alpha;
+      }
+      m[t] = m_new;
+      l[t] += ps_;  // partial over this lane's keys; lane groups are summed at the end
     }
     // O^T += V^T . P
 #pragma unroll
@@ -384,7 +392,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 8)))
   if (i16 < G) {
     float* pp = part + (((int64_t)b * H + hk * G + i16) * splits + sp) * (D + 4);
     if (g4 == 0) {
-      pp[0] = tl.m[0];
+      pp[0] = tl.m[0] * scale_log2e;  // the tile keeps raw maxima; partials carry base-2 units
       pp[1] = lt;
     }
 #pragma unroll
@@ -499,6 +507,7 @@ extern "C" int dinfer_attn_mfma_supports(int head_dim, int page_size, int heads,
   return page_size > 0 && page_size % 8 == 0 && kv_heads > 0 && heads % kv_heads == 0 ? 1 : 0;
 }
 
+// skip_single: requests with one row are left to the split-K kernel.
 extern "C" int dinfer_attn_flash(const void* q, int64_t ld_q, void* out, int64_t ld_out, const void* k_cache,
                                  const void* v_cache, const int32_t* block_table, int64_t max_blocks,
                                  const int32_t* cu_seqlens, const int32_t* seq_lens, int num_reqs, int max_q_len,

@@ -250,6 +250,20 @@ def test_attention_decode_split_k(H, Hkv, D, page, window):
         torch.testing.assert_close(out.double().cpu().view(-1, H, D), want, rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("window", [0, 200])
+@pytest.mark.parametrize("H,Hkv,D,page", [(8, 2, 128, 16), (5, 5, 64, 8), (6, 1, 128, 24), (4, 2, 256, 16)])
+def test_attention_flash_long_portions(H, Hkv, D, page, window):
+    """Long portions: a whole prompt of 700, a portion of 300 on top of a history of 333, short requests in
+    the same launch (idle waves), and a single row behind 1000 keys."""
+    hist, new = [0, 333, 0, 77, 1000], [700, 300, 5, 130, 1]
+    q, kc, vc, m, outs = paged_case(torch.bfloat16, H, Hkv, D, page, hist, new, seed=13)
+    out = torch.zeros(sum(new), H * D, device=DEV, dtype=torch.bfloat16)
+    ops().attn_flash(q, out, kc, vc, m["bt"], m["cu"], m["sl"], len(hist), sum(new), max(new), scale=D ** -0.5,
+                     window=window, heads=H, kv_heads=Hkv, head_dim=D, page_size=page)
+    want = expected_attention(outs, hist, D ** -0.5, window)
+    torch.testing.assert_close(out.double().cpu().view(-1, H, D), want, rtol=2e-2, atol=2e-2)
+
+
 def test_attention_mixed_routes_single_rows_to_split_k():
     H, Hkv, D, page = 16, 4, 128, 16
     hist, new = [500, 0, 64, 900, 33, 10], [1, 40, 1, 1, 20, 1]
