@@ -1,5 +1,7 @@
 """The cache manager: pages per group of layers, a block table per request and
-group, and a slot of fixed size per request.
+group, and a slot of fixed size per request. The state lives in the C++ class
+of csrc/host/cache_manager.hpp; this front names requests by any hashable id
+and turns status codes into exceptions.
 
 Groups. Layers whose caches have the same page geometry and the same need
 ("all keys" or "the last W keys") form a group. A group has its own pool of
@@ -25,9 +27,13 @@ before the first step that uses it.
 """
 from __future__ import annotations
 
+import ctypes
+import itertools
 from dataclasses import dataclass
 
-from .block_pool import BlockPool
+from .. import native
+
+_I32, _I64 = ctypes.c_int32, ctypes.c_int64
 
 
 @dataclass(frozen=True)
@@ -38,149 +44,139 @@ class GroupSpec:
     window: int | None = None
 
 
-class _Req:
-    __slots__ = ("tables", "num_tokens", "slot")
+class _PoolView:
+    """What tests and reports read of one group's pool."""
 
-    def __init__(self, n_groups: int, slot: int):
-        self.tables: list[list[int]] = [[] for _ in range(n_groups)]
-        self.num_tokens = 0  # tokens for which pages have been allocated
-        self.slot = slot
+    def __init__(self, manager: "CacheManager", group: int):
+        self._m, self._g = manager, group
+        self.num_blocks = manager.groups[group].num_blocks
+
+    @property
+    def num_free(self) -> int:
+        return self._m.num_free(self._g)
+
+    def free_list(self) -> list[int]:
+        out = (_I32 * self.num_blocks)()
+        n = native.checked("dh_cache_free_list", self._m._h, self._g, out, self.num_blocks)
+        return list(out[:n])
 
 
 class CacheManager:
     def __init__(self, groups: list[GroupSpec], max_seqs: int):
-        if max_seqs <= 0:
-            raise ValueError("max_seqs must be positive")
         self.groups = list(groups)
-        self.pools = [BlockPool(g.num_blocks) for g in self.groups]
+        if len(self.groups) > native.MAX_GROUPS:
+            raise ValueError(f"{len(self.groups)} cache groups; at most {native.MAX_GROUPS} are supported")
+        n = len(self.groups)
+        arr = lambda vals: (_I32 * max(n, 1))(*vals)
+        self._h = native.created("dh_cache_create", n, arr([g.page_size for g in self.groups]),
+                                 arr([g.num_blocks for g in self.groups]),
+                                 arr([-1 if g.window is None else g.window for g in self.groups]), int(max_seqs))
         self.max_seqs = max_seqs
-        self._free_slots = list(range(max_seqs - 1, -1, -1))
-        self._fresh_slots: list[int] = []
-        self._reqs: dict = {}
+        self.pools = [_PoolView(self, g) for g in range(n)]
+        self._handles: dict = {}          # request id -> the number the core knows it by
+        self._pinned: set = set()         # ids whose number outlives free() (a scheduler owns them)
+        self._numbers = itertools.count(1)
+        self._slots = (_I32 * max_seqs)()
+        self._need = (_I32 * max(n, 1))()
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            native.fn("dh_cache_destroy")(h)
+
+    # ---- request numbers -------------------------------------------------------------------------
+    def handle(self, req_id, create: bool = False, pin: bool = False) -> int:
+        h = self._handles.get(req_id)
+        if h is None:
+            if not create:
+                raise KeyError(f"request {req_id!r} is not live")
+            h = self._handles[req_id] = next(self._numbers)
+        if pin:
+            self._pinned.add(req_id)
+        return h
+
+    def forget(self, req_id) -> None:
+        """Drops the number of a request that a scheduler owned (after it has finished)."""
+        self._pinned.discard(req_id)
+        self._handles.pop(req_id, None)
 
     # ---- requests ------------------------------------------------------------------------------
     def has(self, req_id) -> bool:
-        return req_id in self._reqs
+        h = self._handles.get(req_id)
+        return h is not None and bool(native.fn("dh_cache_has")(self._h, h))
 
     def can_admit(self) -> bool:
-        return bool(self._free_slots)
+        return bool(native.fn("dh_cache_can_admit")(self._h))
 
     def admit(self, req_id) -> int:
         """Registers a request and gives it a state slot. Raises if it is known or no slot is free."""
-        if req_id in self._reqs:
+        if self.has(req_id):
             raise KeyError(f"request {req_id!r} is already live")
-        if not self._free_slots:
-            raise RuntimeError(f"all {self.max_seqs} request slots are taken")
-        slot = self._free_slots.pop()
-        self._fresh_slots.append(slot)
-        self._reqs[req_id] = _Req(len(self.groups), slot)
-        return slot
+        fresh = req_id not in self._handles
+        try:
+            return native.checked("dh_cache_admit", self._h, self.handle(req_id, create=True))
+        except Exception:
+            if fresh:
+                self._handles.pop(req_id, None)
+            raise
 
     def take_fresh_slots(self) -> list[int]:
-        out, self._fresh_slots = self._fresh_slots, []
-        return out
+        n = native.checked("dh_cache_take_fresh_slots", self._h, self._slots, self.max_seqs)
+        return list(self._slots[:n])
 
     def slot_of(self, req_id) -> int:
-        return self._reqs[req_id].slot
+        return native.checked("dh_cache_slot_of", self._h, self.handle(req_id))
 
     def live_requests(self) -> list:
-        return list(self._reqs)
+        out = (_I64 * self.max_seqs)()
+        n = native.fn("dh_cache_live_requests")(self._h, out, self.max_seqs)
+        by_number = {h: rid for rid, h in self._handles.items()}
+        return [by_number[h] for h in out[:n]]
 
     # ---- pages ---------------------------------------------------------------------------------
-    def _first_needed_page(self, g: GroupSpec, next_pos: int) -> int:
-        """Index of the first page a token at next_pos (and later ones) can still read."""
-        if g.window is None:
-            return 0
-        first_key = max(0, next_pos - g.window + 1)
-        return first_key // g.page_size
-
     def pages_needed(self, req_id, num_computed: int, num_new: int) -> list[int]:
         """Per group, how many new pages the tokens [num_computed, num_computed + num_new) need."""
-        r = self._reqs[req_id]
-        end = num_computed + num_new
-        need = []
-        for g, tab in zip(self.groups, r.tables):
-            want = -(-end // g.page_size)
-            need.append(max(0, want - len(tab)))
-        return need
+        native.checked("dh_cache_pages_needed", self._h, self.handle(req_id), num_computed, num_new, self._need)
+        return list(self._need[:len(self.groups)])
 
     def allocate(self, req_id, num_computed: int, num_new: int) -> bool:
         """Pages for tokens [num_computed, num_computed + num_new) in every group, or nothing at all."""
-        if num_new <= 0:
-            raise ValueError("a step feeds at least one token per request")
-        r = self._reqs[req_id]
-        need = self.pages_needed(req_id, num_computed, num_new)
-        if any(n > p.num_free for n, p in zip(need, self.pools)):
-            return False
-        for n, pool, tab in zip(need, self.pools, r.tables):
-            tab.extend(pool.allocate(n))
-        r.num_tokens = max(r.num_tokens, num_computed + num_new)
-        return True
+        return bool(native.checked("dh_cache_allocate", self._h, self.handle(req_id), num_computed, num_new))
 
     def release_passed(self, req_id, num_computed: int) -> int:
         """After a step: frees the pages of window groups that the token at position
         num_computed and all later ones cannot see. Returns how many were freed."""
-        r = self._reqs[req_id]
-        n = 0
-        for g, pool, tab in zip(self.groups, self.pools, r.tables):
-            if g.window is None:
-                continue
-            first = min(self._first_needed_page(g, num_computed), len(tab))
-            dead = [b for b in tab[:first] if b >= 0]
-            if dead:
-                pool.free(dead)
-                n += len(dead)
-                for i in range(first):
-                    tab[i] = -1
-        return n
+        return native.checked("dh_cache_release_passed", self._h, self.handle(req_id), num_computed)
 
     def free(self, req_id) -> None:
         """Gives back everything the request holds, the last page first, so the tail of a
         request is what the next allocation takes (kv/manager.rs:338-345)."""
-        r = self._reqs.pop(req_id)
-        for pool, tab in zip(self.pools, r.tables):
-            pool.free([b for b in reversed(tab) if b >= 0])
-        self._free_slots.append(r.slot)
-        if r.slot in self._fresh_slots:
-            self._fresh_slots.remove(r.slot)
+        native.checked("dh_cache_free", self._h, self.handle(req_id))
+        if req_id not in self._pinned:
+            del self._handles[req_id]
 
     # ---- views for the step --------------------------------------------------------------------
     def block_table(self, req_id, group: int) -> list[int]:
-        return self._reqs[req_id].tables[group]
+        cap = self.groups[group].num_blocks
+        out = (_I32 * cap)()
+        n = native.checked("dh_cache_block_table", self._h, self.handle(req_id), group, out, cap)
+        if n > cap:  # more entries than pages: entries of pages given back stay in the table as -1
+            out = (_I32 * n)()
+            n = native.checked("dh_cache_block_table", self._h, self.handle(req_id), group, out, n)
+        return list(out[:n])
 
     def slot_mapping(self, req_id, group: int, start: int, n: int) -> list[int]:
         """Cache slots (page * page_size + offset) of positions start .. start + n - 1."""
-        tab = self._reqs[req_id].tables[group]
-        ps = self.groups[group].page_size
-        out = []
-        for pos in range(start, start + n):
-            b = tab[pos // ps]
-            if b < 0:
-                raise RuntimeError(f"request {req_id!r}: position {pos} lies in a page that was given back")
-            out.append(b * ps + pos % ps)
-        return out
+        out = (_I64 * max(n, 1))()
+        native.checked("dh_cache_slot_mapping", self._h, self.handle(req_id), group, start, n, out,
+                       context=f"request {req_id!r}: ")
+        return list(out[:n])
 
     def num_free(self, group: int = 0) -> int:
-        return self.pools[group].num_free
+        return native.checked("dh_cache_num_free", self._h, group)
 
     def check(self) -> None:
-        """Invariants: no page lost, none held twice, every held page in exactly one table."""
-        for gi, pool in enumerate(self.pools):
-            pool.check()
-            seen = set()
-            for rid, r in self._reqs.items():
-                for b in r.tables[gi]:
-                    if b < 0:
-                        continue
-                    if b in seen:
-                        raise AssertionError(f"group {gi}: page {b} is in two block tables")
-                    if not pool.is_held(b):
-                        raise AssertionError(f"group {gi}: page {b} of {rid!r} is on the free list")
-                    seen.add(b)
-            if len(seen) + pool.num_free != pool.num_blocks:
-                raise AssertionError(f"group {gi}: {pool.num_blocks - pool.num_free - len(seen)} pages are lost")
-        slots = [r.slot for r in self._reqs.values()]
-        if len(set(slots)) != len(slots) or set(slots) & set(self._free_slots):
-            raise AssertionError("a state slot is held twice")
-        if len(slots) + len(self._free_slots) != self.max_seqs:
-            raise AssertionError("a state slot is lost")
+        """Invariants: no page lost, none held twice, every held page in exactly one table;
+        no state slot lost or held twice; every live request of the core has a name here."""
+        native.checked("dh_cache_check", self._h)
+        self.live_requests()

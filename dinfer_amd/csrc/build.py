@@ -1,6 +1,7 @@
-"""Compiles the HIP sources of this folder for gfx950, one shared library per
-source file, into ``dinfer_amd/_lib/`` (or a per-user temporary folder when the
-package folder is read-only).
+"""Compiles the sources of this folder, one shared library per entry of SOURCES,
+into ``dinfer_amd/_lib/`` (or a per-user temporary folder when the package folder
+is read-only): the HIP kernels for gfx950 with hipcc, the host core (page pools,
+cache manager, scheduler, batch fill; plain C++) with the host compiler.
 
 A library is built on first use and reused afterwards; ``build_all(force=True)``
 recompiles everything. Only what a caller asks for is compiled, so a program
@@ -31,8 +32,13 @@ SOURCES = {
     "gemm_ref": "gemm_ref.hip",
     "gemm": "gemm.hip",
     "sampling": "sampling.hip",
+    "host": "host/api.cpp",
 }
 HEADERS = ["common.cuh"]
+# libraries without device code, and the headers each is made of
+HOST_ONLY = {"host": ["host/dinfer_host.h", "host/errors.hpp", "host/block_pool.hpp", "host/cache_manager.hpp",
+                      "host/step_batch.hpp", "host/scheduler.hpp"]}
+HOST_FLAGS = ["-O2", "-std=c++17", "-shared", "-fPIC", "-Wall"]
 
 ARCH = "gfx950"
 # -packed-fp32-ops is switched off for device code: hipcc -O3 otherwise forms packed
@@ -47,6 +53,14 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result",
 ]
+
+
+def _host_cxx() -> str:
+    for cand in (os.environ.get("CXX"), "g++", "c++", "clang++"):
+        path = shutil.which(cand) if cand else None
+        if path:
+            return path
+    return _hipcc()  # hipcc compiles plain C++ too
 
 
 def _hipcc() -> str:
@@ -73,9 +87,9 @@ def lib_dir() -> Path:
 
 def source_hash(name: str) -> str:
     h = hashlib.sha256()
-    for f in HEADERS + [SOURCES[name]]:
+    for f in HOST_ONLY.get(name, HEADERS) + [SOURCES[name]]:
         h.update((CSRC / f).read_bytes())
-    h.update(" ".join(FLAGS).encode())
+    h.update(" ".join(HOST_FLAGS if name in HOST_ONLY else FLAGS).encode())
     return h.hexdigest()[:16]
 
 
@@ -101,15 +115,20 @@ def is_stale(name: str, path: Path) -> bool:
 
 
 def build(name: str, verbose: bool = True) -> Path:
-    """Compiles one library and returns its path. Prints a line now and then while hipcc runs."""
+    """Compiles one library and returns its path. Prints a line now and then while the compiler runs."""
     if name not in SOURCES:
-        raise KeyError(f"unknown kernel library {name!r}; known: {sorted(SOURCES)}")
+        raise KeyError(f"unknown library {name!r}; known: {sorted(SOURCES)}")
     out = lib_path(name)
     tmp = out.with_name(f".{out.name}.{os.getpid()}.tmp")
-    cmd = [_hipcc(), *FLAGS, str(CSRC / SOURCES[name]), "-o", str(tmp)]
+    if name in HOST_ONLY:
+        cmd = [_host_cxx(), *HOST_FLAGS, str(CSRC / SOURCES[name]), "-o", str(tmp)]
+        what = "the host"
+    else:
+        cmd = [_hipcc(), *FLAGS, str(CSRC / SOURCES[name]), "-o", str(tmp)]
+        what = ARCH
     t0 = time.time()
     if verbose:
-        print(f"[dinfer_amd] compiling {SOURCES[name]} for {ARCH} ...", file=sys.stderr, flush=True)
+        print(f"[dinfer_amd] compiling {SOURCES[name]} for {what} ...", file=sys.stderr, flush=True)
     proc = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, cwd=str(CSRC))
     done = threading.Event()
 
@@ -125,7 +144,7 @@ def build(name: str, verbose: bool = True) -> Path:
     log = "\n".join(l for l in log.splitlines() if "packed-fp32-ops" not in l)
     if proc.returncode != 0:
         tmp.unlink(missing_ok=True)
-        raise RuntimeError(f"hipcc failed for {SOURCES[name]}:\n{log}")
+        raise RuntimeError(f"{Path(cmd[0]).name} failed for {SOURCES[name]}:\n{log}")
     os.replace(tmp, out)
     out.with_suffix(".hash").write_text(source_hash(name))
     if verbose:

@@ -1,0 +1,280 @@
+// Continuous batching: admits requests, cuts prompts into portions under a token budget,
+// decodes, finishes and frees. It sees the cache only through the cache manager. The rules are
+// the reference's (crates/core/src/sched/mod.rs):
+//
+//   * no separate prefill and decode phases: each step a request gets min(tokens it still has
+//     to compute, what the budget allows) tokens (:1-11,377);
+//   * running requests first, in admission order, then waiting ones first-come first-served
+//     while budget, request slots and pages last (:350-477);
+//   * a decode row (one token, with history) does not consume the budget when
+//     decode_exempt_from_budget is set (:351,361-365);
+//   * when pages run out for a running request, the last running request is preempted: its
+//     pages are freed, it forgets what it computed and goes to the front of the waiting queue,
+//     to recompute prompt and outputs later (:402-436,672-680). If the requester is itself the
+//     last one it is skipped this step while others run, and finished with "length" if it is
+//     alone (:414-432). A waiting request that cannot get pages waits (:571-573). A step that
+//     preempted admits nobody (:473);
+//   * finish: eos or stop id (after min_tokens, unless ignore_eos), max_tokens outputs, or
+//     max_model_len tokens (:816-828).
+#pragma once
+#include <algorithm>
+#include <cstdint>
+#include <deque>
+#include <memory>
+#include <unordered_map>
+#include <unordered_set>
+#include <vector>
+
+#include "cache_manager.hpp"
+#include "step_batch.hpp"
+
+namespace dinfer {
+
+struct SchedOptions {
+    int32_t max_num_batched_tokens;
+    int32_t max_num_seqs;
+    int32_t max_model_len;
+    int32_t prefill_tokens_per_step;       // 0: no cap
+    int32_t long_prefill_token_threshold;  // 0: no cap
+    int32_t enable_chunked_prefill;
+    int32_t decode_exempt_from_budget;
+};
+
+enum Status : int32_t { WAITING = 0, RUNNING = 1, PREEMPTED = 2, FINISHED = 3 };
+enum Reason : int32_t { NO_REASON = 0, STOP = 1, LENGTH = 2, ABORT = 3 };
+
+struct Request {
+    int64_t id = 0;
+    std::vector<int32_t> tokens;  // prompt, then outputs
+    int32_t num_prompt = 0;
+    int32_t num_computed = 0;
+    Status status = WAITING;
+    Reason reason = NO_REASON;
+    int32_t max_tokens = 0, min_tokens = 0;
+    bool ignore_eos = false;
+    std::vector<int32_t> stop_ids;
+    int32_t preemptions = 0;
+
+    int32_t num_tokens() const { return static_cast<int32_t>(tokens.size()); }
+    int32_t num_output() const { return num_tokens() - num_prompt; }
+};
+
+struct Scheduled {
+    int64_t id;
+    int32_t start;    // tokens computed before this step
+    int32_t num_new;  // tokens this step feeds
+    int32_t samples;  // the step reaches the end of the known tokens, so a token is sampled
+};
+
+struct StepPlan {
+    std::vector<Scheduled> scheduled;  // running first, then newly admitted
+    std::vector<int64_t> preempted;
+    std::vector<std::pair<int64_t, Reason>> force_finished;  // ended by the scheduler itself
+};
+
+struct UpdateResult {
+    int64_t id;
+    int32_t token;   // -1: nothing sampled
+    int32_t reason;  // Reason; NO_REASON while the request goes on
+};
+
+class Scheduler {
+public:
+    Scheduler(const SchedOptions& opt, CacheManager* cache, const int32_t* eos, int n_eos)
+        : opt_(opt), cache_(cache), eos_(eos, eos + n_eos) {}
+
+    // ---- intake
+    void add(std::unique_ptr<Request> req) {
+        if (reqs_.count(req->id)) throw Error(ERR_KEY, "the request id is in use");
+        if (req->tokens.empty()) throw Error(ERR_VALUE, "a prompt needs at least one token");
+        req->num_prompt = req->num_tokens();
+        if (req->num_prompt >= opt_.max_model_len)
+            throw Error(ERR_VALUE, "prompt of " + std::to_string(req->num_prompt) +
+                                       " tokens leaves no room for output within max_model_len " +
+                                       std::to_string(opt_.max_model_len));
+        req->status = WAITING;
+        req->num_computed = 0;
+        Request* r = req.get();
+        reqs_.emplace(r->id, std::move(req));
+        waiting_.push_back(r);
+    }
+
+    bool has_unfinished() const { return !waiting_.empty() || !running_.empty(); }
+    const Request* get(int64_t id) const {
+        auto it = reqs_.find(id);
+        return it == reqs_.end() ? nullptr : it->second.get();
+    }
+    const std::deque<Request*>& waiting() const { return waiting_; }
+    const std::vector<Request*>& running() const { return running_; }
+    const StepPlan& plan() const { return plan_; }
+    const CacheManager* cache() const { return cache_; }
+
+    void abort(int64_t id) {
+        auto it = reqs_.find(id);
+        if (it != reqs_.end()) finish(it->second.get(), ABORT);
+    }
+
+    // A finished request stays readable until the owner has taken its final state.
+    void forget(int64_t id) {
+        auto it = reqs_.find(id);
+        if (it != reqs_.end() && it->second->status == FINISHED) reqs_.erase(it);
+    }
+
+    // ---- one step
+    const StepPlan& schedule() {
+        plan_.scheduled.clear();
+        plan_.preempted.clear();
+        plan_.force_finished.clear();
+        int64_t budget = opt_.max_num_batched_tokens;
+        int64_t quota = opt_.prefill_tokens_per_step > 0 ? opt_.prefill_tokens_per_step : (int64_t(1) << 62);
+        const size_t eligible = running_.size() + waiting_.size();
+        const int64_t threshold = eligible > 1 ? opt_.long_prefill_token_threshold : 0;
+        bool preempted_any = false;
+
+        size_t i = 0;
+        while (i < running_.size()) {
+            Request* r = running_[i];
+            const int64_t remaining = r->num_tokens() - r->num_computed;
+            const bool is_decode = remaining == 1 && r->num_computed > 0;
+            const bool charged = !(opt_.decode_exempt_from_budget && is_decode);
+            if (charged && budget == 0) break;
+            int64_t n = remaining;
+            if (threshold && n > threshold) n = threshold;
+            if (charged) n = std::min(n, budget);
+            if (!is_decode) n = std::min(n, quota);
+            if (n < remaining && !opt_.enable_chunked_prefill) n = 0;
+            if (n <= 0) {
+                ++i;
+                continue;
+            }
+            bool got = false;
+            for (;;) {
+                if (cache_->allocate(r->id, r->num_computed, n)) {
+                    got = true;
+                    break;
+                }
+                Request* victim = running_.back();
+                if (victim == r) {
+                    if (running_.size() > 1) break;  // others hold the pages; try again next step, never preempt oneself
+                    finish(r, LENGTH);               // alone and still no page: the pool cannot hold it
+                    plan_.force_finished.emplace_back(r->id, LENGTH);
+                    break;
+                }
+                running_.pop_back();
+                preempt(victim);
+                plan_.preempted.push_back(victim->id);
+                preempted_any = true;
+            }
+            if (!got) break;
+            plan_.scheduled.push_back({r->id, r->num_computed, static_cast<int32_t>(n),
+                                       r->num_computed + n == r->num_tokens()});
+            if (charged) budget -= n;
+            if (!is_decode) quota -= n;
+            ++i;
+        }
+
+        if (!preempted_any) {
+            while (budget > 0 && !waiting_.empty() && static_cast<int>(running_.size()) < opt_.max_num_seqs) {
+                Request* r = waiting_.front();
+                const int64_t remaining = r->num_tokens() - r->num_computed;
+                int64_t n = remaining;
+                if (threshold && n > threshold) n = threshold;
+                n = std::min(n, std::min(budget, quota));
+                if (n < remaining && !opt_.enable_chunked_prefill) n = 0;
+                if (n <= 0) break;
+                if (!cache_->can_admit()) break;
+                cache_->admit(r->id);
+                if (!cache_->allocate(r->id, r->num_computed, n)) {
+                    cache_->free(r->id);  // no pages now: wait
+                    break;
+                }
+                waiting_.pop_front();
+                r->status = RUNNING;
+                running_.push_back(r);
+                plan_.scheduled.push_back({r->id, r->num_computed, static_cast<int32_t>(n),
+                                           r->num_computed + n == r->num_tokens()});
+                budget -= n;
+                quota -= n;
+            }
+        }
+        // advance at once, as the reference does after scheduling (:646-670)
+        for (const Scheduled& s : plan_.scheduled) {
+            Request* r = reqs_.at(s.id).get();
+            if (r->status == RUNNING) r->num_computed = s.start + s.num_new;
+        }
+        return plan_;
+    }
+
+    // sampled: one token for every scheduled request that samples, in the plan's order.
+    // Appends one result for every scheduled request that is still running.
+    void update(const int32_t* sampled, int n_sampled, std::vector<UpdateResult>& results) {
+        int k = 0;
+        for (const Scheduled& s : plan_.scheduled) {
+            const int at = s.samples ? k++ : -1;
+            auto it = reqs_.find(s.id);
+            if (it == reqs_.end() || it->second->status != RUNNING) continue;  // preempted or aborted meanwhile
+            Request* r = it->second.get();
+            cache_->release_passed(r->id, r->num_computed);
+            int32_t tok = -1;
+            Reason reason = NO_REASON;
+            if (s.samples) {
+                if (at >= n_sampled) throw Error(ERR_VALUE, "fewer sampled tokens than sampling requests");
+                tok = sampled[at];
+                r->tokens.push_back(tok);
+                reason = check_stop(*r, tok);
+                if (reason != NO_REASON) finish(r, reason);
+            }
+            results.push_back({r->id, tok, reason});
+        }
+    }
+
+    // The plan's entries over the requests' own token storage (valid until the next update).
+    void plan_entries(std::vector<EntryView>& entries, std::vector<int32_t>& want_store) const {
+        entries.clear();
+        want_store.assign(plan_.scheduled.size(), 0);
+        size_t i = 0;
+        for (const Scheduled& s : plan_.scheduled) {
+            const Request* r = reqs_.at(s.id).get();
+            want_store[i] = s.num_new - 1;
+            entries.push_back({s.id, s.start, s.num_new, r->tokens.data() + s.start, &want_store[i], s.samples ? 1 : 0});
+            ++i;
+        }
+    }
+
+private:
+    Reason check_stop(const Request& r, int32_t tok) const {
+        if (r.num_output() >= r.min_tokens) {
+            if (!r.ignore_eos && eos_.count(tok)) return STOP;
+            if (std::find(r.stop_ids.begin(), r.stop_ids.end(), tok) != r.stop_ids.end()) return STOP;
+        }
+        if (r.num_tokens() >= opt_.max_model_len || r.num_output() >= r.max_tokens) return LENGTH;
+        return NO_REASON;
+    }
+
+    void preempt(Request* r) {
+        cache_->free(r->id);
+        r->num_computed = 0;
+        r->status = PREEMPTED;
+        ++r->preemptions;
+        waiting_.push_front(r);
+    }
+
+    void finish(Request* r, Reason reason) {
+        if (r->status == FINISHED) return;
+        if (cache_->has(r->id)) cache_->free(r->id);
+        running_.erase(std::remove(running_.begin(), running_.end(), r), running_.end());
+        waiting_.erase(std::remove(waiting_.begin(), waiting_.end(), r), waiting_.end());
+        r->status = FINISHED;
+        r->reason = reason;
+    }
+
+    SchedOptions opt_;
+    CacheManager* cache_;
+    std::unordered_set<int32_t> eos_;
+    std::deque<Request*> waiting_;
+    std::vector<Request*> running_;
+    std::unordered_map<int64_t, std::unique_ptr<Request>> reqs_;
+    StepPlan plan_;
+};
+
+}  // namespace dinfer

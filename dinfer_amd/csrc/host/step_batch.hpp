@@ -1,0 +1,139 @@
+// Writes the flat batch of one step into the pinned host buffer.
+//
+// A step holds, for each request in it, a contiguous run of its next tokens: whole prompts,
+// portions of prompts and single decoded tokens side by side (crates/core/src/runner.rs:745-876):
+//
+//   input_ids    [T]     the tokens
+//   positions    [T]     absolute position of each token
+//   slot_mapping [T]     per cache group: page * page_size + position % page_size
+//   cu_seqlens   [B+1]   prefix sums of the tokens per request
+//   seq_lens     [B]     request length after this step (start + n)
+//   block_table  [B, MB] per cache group, -1 where no page is held
+//   state_slots  [B]     the request's fixed-size state slot
+//   logits_rows  [R]     rows of the flat batch whose logits are wanted
+//
+// Padding (pad_to > B): a step of single rows that replays a captured graph of pad_to requests
+// is filled up with requests of one token at position 0 that write no cache slot (slot -1) and
+// read page 0, which always exists (crates/layers/src/exec.rs:388-426).
+#pragma once
+#include <cstdint>
+#include <cstring>
+#include <string>
+
+#include "cache_manager.hpp"
+
+namespace dinfer {
+
+constexpr int MAX_GROUPS = 8;
+
+// Addresses inside the pinned buffer and the capacities they were sized for.
+struct BatchBuffers {
+    int32_t n_groups, max_tokens, max_reqs, max_rows;
+    int32_t* input_ids;
+    int32_t* positions;
+    int32_t* cu_seqlens;
+    int32_t* seq_lens;
+    int32_t* state_slots;
+    int32_t* logits_rows;
+    int64_t* slot_mapping[MAX_GROUPS];
+    int32_t* block_table[MAX_GROUPS];
+    int32_t max_blocks[MAX_GROUPS];
+};
+
+// What the host needs to know about the step it just described.
+struct BatchFacts {
+    int32_t num_tokens, num_reqs, num_rows, max_q_len, max_seq_len, num_singles;
+};
+
+// One request's share of a step. `tokens` has `count` ids; `want` has `n_want` indices into them.
+struct EntryView {
+    int64_t rid;
+    int32_t start, count;
+    const int32_t* tokens;
+    const int32_t* want;
+    int32_t n_want;
+};
+
+inline void fill_batch(const CacheManager& cache, const BatchBuffers& buf, const EntryView* entries, int n_entries,
+                       int pad_to, BatchFacts* facts) {
+    if (buf.n_groups != cache.num_groups() || buf.n_groups > MAX_GROUPS)
+        throw Error(ERR_VALUE, "the batch buffers were laid out for another number of cache groups");
+    int64_t T = 0, R = 0;
+    for (int b = 0; b < n_entries; ++b) {
+        if (entries[b].count <= 0) throw Error(ERR_VALUE, "entry " + std::to_string(b) + " brings no token to this step");
+        T += entries[b].count;
+        R += entries[b].n_want;
+    }
+    const int B = n_entries;
+    if (B == 0) throw Error(ERR_VALUE, "a step needs at least one request with at least one token");
+    if (B > buf.max_reqs)
+        throw Error(ERR_VALUE, std::to_string(B) + " requests in one step, the engine was built for " + std::to_string(buf.max_reqs));
+    if (T > buf.max_tokens)
+        throw Error(ERR_VALUE, std::to_string(T) + " tokens in one step, the engine was built for " + std::to_string(buf.max_tokens));
+    if (R > buf.max_rows)
+        throw Error(ERR_VALUE, "logits wanted at " + std::to_string(R) + " places, the engine was built for " + std::to_string(buf.max_rows));
+
+    int t = 0, r = 0, max_q = 0, max_len = 0, singles = 0;
+    buf.cu_seqlens[0] = 0;
+    for (int b = 0; b < B; ++b) {
+        const EntryView& e = entries[b];
+        const int n = e.count;
+        std::memcpy(buf.input_ids + t, e.tokens, sizeof(int32_t) * n);
+        for (int i = 0; i < n; ++i) buf.positions[t + i] = e.start + i;
+        for (int g = 0; g < buf.n_groups; ++g) {
+            const std::vector<int32_t>& tab = cache.block_table(e.rid, g);
+            const int mb = buf.max_blocks[g];
+            if (static_cast<int>(tab.size()) > mb)
+                throw Error(ERR_VALUE, "entry " + std::to_string(b) + " holds " + std::to_string(tab.size()) +
+                                           " pages, the block table has " + std::to_string(mb) + " columns");
+            int32_t* row = buf.block_table[g] + static_cast<int64_t>(b) * mb;
+            std::memcpy(row, tab.data(), sizeof(int32_t) * tab.size());
+            for (int i = static_cast<int>(tab.size()); i < mb; ++i) row[i] = -1;
+            cache.slot_mapping(e.rid, g, e.start, n, buf.slot_mapping[g] + t);
+        }
+        buf.cu_seqlens[b + 1] = t + n;
+        buf.seq_lens[b] = e.start + n;
+        buf.state_slots[b] = cache.slot_of(e.rid);
+        for (int i = 0; i < e.n_want; ++i) {
+            int w = e.want[i];
+            if (w < 0 || w >= n)
+                throw Error(ERR_VALUE, "entry " + std::to_string(b) + ": wanted place " + std::to_string(w) +
+                                           " is outside its " + std::to_string(n) + " tokens");
+            buf.logits_rows[r++] = t + w;
+        }
+        max_q = n > max_q ? n : max_q;
+        max_len = e.start + n > max_len ? e.start + n : max_len;
+        singles += n == 1;
+        t += n;
+    }
+    int Bp = B;
+    if (pad_to > B) {
+        const int P = pad_to;
+        if (T != B || R != B || P > buf.max_reqs || P > buf.max_tokens || P > buf.max_rows)
+            throw Error(ERR_VALUE, "only a step of single rows that all want logits can be padded");
+        for (int b = B; b < P; ++b) {
+            buf.input_ids[b] = 0;
+            buf.positions[b] = 0;
+            buf.cu_seqlens[b + 1] = b + 1;
+            buf.seq_lens[b] = 1;
+            buf.state_slots[b] = 0;
+            buf.logits_rows[b] = b;
+            for (int g = 0; g < buf.n_groups; ++g) {
+                int32_t* row = buf.block_table[g] + static_cast<int64_t>(b) * buf.max_blocks[g];
+                std::memset(row, 0, sizeof(int32_t) * buf.max_blocks[g]);
+                buf.slot_mapping[g][b] = -1;
+            }
+        }
+        singles += P - B;
+        if (max_len < 1) max_len = 1;
+        T = R = Bp = P;
+    }
+    facts->num_tokens = static_cast<int32_t>(T);
+    facts->num_reqs = Bp;
+    facts->num_rows = static_cast<int32_t>(R);
+    facts->max_q_len = max_q;
+    facts->max_seq_len = max_len;
+    facts->num_singles = singles;
+}
+
+}  // namespace dinfer

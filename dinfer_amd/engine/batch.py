@@ -24,6 +24,8 @@ from dataclasses import dataclass
 import numpy as np
 import torch
 
+from .. import native
+
 
 @dataclass
 class Entry:
@@ -65,88 +67,82 @@ class StepBatch:
         self.state_slots, self.logits_rows = d["state_slots"], d["logits_rows"]
         self.slot_mapping = [d["slot_mapping%d" % g] for g in range(len(max_blocks))]
         self.block_table = [d["block_table%d" % g] for g in range(len(max_blocks))]
+        # where the C++ core writes: addresses inside the pinned buffer
+        self._buffers = native.BatchBuffers()
+        bb = self._buffers
+        bb.n_groups, bb.max_tokens, bb.max_reqs, bb.max_rows = len(max_blocks), max_tokens, max_reqs, max_rows
+        for name in ("input_ids", "positions", "cu_seqlens", "seq_lens", "state_slots", "logits_rows"):
+            setattr(bb, name, self.h[name].ctypes.data)
+        for g, mb in enumerate(max_blocks):
+            bb.slot_mapping[g] = self.h["slot_mapping%d" % g].ctypes.data
+            bb.block_table[g] = self.h["block_table%d" % g].ctypes.data
+            bb.max_blocks[g] = mb
+        self._facts = native.BatchFacts()
         # host-side facts of the current step
         self.num_tokens = self.num_reqs = self.num_rows = 0
-        self.q_lens: list[int] = []
-        self.starts: list[int] = []
-        self.max_q_len = self.max_seq_len = 0
+        self.max_q_len = self.max_seq_len = self.num_singles = 0
         self.all_decode = False
         self.max_len_bound = 0
         self.req_ids: list = []
-        self.row_owner: list[tuple] = []  # (request index, token index) per logits row
         self._copied = torch.cuda.Event() if pin else None
 
+    @property
+    def q_lens(self) -> list[int]:
+        """Tokens per request of the current step (padding rows included)."""
+        return np.diff(self.h["cu_seqlens"][:self.num_reqs + 1]).tolist()
+
     def fill(self, entries: list[Entry], cache, pad_to: int | None = None) -> None:
-        """Writes the step into the pinned buffer from the entries and the cache manager's tables.
+        """Writes the step into the pinned buffer from the entries and the cache manager's tables
+        (csrc/host/step_batch.hpp does the writing).
 
         pad_to: for a step of single rows that replays a captured graph of that many requests, the
         batch is filled up with requests of one token at position 0 that write no cache slot
         (slot -1) and read page 0, which always exists (crates/layers/src/exec.rs:388-426).
         Their logits rows are computed and ignored."""
         B = len(entries)
-        T = sum(len(e.tokens) for e in entries)
-        R = sum(len(e.want) for e in entries)
-        if B == 0 or T == 0:
+        if B == 0:
             raise ValueError("a step needs at least one request with at least one token")
-        if B > self.max_reqs:
-            raise ValueError(f"{B} requests in one step, the engine was built for {self.max_reqs}")
-        if T > self.max_tokens:
-            raise ValueError(f"{T} tokens in one step, the engine was built for {self.max_tokens}")
-        if R > self.max_rows:
-            raise ValueError(f"logits wanted at {R} places, the engine was built for {self.max_rows}")
+        i32 = np.int32
+        rids = np.array([cache.handle(e.req_id) for e in entries], dtype=np.int64)
+        starts = np.array([e.start for e in entries], dtype=i32)
+        counts = np.array([len(e.tokens) for e in entries], dtype=i32)
+        want_counts = np.array([len(e.want) for e in entries], dtype=i32)
+        tokens = np.array([t for e in entries for t in e.tokens] or [0], dtype=i32)
+        wants = np.array([w for e in entries for w in e.want] or [0], dtype=i32)
+        self._wait_for_upload()
+        rc = native.fn("dh_batch_fill")(cache._h, self._buffers, B, rids.ctypes.data, starts.ctypes.data,
+                                        counts.ctypes.data, tokens.ctypes.data, want_counts.ctypes.data,
+                                        wants.ctypes.data, pad_to or 0, self._facts)
+        if rc < 0:
+            raise self._named(native.error(rc), [e.req_id for e in entries])
+        self.req_ids = [e.req_id for e in entries]
+        self._take_facts()
+
+    def fill_planned(self, scheduler, pad_to: int | None = None) -> None:
+        """The same for the step a scheduler has just planned, straight from the tokens it holds."""
+        self._wait_for_upload()
+        rc = native.fn("dh_sched_fill")(scheduler._h, self._buffers, pad_to or 0, self._facts)
+        if rc < 0:
+            raise self._named(native.error(rc), scheduler.planned_ids())
+        self.req_ids = scheduler.planned_ids()
+        self._take_facts()
+
+    @staticmethod
+    def _named(exc: Exception, ids: list) -> Exception:
+        """The core names an entry by its index; say which request that is."""
+        import re
+        msg = re.sub(r"entry (\d+)", lambda m: f"request {ids[int(m.group(1))]!r}", str(exc.args[0]))
+        return type(exc)(msg)
+
+    def _wait_for_upload(self) -> None:
         if self._copied is not None:
             self._copied.synchronize()  # the last upload has read the pinned buffer
-        h = self.h
-        t = r = 0
-        self.q_lens, self.starts, self.req_ids, self.row_owner = [], [], [], []
-        h["cu_seqlens"][0] = 0
-        for g in range(len(self.max_blocks)):
-            h["block_table%d" % g][:B].fill(-1)
-        for b, e in enumerate(entries):
-            n = len(e.tokens)
-            if n == 0:
-                raise ValueError(f"request {e.req_id!r} brings no token to this step")
-            h["input_ids"][t:t + n] = e.tokens
-            h["positions"][t:t + n] = np.arange(e.start, e.start + n, dtype=np.int32)
-            for g, mb in enumerate(self.max_blocks):
-                tab = cache.block_table(e.req_id, g)
-                if len(tab) > mb:
-                    raise ValueError(f"request {e.req_id!r} holds {len(tab)} pages, the block table has {mb} columns")
-                h["block_table%d" % g][b, :len(tab)] = tab
-                h["slot_mapping%d" % g][t:t + n] = cache.slot_mapping(e.req_id, g, e.start, n)
-            h["cu_seqlens"][b + 1] = t + n
-            h["seq_lens"][b] = e.start + n
-            h["state_slots"][b] = cache.slot_of(e.req_id)
-            for w in e.want:
-                if not (0 <= w < n):
-                    raise ValueError(f"request {e.req_id!r}: wanted place {w} is outside its {n} tokens")
-                h["logits_rows"][r] = t + w
-                self.row_owner.append((b, w))
-                r += 1
-            self.q_lens.append(n)
-            self.starts.append(e.start)
-            self.req_ids.append(e.req_id)
-            t += n
-        if pad_to is not None and pad_to > B:
-            if T != B or R != B or pad_to > self.max_reqs or pad_to > self.max_tokens or pad_to > self.max_rows:
-                raise ValueError("only a step of single rows that all want logits can be padded")
-            P = pad_to
-            h["input_ids"][B:P] = 0
-            h["positions"][B:P] = 0
-            h["cu_seqlens"][B + 1:P + 1] = np.arange(B + 1, P + 1, dtype=np.int32)
-            h["seq_lens"][B:P] = 1
-            h["state_slots"][B:P] = 0
-            h["logits_rows"][B:P] = np.arange(B, P, dtype=np.int32)
-            for g in range(len(self.max_blocks)):
-                h["block_table%d" % g][B:P].fill(0)
-                h["slot_mapping%d" % g][B:P] = -1
-            self.q_lens += [1] * (P - B)
-            self.starts += [0] * (P - B)
-            T = B = R = P
-        self.num_tokens, self.num_reqs, self.num_rows = T, B, R
-        self.max_q_len = max(self.q_lens)
-        self.max_seq_len = max(s + n for s, n in zip(self.starts, self.q_lens))
-        self.all_decode = all(n == 1 for n in self.q_lens)
+
+    def _take_facts(self) -> None:
+        f = self._facts
+        self.num_tokens, self.num_reqs, self.num_rows = f.num_tokens, f.num_reqs, f.num_rows
+        self.max_q_len, self.max_seq_len, self.num_singles = f.max_q_len, f.max_seq_len, f.num_singles
+        self.all_decode = f.num_singles == f.num_reqs
         # what kernels may assume about every seq_len of this step (a replayed graph fixes it to the model's limit)
         self.max_len_bound = self.max_seq_len
 

@@ -17,7 +17,6 @@ from dataclasses import dataclass
 from ..config import EngineOptions
 from ..sampling.params import SamplingParams
 from ..sampling.sampler import Sampler
-from .batch import Entry
 from .request import Request
 from .runner import ModelRunner
 from .scheduler import Scheduler
@@ -74,18 +73,12 @@ class Engine:
     def step(self) -> list[StepOutput]:
         so = self.scheduler.schedule()
         outs = [StepOutput(rid, None, True, reason) for rid, reason in so.force_finished]
-        if not so.scheduled:
+        if not len(so):
             return outs
-        entries, rows = [], []
-        for s in so.scheduled:
-            r = s.request
-            entries.append(Entry(r.id, r.tokens(s.start, s.num_new), s.start, [s.num_new - 1] if s.samples else []))
-            if s.samples:
-                rows.append((r.sampling, r.num_output, r.prompt_ids, r.output_ids, r.seed))
-        logits = self.runner.step(entries)
+        logits = self.runner.step_planned(self.scheduler, so)
+        rows = [(r.sampling, len(r.output_ids), r.prompt_ids, r.output_ids, r.seed) for r in so.sampling_requests()]
         tokens = self.sampler.sample(logits, rows)
-        sampled = {s.request.id: t for s, t in zip((s for s in so.scheduled if s.samples), tokens)}
-        for r, tok, reason in self.scheduler.update(so, sampled):
+        for r, tok, reason in self.scheduler.update(so, tokens):
             outs.append(StepOutput(r.id, tok, reason is not None, reason))
         return outs
 

@@ -156,12 +156,21 @@ class ModelRunner:
         """Runs one batch. Pages for every entry's tokens must have been allocated.
         Returns float32 logits [sum(len(e.want)), vocab] in the order of entries and of want
         (a view of a buffer that the next step overwrites)."""
+        single_rows = all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)
+        return self._run(len(entries), single_rows, lambda pad: self.batch.fill(entries, self.cache, pad_to=pad))
+
+    def step_planned(self, scheduler, plan) -> torch.Tensor:
+        """The same step function for the step a scheduler has just planned: the batch is written
+        straight from the tokens and tables the host core holds. Logits come back for the
+        requests of the plan that sample, in the plan's order."""
+        return self._run(len(plan), plan.single_rows_that_sample,
+                         lambda pad: self.batch.fill_planned(scheduler, pad_to=pad))
+
+    def _run(self, n: int, single_rows: bool, fill) -> torch.Tensor:
         b = self.batch
-        n = len(entries)
-        if (self.options.hip_graph and not self.state_tensors and n <= self._buckets[-1]
-                and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)):
-            return self._graph_step(entries)
-        b.fill(entries, self.cache)
+        if self.options.hip_graph and not self.state_tensors and single_rows and 0 < n <= self._buckets[-1]:
+            return self._graph_step(n, fill)
+        fill(None)
         b.upload()
         fresh = self.cache.take_fresh_slots()
         if fresh and self.state_tensors:
@@ -170,13 +179,13 @@ class ModelRunner:
                 st.index_fill_(0, idx, 0)
         return self.model.forward(b, self.cache_views)
 
-    def _graph_step(self, entries: list[Entry]) -> torch.Tensor:
+    def _graph_step(self, n: int, fill) -> torch.Tensor:
         """A step of single rows replays a HIP graph captured for its batch-size bucket
         (crates/layers/src/exec.rs:83-222, models/qwen3/src/executor.rs:995-1014). All step
         inputs live at fixed addresses; what varies between replays is their content."""
-        b, n = self.batch, len(entries)
+        b = self.batch
         bucket = next(x for x in self._buckets if x >= n)
-        b.fill(entries, self.cache, pad_to=bucket)
+        fill(bucket)
         b.max_len_bound = self.options.max_model_len  # the graph must hold for every later length
         b.upload()
         self.cache.take_fresh_slots()

@@ -1,6 +1,8 @@
 """Continuous batching: admits requests, cuts prompts into portions under a token
-budget, decodes, finishes and frees. Pure host code; it sees the cache only through
-the cache manager. The rules are the reference's (crates/core/src/sched/mod.rs):
+budget, decodes, finishes and frees. The decisions are made by the C++ class of
+csrc/host/scheduler.hpp, which sees the cache only through the cache manager; this
+front keeps the Python-side request objects and turns plans into Python values.
+The rules are the reference's (crates/core/src/sched/mod.rs):
 
   * no separate prefill and decode phases: each step a request gets
     min(tokens it still has to compute, what the budget allows) tokens (:1-11,377);
@@ -19,12 +21,20 @@ the cache manager. The rules are the reference's (crates/core/src/sched/mod.rs):
 """
 from __future__ import annotations
 
-from collections import deque
-from dataclasses import dataclass, field
+import ctypes
+from dataclasses import dataclass
 
+import numpy as np
+
+from .. import native
 from ..cache import CacheManager
 from ..config import EngineOptions
-from .request import FINISHED, LENGTH, PREEMPTED, RUNNING, STOP, WAITING, ABORT, Request
+from .request import REASON_NAMES, Request
+
+_SCHEDULED = np.dtype([("id", "<i8"), ("start", "<i4"), ("num_new", "<i4"), ("samples", "<i4")], align=True)
+_RESULT = np.dtype([("id", "<i8"), ("token", "<i4"), ("reason", "<i4")], align=True)
+assert _SCHEDULED.itemsize == ctypes.sizeof(native.Scheduled) and _RESULT.itemsize == ctypes.sizeof(native.UpdateResult)
+_INT32_MAX = 2**31 - 1
 
 
 @dataclass
@@ -35,24 +45,60 @@ class ScheduledRequest:
     samples: bool    # the step reaches the end of the known tokens, so a token is sampled
 
 
-@dataclass
 class SchedulerOutput:
-    scheduled: list = field(default_factory=list)      # [ScheduledRequest], running first then newly admitted
-    preempted: list = field(default_factory=list)      # request ids preempted while scheduling
-    force_finished: list = field(default_factory=list) # [(id, reason)] ended by the scheduler itself
+    """One planned step. `rows` is the plan as the core wrote it (id, start, num_new, samples)."""
+
+    def __init__(self, rows: np.ndarray, requests: list, preempted: list, force_finished: list):
+        self.rows = rows
+        self.requests = requests              # the Request of every row, running first then newly admitted
+        self.preempted = preempted            # request ids preempted while scheduling
+        self.force_finished = force_finished  # [(id, reason)] ended by the scheduler itself
+        self._scheduled = None
+
+    @property
+    def scheduled(self) -> list:
+        if self._scheduled is None:
+            self._scheduled = [ScheduledRequest(r, int(x["start"]), int(x["num_new"]), bool(x["samples"]))
+                               for r, x in zip(self.requests, self.rows)]
+        return self._scheduled
+
+    def __len__(self) -> int:
+        return len(self.requests)
 
     @property
     def total_tokens(self) -> int:
-        return sum(s.num_new for s in self.scheduled)
+        return int(self.rows["num_new"].sum())
+
+    @property
+    def single_rows_that_sample(self) -> bool:
+        """Every request feeds one token and samples: the shape of a step that a captured graph replays."""
+        return bool(len(self.rows)) and bool((self.rows["num_new"] == 1).all() and self.rows["samples"].all())
+
+    def sampling_requests(self) -> list:
+        return [r for r, s in zip(self.requests, self.rows["samples"].tolist()) if s]
 
 
 class Scheduler:
     def __init__(self, options: EngineOptions, cache: CacheManager, eos_token_ids=()):
         self.opt, self.cache = options, cache
         self.eos = set(eos_token_ids)
-        self.waiting: deque[Request] = deque()
-        self.running: list[Request] = []
-        self.requests: dict = {}
+        o = native.SchedOptions(options.max_num_batched_tokens, options.max_num_seqs, options.max_model_len,
+                                options.prefill_tokens_per_step or 0, options.long_prefill_token_threshold or 0,
+                                int(options.enable_chunked_prefill), int(options.decode_exempt_from_budget))
+        eos = np.array(sorted(self.eos) or [0], dtype=np.int32)
+        self._h = native.created("dh_sched_create", o, cache._h, eos.ctypes.data, len(self.eos))
+        self.requests: dict = {}        # id -> Request, for every request that is not finished
+        self._by_number: dict = {}      # the core's number -> Request
+        self._info = native.RequestInfo()
+        self._counts = (ctypes.c_int32 * 3)()
+        cap = options.max_num_seqs
+        self._results = np.zeros(cap, dtype=_RESULT)
+        self._planned: list = []
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            native.fn("dh_sched_destroy")(h)
 
     # ---- intake --------------------------------------------------------------------------------
     def add_request(self, req: Request) -> None:
@@ -60,153 +106,104 @@ class Scheduler:
             raise KeyError(f"request id {req.id!r} is in use")
         if not req.prompt_ids:
             raise ValueError("a prompt needs at least one token")
-        if req.num_prompt >= self.opt.max_model_len:
-            raise ValueError(f"prompt of {req.num_prompt} tokens leaves no room for output within "
-                             f"max_model_len {self.opt.max_model_len}")
-        req.sampling.validate()
-        req.status = WAITING
+        sp = req.sampling
+        sp.validate()
+        prompt = np.array(req.prompt_ids, dtype=np.int32)
+        stop = np.array(list(sp.stop_token_ids) or [0], dtype=np.int32)
+        number = self.cache.handle(req.id, create=True, pin=True)
+        try:
+            native.checked("dh_sched_add", self._h, number, prompt.ctypes.data, len(prompt),
+                           min(sp.max_tokens, _INT32_MAX), sp.min_tokens, int(sp.ignore_eos), stop.ctypes.data,
+                           len(sp.stop_token_ids))
+        except Exception:
+            self.cache.forget(req.id)
+            raise
+        req._owner = self
+        req._number = number
         self.requests[req.id] = req
-        self.waiting.append(req)
+        self._by_number[number] = req
 
     def has_unfinished(self) -> bool:
-        return bool(self.waiting or self.running)
+        return bool(native.fn("dh_sched_has_unfinished")(self._h))
 
     def abort(self, req_id) -> None:
         req = self.requests.get(req_id)
         if req is None:
             return
-        self._finish(req, ABORT)
+        native.checked("dh_sched_abort", self._h, req._number)
+        self._release(req)
+
+    def request_info(self, req: Request):
+        native.checked("dh_sched_request_info", self._h, req._number, self._info)
+        return self._info
+
+    @property
+    def waiting(self) -> list:
+        return self._queue(0)
+
+    @property
+    def running(self) -> list:
+        return self._queue(1)
+
+    def _queue(self, running: int) -> list:
+        cap = len(self.requests)
+        out = np.zeros(max(cap, 1), dtype=np.int64)
+        n = native.fn("dh_sched_queue")(self._h, running, out.ctypes.data, cap)
+        return [self._by_number[h] for h in out[:n].tolist()]
 
     # ---- one step ------------------------------------------------------------------------------
     def schedule(self) -> SchedulerOutput:
-        opt, out = self.opt, SchedulerOutput()
-        budget = opt.max_num_batched_tokens
-        quota = opt.prefill_tokens_per_step or (1 << 62)
-        eligible = len(self.running) + len(self.waiting)
-        threshold = opt.long_prefill_token_threshold if eligible > 1 else 0
-        preempted_any = False
+        native.checked("dh_sched_schedule", self._h, self._counts)
+        n, n_pre, n_fin = self._counts
+        rows = np.zeros(n, dtype=_SCHEDULED)
+        pre = np.zeros(max(n_pre, 1), dtype=np.int64)
+        fin = np.zeros(max(n_fin, 1), dtype=np.int64)
+        why = np.zeros(max(n_fin, 1), dtype=np.int32)
+        native.fn("dh_sched_plan")(self._h, rows.ctypes.data, pre.ctypes.data, fin.ctypes.data, why.ctypes.data)
+        by = self._by_number
+        requests = [by[h] for h in rows["id"].tolist()]
+        preempted = [by[h].id for h in pre[:n_pre].tolist()]
+        forced = []
+        for h, reason in zip(fin[:n_fin].tolist(), why[:n_fin].tolist()):
+            r = by[h]
+            forced.append((r.id, REASON_NAMES[reason]))
+            self._release(r)
+        self._planned = requests
+        return SchedulerOutput(rows, requests, preempted, forced)
 
-        i = 0
-        while i < len(self.running):
-            r = self.running[i]
-            remaining = r.num_tokens - r.num_computed
-            is_decode = remaining == 1 and r.num_computed > 0
-            charged = not (opt.decode_exempt_from_budget and is_decode)
-            if charged and budget == 0:
-                break
-            n = remaining
-            if threshold and n > threshold:
-                n = threshold
-            if charged:
-                n = min(n, budget)
-            if not is_decode:
-                n = min(n, quota)
-            if n < remaining and not opt.enable_chunked_prefill:
-                n = 0
-            if n <= 0:
-                i += 1
-                continue
-            got = False
-            while True:
-                if self.cache.allocate(r.id, r.num_computed, n):
-                    got = True
-                    break
-                victim = self.running[-1]
-                if victim is r:
-                    if len(self.running) > 1:
-                        break  # others hold the pages; try again next step, never preempt oneself
-                    self._finish(r, LENGTH)  # alone and still no page: the pool cannot hold it
-                    out.force_finished.append((r.id, LENGTH))
-                    break
-                self.running.pop()
-                self._preempt(victim)
-                out.preempted.append(victim.id)
-                preempted_any = True
-            if not got:
-                break
-            out.scheduled.append(ScheduledRequest(r, r.num_computed, n, r.num_computed + n == r.num_tokens))
-            if charged:
-                budget -= n
-            if not is_decode:
-                quota -= n
-            i += 1
+    def planned_ids(self) -> list:
+        return [r.id for r in self._planned]
 
-        if not preempted_any:
-            while budget > 0 and self.waiting and len(self.running) < opt.max_num_seqs:
-                r = self.waiting[0]
-                remaining = r.num_tokens - r.num_computed
-                n = remaining
-                if threshold and n > threshold:
-                    n = threshold
-                n = min(n, budget, quota)
-                if n < remaining and not opt.enable_chunked_prefill:
-                    n = 0
-                if n <= 0:
-                    break
-                if not self.cache.can_admit():
-                    break
-                self.cache.admit(r.id)
-                if not self.cache.allocate(r.id, r.num_computed, n):
-                    self.cache.free(r.id)  # no pages now: wait
-                    break
-                self.waiting.popleft()
-                r.status = RUNNING
-                self.running.append(r)
-                out.scheduled.append(ScheduledRequest(r, r.num_computed, n, r.num_computed + n == r.num_tokens))
-                budget -= n
-                quota -= n
-
-        for s in out.scheduled:  # advance at once, as the reference does after scheduling (:646-670)
-            s.request.num_computed += s.num_new
-        return out
-
-    def update(self, out: SchedulerOutput, sampled: dict) -> list:
-        """sampled: request id -> token for the scheduled requests that sample.
-        Returns [(request, new token or None, finish reason or None)] for every scheduled request."""
+    def update(self, out: SchedulerOutput, sampled) -> list:
+        """sampled: request id -> token for the scheduled requests that sample, or the tokens alone
+        in the order of those requests. Returns [(request, new token or None, finish reason or None)]
+        for every scheduled request that is still running."""
+        if isinstance(sampled, dict):
+            sampled = [sampled[r.id] for r in out.sampling_requests()]
+        toks = np.array(list(sampled) or [0], dtype=np.int32)
+        if len(self._results) < len(out):
+            self._results = np.zeros(len(out), dtype=_RESULT)
+        n = native.checked("dh_sched_update", self._h, toks.ctypes.data, len(sampled), self._results.ctypes.data,
+                           len(self._results))
+        res = self._results[:n]
         results = []
-        for s in out.scheduled:
-            r = s.request
-            if r.status != RUNNING:
-                continue  # preempted later in the same schedule() call
-            self.cache.release_passed(r.id, r.num_computed)
-            tok = None
-            reason = None
-            if s.samples:
-                tok = int(sampled[r.id])
+        by = self._by_number
+        for h, tok, reason in zip(res["id"].tolist(), res["token"].tolist(), res["reason"].tolist()):
+            r = by[h]
+            if tok >= 0:
                 r.output_ids.append(tok)
-                reason = self._check_stop(r, tok)
-                if reason:
-                    self._finish(r, reason)
-            results.append((r, tok, reason))
+            else:
+                tok = None
+            if reason:
+                self._release(r)
+            results.append((r, tok, REASON_NAMES[reason]))
         return results
 
     # ---- internals -----------------------------------------------------------------------------
-    def _check_stop(self, r: Request, tok: int) -> str | None:
-        sp = r.sampling
-        if r.num_output >= sp.min_tokens:
-            if (not sp.ignore_eos and tok in self.eos) or tok in sp.stop_token_ids:
-                return STOP
-        if r.num_tokens >= self.opt.max_model_len or r.num_output >= sp.max_tokens:
-            return LENGTH
-        return None
-
-    def _preempt(self, r: Request) -> None:
-        self.cache.free(r.id)
-        r.num_computed = 0
-        r.status = PREEMPTED
-        r.num_preemptions += 1
-        self.waiting.appendleft(r)
-
-    def _finish(self, r: Request, reason: str) -> None:
-        if r.status == FINISHED:
-            return
-        if self.cache.has(r.id):
-            self.cache.free(r.id)
-        if r in self.running:
-            self.running.remove(r)
-        try:
-            self.waiting.remove(r)
-        except ValueError:
-            pass
-        r.status, r.finish_reason = FINISHED, reason
-        self.requests.pop(r.id, None)
+    def _release(self, req: Request) -> None:
+        """A finished request: keep its last state on the Python object, drop it from the core."""
+        req._detach(self.request_info(req))
+        native.checked("dh_sched_forget", self._h, req._number)
+        self.requests.pop(req.id, None)
+        self._by_number.pop(req._number, None)
+        self.cache.forget(req.id)

@@ -42,7 +42,7 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k_cache, v_cache, batc
     B, T = batch.num_reqs, batch.num_tokens
     if not ws.mfma:
         return ops.attn_paged_ref(qkv, out, k_cache, v_cache, bt, batch.cu_seqlens, batch.seq_lens, B, T, **geo)
-    singles = sum(1 for n in batch.q_lens if n == 1) if ws.split_k else 0
+    singles = batch.num_singles if ws.split_k else 0
     # a few single rows beside long portions are not worth two more launches
     use_decode = singles == B or singles >= 4
     if use_decode:

@@ -122,9 +122,9 @@ def test_engine_loop_with_a_stand_in_runner():
             self.cache = CacheManager([GroupSpec(4, 32)], 3)
             self.model, self.device, self.max_rows, self.steps = FakeModel, torch.device("cpu"), 3, []
 
-        def step(self, entries):
-            self.steps.append([(e.req_id, len(e.tokens), e.start) for e in entries])
-            rows = [(e.start + len(e.tokens)) % 50 for e in entries for _ in e.want]
+        def step_planned(self, scheduler, plan):
+            self.steps.append([(x.request.id, x.num_new, x.start) for x in plan.scheduled])
+            rows = [(x.start + x.num_new) % 50 for x in plan.scheduled if x.samples]
             return torch.nn.functional.one_hot(torch.tensor(rows, dtype=torch.long), 50).float()
 
     class FakeSampler:
@@ -140,3 +140,33 @@ def test_engine_loop_with_a_stand_in_runner():
     assert eng.runner.cache.num_free() == 32 and not eng.has_unfinished()
     outs = eng.generate([[5] * 47], SamplingParams(max_tokens=10, temperature=0.0))
     assert outs == [[47, 48, 49]]                                           # 49 is eos
+
+
+def test_planned_fill_writes_what_the_entries_would():
+    """The scheduler's plan written straight from the core's tokens equals the same step given as entries."""
+    import numpy as np
+    opt = EngineOptions(max_num_seqs=4, max_num_batched_tokens=12, block_size=4, max_model_len=64, num_blocks=40)
+    cache = CacheManager([GroupSpec(4, 40), GroupSpec(4, 40, 6)], 4)
+    s = Scheduler(opt, cache, eos_token_ids=[])
+    mk = lambda: StepBatch(torch.device("cpu"), 16, 4, 4, [16, 16])
+    a, b = mk(), mk()
+    for i, n in enumerate((9, 3, 14)):
+        s.add_request(Request(i, [100 * i + j for j in range(n)], SamplingParams(max_tokens=4)))
+    for step in range(8):
+        out = s.schedule()
+        if not len(out):
+            break
+        a.fill_planned(s)
+        entries = [Entry(x.request.id, x.request.tokens(x.start, x.num_new), x.start, [x.num_new - 1] if x.samples else [])
+                   for x in out.scheduled]
+        b.fill(entries, cache)
+        assert (a.num_tokens, a.num_reqs, a.num_rows, a.max_q_len, a.max_seq_len, a.num_singles, a.req_ids) == \
+               (b.num_tokens, b.num_reqs, b.num_rows, b.max_q_len, b.max_seq_len, b.num_singles, b.req_ids)
+        T, B, R = a.num_tokens, a.num_reqs, a.num_rows
+        for name, n in (("input_ids", T), ("positions", T), ("slot_mapping0", T), ("slot_mapping1", T),
+                        ("cu_seqlens", B + 1), ("seq_lens", B), ("state_slots", B), ("logits_rows", R),
+                        ("block_table0", B), ("block_table1", B)):
+            assert np.array_equal(a.h[name][:n], b.h[name][:n]), (step, name)
+        s.update(out, [7000 + step] * len(out.sampling_requests()))
+        cache.check()
+    assert step >= 5

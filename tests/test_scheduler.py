@@ -8,8 +8,8 @@ from dinfer_amd.sampling import SamplingParams
 
 
 def mk(max_seqs, budget, blocks, **kw):
-    opt = EngineOptions(max_num_seqs=max_seqs, max_num_batched_tokens=budget, block_size=16, max_model_len=4096,
-                        num_blocks=blocks, decode_exempt_from_budget=False, **kw)
+    kw = {"max_model_len": 4096, "decode_exempt_from_budget": False, **kw}
+    opt = EngineOptions(max_num_seqs=max_seqs, max_num_batched_tokens=budget, block_size=16, num_blocks=blocks, **kw)
     cache = CacheManager([GroupSpec(16, blocks)], max_seqs)
     return Scheduler(opt, cache, eos_token_ids=[2])
 
@@ -82,8 +82,7 @@ def test_step_that_preempted_admits_nobody():
 
 
 def test_decode_exempt_from_budget_coschedules_decode_and_prefill():
-    s = mk(4, 8, 64)
-    s.opt.decode_exempt_from_budget = True
+    s = mk(4, 8, 64, decode_exempt_from_budget=True)
     s.add_request(req(1, 4, 16))
     assert step(s, {1: 1})[0] == [(1, 4)]
     s.add_request(req(2, 20, 16))
@@ -151,8 +150,7 @@ def test_finish_reasons():
 
 
 def test_max_model_len_finishes_with_length():
-    s = mk(8, 1000, 32)
-    s.opt.max_model_len = 8
+    s = mk(8, 1000, 32, max_model_len=8)
     s.add_request(req(1, 6, 100))
     step(s, {1: 5})
     assert step(s, {1: 5})[2][0][2] == LENGTH        # 8 tokens reached
@@ -184,8 +182,9 @@ def test_max_num_seqs_limits_admission():
 
 
 def test_schedule_and_update_are_cheap_for_many_decode_rows():
-    """The reference gates 1024 decode requests at 200 us in Rust (crates/core/benches/scheduler.rs);
-    this host code is Python, so the gate here only guards against quadratic behaviour."""
+    """The reference gates 1024 decode requests at 200 us (crates/core/benches/scheduler.rs). The
+    decisions here are C++ too, but this gate times the Python front with them (one object per
+    request and step), so it is wider: 256 decode rows within 1 ms."""
     import time
     n = 256
     s = mk(n, 100000, n * 4)
@@ -197,4 +196,40 @@ def test_schedule_and_update_are_cheap_for_many_decode_rows():
     for _ in range(10):
         out = s.schedule()
         s.update(out, {i: 1 for i in range(n)})
-    assert (time.perf_counter() - t0) / 10 < 0.02
+    assert (time.perf_counter() - t0) / 10 < 0.001
+
+
+def test_random_loads_keep_every_rule():
+    """Random prompts, limits and arrival times against a tight pool: every step obeys the budget and
+    the request limit, only the last running request is ever preempted, nothing is lost in the cache,
+    and every request ends with exactly the outputs it was allowed."""
+    import random
+    preemptions = 0
+    for seed in range(6):
+        rng = random.Random(seed)
+        budget, max_seqs, blocks = rng.choice([8, 24, 64]), rng.choice([2, 3, 5]), rng.choice([6, 9, 14])
+        s = mk(max_seqs, budget, blocks, decode_exempt_from_budget=bool(seed % 2), max_model_len=blocks * 16)
+        todo = [req(i, rng.randrange(1, 60), rng.randrange(1, 30)) for i in range(12)]
+        todo = [r for r in todo if r.num_prompt + r.sampling.max_tokens <= blocks * 16 - 16]
+        everyone = list(todo)
+        steps = 0
+        while todo or s.has_unfinished():
+            steps += 1
+            assert steps < 5000
+            while todo and rng.random() < 0.4:
+                s.add_request(todo.pop())
+            running_before = [r.id for r in s.running]
+            out = s.schedule()
+            charged = sum(x.num_new for x in out.scheduled
+                          if not (s.opt.decode_exempt_from_budget and x.num_new == 1 and x.start > 0))
+            assert charged <= budget and len(s.running) <= max_seqs
+            assert out.preempted == running_before[len(running_before) - len(out.preempted):][::-1]
+            preemptions += len(out.preempted)
+            for x in out.scheduled:
+                assert x.start + x.num_new <= x.request.num_tokens and x.samples == (x.start + x.num_new == x.request.num_tokens)
+            s.update(out, {x.request.id: 3 for x in out.scheduled if x.samples})
+            s.cache.check()
+        for r in everyone:
+            assert r.status == "finished" and r.finish_reason == LENGTH and r.num_output == r.sampling.max_tokens, r
+        assert s.cache.num_free() == blocks and not s.requests
+    assert preemptions > 10
