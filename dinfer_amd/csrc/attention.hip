@@ -48,12 +48,17 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
+// 2^x by the hardware instruction alone: results below 2^-126 become 0, which a softmax weight may
+__device__ __forceinline__ float exp2_raw(float x) { return __builtin_amdgcn_exp2f(x); }
+
 __device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
 
 // Block-table entries of 64 consecutive pages of one request, one per lane; a lane gets the
 // entry it needs by a cross-lane read, so no key block waits for a table load of its own.
+// P2: the page size is a power of two (shifts and masks instead of divisions).
+template <bool P2>
 struct Pages {
   const int32_t* bt;
   int max_blocks, base, reg, ps, ps_shift;
@@ -62,11 +67,11 @@ struct Pages {
     bt = table;
     max_blocks = max_blocks_;
     ps = page_size;
-    ps_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
+    ps_shift = P2 ? __builtin_ctz(page_size) : 0;
     fetch(page_of(first_key));
   }
-  __device__ __forceinline__ int page_of(int key) const { return ps_shift >= 0 ? key >> ps_shift : key / ps; }
-  __device__ __forceinline__ int offset_of(int key) const { return ps_shift >= 0 ? key & (ps - 1) : key % ps; }
+  __device__ __forceinline__ int page_of(int key) const { return P2 ? key >> ps_shift : key / ps; }
+  __device__ __forceinline__ int offset_of(int key) const { return P2 ? key & (ps - 1) : key % ps; }
   __device__ __forceinline__ void fetch(int first_page) {
     base = first_page;
     const int i = base + (int)(threadIdx.x & 63);
@@ -93,12 +98,12 @@ struct Frags {
 //   k_lo, k_hi  the keys this wave may touch at all (held pages, written slots)
 // load() issues the loads of one block, compute() consumes them; walk() keeps the next block's
 // loads in flight while the current one is computed.
-template <int DT, int NT>
+template <int DT, int NT, bool P2>
 struct Tile {
   static constexpr int KS = (DT + 1) / 2;  // 32-wide steps over the head dimension
   f32x4 o[NT][DT];
   float m[NT], l[NT];
-  Pages pages;
+  Pages<P2> pages;
   const bf16* kc;
   const bf16* vc;
   int hk, Hkv, k_lo, k_hi;
@@ -131,15 +136,18 @@ struct Tile {
     key0 = key0 < k_lo ? k_lo : (key0 > last ? last : key0);
     key1 = key1 < k_lo ? k_lo : (key1 > last ? last : key1);
     const int pg0 = pages.get(pages.page_of(key0)), pg1 = pages.get(pages.page_of(key1));
-    const bf16* kr0 = kc + (((int64_t)pg0 * Hkv + hk) * ps + pages.offset_of(key0)) * D;
-    const bf16* kr1 = kc + (((int64_t)pg1 * Hkv + hk) * ps + pages.offset_of(key1)) * D;
+    // K pages are [Hkv][D / 8][page][8]: the 16-byte pieces of consecutive keys lie next to each other,
+    // so the four lanes of a quad (four consecutive keys, one piece index) read 64 contiguous bytes
+    const bf16* kr0 = kc + ((int64_t)pg0 * Hkv + hk) * ps * D + pages.offset_of(key0) * 8;
+    const bf16* kr1 = kc + ((int64_t)pg1 * Hkv + hk) * ps * D + pages.offset_of(key1) * 8;
+    const int piece = ps * 8;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      int d = ks * 32 + g4 * 8;
-      const bool dv = d < D;  // D % 32 == 16: the upper half of the last step is padding
-      if (!dv) d = 0;
-      f.k[0][ks] = *(const bf16x8*)(kr0 + d);
-      f.k[1][ks] = *(const bf16x8*)(kr1 + d);
+      int c = ks * 4 + g4;
+      const bool dv = c * 8 < D;  // D % 32 == 16: the upper half of the last step is padding
+      if (!dv) c = 0;
+      f.k[0][ks] = *(const bf16x8*)(kr0 + c * piece);
+      f.k[1][ks] = *(const bf16x8*)(kr1 + c * piece);
       if (DT % 2 == 1 && ks == KS - 1 && !dv) f.k[0][ks] = f.k[1][ks] = zero8();
     }
     // V^T rows of this lane: d = 16 dt + i16, keys kg .. kg + 7 (one page)
@@ -152,8 +160,11 @@ struct Tile {
     for (int d = 0; d < DT; ++d) f.v[d] = *(const bf16x8*)(vrow + (int64_t)d * 16 * ps);
   }
 
+  // MASK: some key of the block is invisible to some column, or lies outside [k_lo, k_hi)
+  template <bool MASK>
   __device__ __forceinline__ void compute(const Frags<DT>& f, const bf16x8 (&qf)[NT][KS], int kb,
-                                          const int (&col_lo)[NT], const int (&col_hi)[NT], bool need_mask) {
+                                          const int (&col_lo)[NT], const int (&col_hi)[NT]) {
+    constexpr bool need_mask = MASK;
     const int lane = threadIdx.x & 63, g4 = lane >> 4;
     f32x4 s[NT][2];
 #pragma unroll
@@ -194,14 +205,14 @@ struct Tile {
       float ps_ = 0.f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float p = exp2f(fmaf(x[e], scale_log2e, -mc));
+        const float p = exp2_raw(fmaf(x[e], scale_log2e, -mc));
         ps_ += p;
         pf[t][e] = (bf16)p;
       }
       // the maximum rarely moves after the first blocks; the output is rescaled only when it did for
       // some column of the wave (a uniform branch)
       if (__any(m_new > m[t])) {
-        const float alpha = exp2f(fmaf(m[t], scale_log2e, -mc));  // m = -inf: 0
+        const float alpha = exp2_raw(fmaf(m[t], scale_log2e, -mc));  // m = -inf: 0
         l[t] *= alpha;
 #pragma unroll
         for (int d = 0; d < DT; ++d) o[t][d] *= alpha;
@@ -227,7 +238,9 @@ struct Tile {
   // All key blocks of [k_lo, k_hi); mask(kb) says whether block kb needs per-key masking.
   // PREFETCH: the next block's loads are issued before the current block is computed (two sets of
   // fragments in registers); without it one set, and latency is hidden by more waves per SIMD.
-  template <bool PREFETCH, class MaskFn>
+  // TWO_BODIES: blocks that need no masking run a body without it (more code and registers, fewer
+  // instructions per block); otherwise every block runs the masking body.
+  template <bool PREFETCH, bool TWO_BODIES, class MaskFn>
   __device__ __forceinline__ void walk(const bf16x8 (&qf)[NT][KS], const int (&col_lo)[NT], const int (&col_hi)[NT],
                                        MaskFn mask) {
     int kb = k_lo & ~31;
@@ -236,7 +249,10 @@ struct Tile {
       for (; kb < k_hi; kb += 32) {
         Frags<DT> f;
         load(f, kb);
-        compute(f, qf, kb, col_lo, col_hi, mask(kb));
+        if (!TWO_BODIES || mask(kb))
+          compute<true>(f, qf, kb, col_lo, col_hi);
+        else
+          compute<false>(f, qf, kb, col_lo, col_hi);
       }
       return;
     }
@@ -245,11 +261,11 @@ struct Tile {
     while (true) {
       const bool more1 = kb + 32 < k_hi;
       if (more1) load(f1, kb + 32);
-      compute(f0, qf, kb, col_lo, col_hi, mask(kb));
+      if (!TWO_BODIES || mask(kb)) compute<true>(f0, qf, kb, col_lo, col_hi); else compute<false>(f0, qf, kb, col_lo, col_hi);
       if (!more1) break;
       const bool more2 = kb + 64 < k_hi;
       if (more2) load(f0, kb + 64);
-      compute(f1, qf, kb + 32, col_lo, col_hi, mask(kb + 32));
+      if (!TWO_BODIES || mask(kb + 32)) compute<true>(f1, qf, kb + 32, col_lo, col_hi); else compute<false>(f1, qf, kb + 32, col_lo, col_hi);
       if (!more2) break;
       kb += 64;
     }
@@ -269,7 +285,7 @@ struct Tile {
 // beat 16 (more waves, 168 us) and 64 (one wave per SIMD, 182 us).
 constexpr bool FLASH_PREFETCH = false;
 
-template <int DT, int QT>
+template <int DT, int QT, bool P2>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) attn_flash_kernel(
     const bf16* __restrict__ q, int64_t ld_q, bf16* __restrict__ out, int64_t ld_out, const bf16* __restrict__ kc,
     const bf16* __restrict__ vc, const int32_t* __restrict__ block_table, int64_t max_blocks,
@@ -317,9 +333,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))
   const int k_hi = p_last + 1;
   const int k_lo = window > 0 ? (p_first - window + 1 > 0 ? p_first - window + 1 : 0) : 0;
 
-  Tile<DT, QT> tl;
+  Tile<DT, QT, P2> tl;
   tl.init(kc, vc, bt, (int)max_blocks, hk, Hkv, ps, k_lo, k_hi, scale_log2e);
-  tl.template walk<FLASH_PREFETCH>(qf, col_lo, col_hi, [&](int kb) {
+  tl.template walk<FLASH_PREFETCH, true>(qf, col_lo, col_hi, [&](int kb) {
     return kb + 31 > p_first || kb < k_lo || (window > 0 && kb < p_last - window + 1);
   });
 #pragma unroll
@@ -353,7 +369,7 @@ __device__ __forceinline__ void split_range(int seq, int window, int splits, int
 }
 
 // One wave per (split, kv head, request). part: [B, H, splits, D + 4] float = (m in base-2 units, l, -, -, o[D]).
-template <int DT>
+template <int DT, bool P2>
 __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 8))) attn_decode_kernel(
     const bf16* __restrict__ q, int64_t ld_q, float* __restrict__ part, const bf16* __restrict__ kc,
     const bf16* __restrict__ vc, const int32_t* __restrict__ block_table, int64_t max_blocks,
@@ -385,9 +401,9 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 8)))
     }
   }
   const int col_lo[1] = {k_lo}, col_hi[1] = {k_hi};
-  Tile<DT, 1> tl;
+  Tile<DT, 1, P2> tl;
   tl.init(kc, vc, bt, (int)max_blocks, hk, Hkv, ps, k_lo, k_hi, scale_log2e);
-  tl.template walk<false>(qf, col_lo, col_hi, [&](int kb) { return kb < k_lo || kb + 32 > k_hi; });
+  tl.template walk<false, false>(qf, col_lo, col_hi, [&](int kb) { return kb < k_lo || kb + 32 > k_hi; });
   const float lt = tl.sum_l(0);
   if (i16 < G) {
     float* pp = part + (((int64_t)b * H + hk * G + i16) * splits + sp) * (D + 4);
@@ -460,15 +476,17 @@ int launch_flash(const bf16* q, int64_t ld_q, bf16* out, int64_t ld_out, const b
     const int tiles = (max_q_len + QB - 1) / QB;
     const int64_t blocks = (int64_t)tiles * H * num_reqs;
     if (blocks > 0x7fffffff) return ERR_UNSUPPORTED;
-    attn_flash_kernel<DT, 2><<<(unsigned)blocks, 256, 0, stream>>>(q, ld_q, out, ld_out, kc, vc, bt, max_blocks, cu, sl,
-                                                                  tiles, sl2, window, H, Hkv, ps, skip_single);
+    auto kernel = (ps & (ps - 1)) == 0 ? attn_flash_kernel<DT, 2, true> : attn_flash_kernel<DT, 2, false>;
+    kernel<<<(unsigned)blocks, 256, 0, stream>>>(q, ld_q, out, ld_out, kc, vc, bt, max_blocks, cu, sl, tiles, sl2,
+                                                 window, H, Hkv, ps, skip_single);
   } else {
     constexpr int QB = 16 * 4;
     const int tiles = (max_q_len + QB - 1) / QB;
     const int64_t blocks = (int64_t)tiles * H * num_reqs;
     if (blocks > 0x7fffffff) return ERR_UNSUPPORTED;
-    attn_flash_kernel<DT, 1><<<(unsigned)blocks, 256, 0, stream>>>(q, ld_q, out, ld_out, kc, vc, bt, max_blocks, cu, sl,
-                                                                  tiles, sl2, window, H, Hkv, ps, skip_single);
+    auto kernel = (ps & (ps - 1)) == 0 ? attn_flash_kernel<DT, 1, true> : attn_flash_kernel<DT, 1, false>;
+    kernel<<<(unsigned)blocks, 256, 0, stream>>>(q, ld_q, out, ld_out, kc, vc, bt, max_blocks, cu, sl, tiles, sl2,
+                                                 window, H, Hkv, ps, skip_single);
   }
   return launch_status();
 }
@@ -477,7 +495,8 @@ template <int DT>
 int launch_decode(const bf16* q, int64_t ld_q, bf16* out, int64_t ld_out, float* part, const bf16* kc, const bf16* vc,
                   const int32_t* bt, int64_t max_blocks, const int32_t* cu, const int32_t* sl, int num_reqs,
                   int splits, float scale, int window, int H, int Hkv, int ps, hipStream_t stream) {
-  attn_decode_kernel<DT><<<dim3((unsigned)splits, (unsigned)Hkv, (unsigned)num_reqs), 64, 0, stream>>>(
+  auto kernel = (ps & (ps - 1)) == 0 ? attn_decode_kernel<DT, true> : attn_decode_kernel<DT, false>;
+  kernel<<<dim3((unsigned)splits, (unsigned)Hkv, (unsigned)num_reqs), 64, 0, stream>>>(
       q, ld_q, part, kc, vc, bt, max_blocks, cu, sl, splits, scale * LOG2E, window, H, Hkv, ps);
   const int D = DT * 16;
   attn_decode_merge_kernel<<<dim3((unsigned)H, (unsigned)num_reqs), 64, 0, stream>>>(part, out, ld_out, cu, sl, splits,

@@ -67,9 +67,10 @@ __global__ void __launch_bounds__(WAVES * 64) attn_paged_ref_kernel(
     float s = -INFINITY;
     if (live && j <= p) {
       const int blk = bt[j / page];
-      const S* kr = k_cache + (((int64_t)blk * Hkv + hk) * page + (j % page)) * D;
+      const S* kr = k_cache + ((int64_t)blk * Hkv + hk) * page * D;  // the head's page
+      const int off = j % page;
       float acc = 0.f;
-      for (int d = 0; d < D; ++d) acc += qs[wave][d] * to_f32(kr[d]);
+      for (int d = 0; d < D; ++d) acc += qs[wave][d] * to_f32(kr[k_page_offset(off, d, page)]);
       s = acc * scale;
     }
     const float m_new = fmaxf(m, wave_max(s));

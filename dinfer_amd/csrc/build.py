@@ -70,19 +70,28 @@ def _hipcc() -> str:
     raise RuntimeError("hipcc not found: the HIP kernels cannot be built (looked in $HIPCC, PATH, /opt/rocm/bin)")
 
 
+_lib_dir: Path | None = None
+_lib_dir_lock = threading.Lock()
+
+
 def lib_dir() -> Path:
-    """Folder for built libraries: in the package if writable, else per-user temporary."""
-    d = PACKAGE / "_lib"
-    try:
-        d.mkdir(exist_ok=True)
-        probe = d / f".w{os.getpid()}"
-        probe.write_text("")
-        probe.unlink()
-        return d
-    except OSError:
-        alt = Path(tempfile.gettempdir()) / f"dinfer_amd_lib_{os.getuid()}"
-        alt.mkdir(parents=True, exist_ok=True)
-        return alt
+    """Folder for built libraries: in the package if writable, else per-user temporary.
+    Decided once per process (parallel builds must all land in the same folder)."""
+    global _lib_dir
+    with _lib_dir_lock:
+        if _lib_dir is None:
+            d = PACKAGE / "_lib"
+            try:
+                d.mkdir(exist_ok=True)
+                probe = d / f".w{os.getpid()}.{threading.get_ident()}"
+                probe.write_text("")
+                probe.unlink()
+                _lib_dir = d
+            except OSError:
+                alt = Path(tempfile.gettempdir()) / f"dinfer_amd_lib_{os.getuid()}"
+                alt.mkdir(parents=True, exist_ok=True)
+                _lib_dir = alt
+        return _lib_dir
 
 
 def source_hash(name: str) -> str:

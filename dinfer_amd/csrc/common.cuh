@@ -88,6 +88,13 @@ __device__ __forceinline__ float block_max(float v, float* red) {
 
 static inline int launch_status() { return hipGetLastError() == hipSuccess ? OK : ERR_LAUNCH; }
 
+// K pages. One kv head of one page is [D / 8][page][8]: the 8-element pieces of consecutive keys lie
+// next to each other, so lanes that read the same piece of consecutive keys (the rows of an MFMA
+// operand) read contiguous memory. Needs D % 8 == 0. Offset of element d of the key at `off`:
+__host__ __device__ __forceinline__ int64_t k_page_offset(int off, int d, int page) {
+  return ((int64_t)(d >> 3) * page + off) * 8 + (d & 7);
+}
+
 }  // namespace dinfer
 
 #define DINFER_DISPATCH_DTYPE(dtype, ...)         \

@@ -85,7 +85,7 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_kernel(
   __syncthreads();  // the rotation reads partners that other lanes wrote
   if (!is_qk) return;
 
-  S* kd = (!is_q && slot >= 0) ? k_cache + ((blk * Hkv + hk) * (int64_t)page + off) * D : nullptr;
+  S* kd = (!is_q && slot >= 0) ? k_cache + (blk * Hkv + hk) * (int64_t)page * D : nullptr;  // the head's page
   const float* cs = cos_sin ? cos_sin + (int64_t)pos[t] * rot : nullptr;
   const int half = rot / 2;
   for (int d = lane; d < D; d += 64) {
@@ -108,7 +108,7 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_kernel(
     }
     const S r = from_f32<S>(y);
     if (is_q) base[d] = r;
-    if (kd) kd[d] = r;
+    if (kd) kd[k_page_offset((int)off, d, page)] = r;
   }
 }
 
@@ -195,7 +195,7 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_neox_kernel(
     }
     const int hk = item - H;
     S* base = is_q ? row + q_off + (int64_t)item * D : nullptr;
-    S* kd = (!is_q && slot >= 0) ? k_cache + ((blk * Hkv + hk) * (int64_t)page + off) * D : nullptr;
+    S* kd = (!is_q && slot >= 0) ? k_cache + (blk * Hkv + hk) * (int64_t)page * D : nullptr;  // the head's page
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
       const int i = lane + 64 * p;
@@ -208,8 +208,8 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_neox_kernel(
           base[i + half] = r2;
         }
         if (kd) {
-          kd[i] = r1;
-          kd[i + half] = r2;
+          kd[k_page_offset((int)off, i, page)] = r1;
+          kd[k_page_offset((int)off, i + half, page)] = r2;
         }
       }
     }
@@ -303,7 +303,7 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_vec_kernel(
   if (is_q) {
     *(bf16x8*)(src + d0) = r;
   } else if (slot >= 0) {
-    *(bf16x8*)(k_cache + ((blk * Hkv + (item - H)) * (int64_t)page + off) * D + d0) = r;
+    *(bf16x8*)(k_cache + (blk * Hkv + (item - H)) * (int64_t)page * D + k_page_offset((int)off, d0, page)) = r;
   }
 }
 

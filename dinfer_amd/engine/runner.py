@@ -137,10 +137,9 @@ class ModelRunner:
                 self.cache_views.append(CacheView(src.group, src.k, src.v, owner=False, state=src.state))
                 continue
             if isinstance(need, KVSpec):
-                k = torch.empty((self.num_blocks, need.kv_heads, self.page_size, need.head_dim),
-                                dtype=self.dtype, device=self.device)
-                v = torch.empty((self.num_blocks, need.kv_heads, need.head_dim, self.page_size),
-                                dtype=self.dtype, device=self.device)
+                geometry = (self.num_blocks, need.kv_heads, self.page_size, need.head_dim)
+                k = torch.empty(ops.k_cache_shape(*geometry), dtype=self.dtype, device=self.device)
+                v = torch.empty(ops.v_cache_shape(*geometry), dtype=self.dtype, device=self.device)
                 view = CacheView(entry_group[i], k, v, owner=True)
             elif isinstance(need, StateSpec):
                 st = torch.zeros((opt.max_num_seqs, *need.shape), dtype=getattr(torch, need.dtype), device=self.device)

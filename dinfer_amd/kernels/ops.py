@@ -124,6 +124,38 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, eps: float
     return out
 
 
+# ---- cache page layouts ------------------------------------------------------------------------
+# K pages [blocks, kv_heads, D / 8, page, 8]: the 8-element pieces of consecutive keys are contiguous,
+# so the rows of an MFMA operand (consecutive keys, one piece) are read as contiguous memory.
+# V pages [blocks, kv_heads, D, page]: transposed, a row holds one dimension of a page's keys.
+def k_cache_shape(blocks: int, kv_heads: int, page_size: int, head_dim: int) -> tuple:
+    if head_dim % 8 != 0:
+        raise ValueError(f"head_dim {head_dim}: the cache stores keys in pieces of 8 elements")
+    return (blocks, kv_heads, head_dim // 8, page_size, 8)
+
+
+def v_cache_shape(blocks: int, kv_heads: int, page_size: int, head_dim: int) -> tuple:
+    return (blocks, kv_heads, head_dim, page_size)
+
+
+def k_cache_pack(rows: torch.Tensor) -> torch.Tensor:
+    """[blocks, kv_heads, page, D] (one row per key) -> the layout of K pages."""
+    nb, hkv, page, d = rows.shape
+    return rows.view(nb, hkv, page, d // 8, 8).permute(0, 1, 3, 2, 4).contiguous()
+
+
+def k_cache_rows(pages: torch.Tensor) -> torch.Tensor:
+    """The layout of K pages -> [blocks, kv_heads, page, D] (one row per key)."""
+    nb, hkv, pieces, page, _ = pages.shape
+    return pages.permute(0, 1, 3, 2, 4).reshape(nb, hkv, page, pieces * 8)
+
+
+def _check_pages(k_cache, v_cache, kv_heads, head_dim, page_size) -> None:
+    nb = k_cache.shape[0]
+    assert tuple(k_cache.shape) == k_cache_shape(nb, kv_heads, page_size, head_dim) and k_cache.is_contiguous()
+    assert tuple(v_cache.shape) == v_cache_shape(nb, kv_heads, page_size, head_dim) and v_cache.is_contiguous()
+
+
 def qkv_post(qkv: torch.Tensor, tokens: int, *, heads: int, kv_heads: int, head_dim: int, q_off: int, k_off: int,
              v_off: int, q_gain: torch.Tensor | None, k_gain: torch.Tensor | None, eps: float, gain_offset: float,
              positions: torch.Tensor, cos_sin: torch.Tensor | None, rotary_dim: int, rope_style: int,
@@ -131,8 +163,8 @@ def qkv_post(qkv: torch.Tensor, tokens: int, *, heads: int, kv_heads: int, head_
              page_size: int) -> None:
     """Per-head q/k norm, rotation, q written back in place, k and v written to the cache pages.
 
-    k_cache [blocks, kv_heads, page, D], v_cache [blocks, kv_heads, D, page]; slot_mapping int64 [T]
-    (None: nothing is written to the cache).
+    k_cache and v_cache in the page layouts above; slot_mapping int64 [T] (None: nothing is written
+    to the cache).
     """
     _need_gpu(qkv, q_gain, k_gain, positions, cos_sin, k_cache, v_cache, slot_mapping)
     ld = _rows(qkv)
@@ -149,9 +181,7 @@ def qkv_post(qkv: torch.Tensor, tokens: int, *, heads: int, kv_heads: int, head_
     if slot_mapping is not None:
         assert slot_mapping.dtype == torch.int64 and slot_mapping.numel() >= tokens
         assert k_cache is not None and v_cache is not None
-        nb = k_cache.shape[0]
-        assert tuple(k_cache.shape) == (nb, kv_heads, page_size, head_dim) and k_cache.is_contiguous()
-        assert tuple(v_cache.shape) == (nb, kv_heads, head_dim, page_size) and v_cache.is_contiguous()
+        _check_pages(k_cache, v_cache, kv_heads, head_dim, page_size)
         assert k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype
     lib.call("dinfer_qkv_post", dtype_code(qkv.dtype), qkv.data_ptr(), tokens, ld, q_off, k_off, v_off,
              _ptr(q_gain), _ptr(k_gain), wf32, float(eps), float(gain_offset), positions.data_ptr(), _ptr(cos_sin),
@@ -170,9 +200,7 @@ def attn_paged_ref(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_
     assert block_table.shape[0] >= num_reqs
     assert cu_seqlens.dtype == torch.int32 and cu_seqlens.numel() >= num_reqs + 1
     assert seq_lens.dtype == torch.int32 and seq_lens.numel() >= num_reqs
-    nb = k_cache.shape[0]
-    assert tuple(k_cache.shape) == (nb, kv_heads, page_size, head_dim) and k_cache.is_contiguous()
-    assert tuple(v_cache.shape) == (nb, kv_heads, head_dim, page_size) and v_cache.is_contiguous()
+    _check_pages(k_cache, v_cache, kv_heads, head_dim, page_size)
     assert q.shape[1] >= heads * head_dim and out.shape[1] >= heads * head_dim
     assert q.shape[0] >= tokens and out.shape[0] >= tokens
     lib.call("dinfer_attn_paged_ref", dtype_code(q.dtype), q.data_ptr(), _rows(q), out.data_ptr(), _rows(out),
@@ -190,9 +218,7 @@ def _check_paged(q, out, k_cache, v_cache, block_table, seq_lens, num_reqs, head
     assert q.dtype == out.dtype == k_cache.dtype == v_cache.dtype == torch.bfloat16
     assert block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous()
     assert block_table.shape[0] >= num_reqs and seq_lens.dtype == torch.int32 and seq_lens.numel() >= num_reqs
-    nb = k_cache.shape[0]
-    assert tuple(k_cache.shape) == (nb, kv_heads, page_size, head_dim) and k_cache.is_contiguous()
-    assert tuple(v_cache.shape) == (nb, kv_heads, head_dim, page_size) and v_cache.is_contiguous()
+    _check_pages(k_cache, v_cache, kv_heads, head_dim, page_size)
     assert q.shape[1] >= heads * head_dim and out.shape[1] >= heads * head_dim
 
 

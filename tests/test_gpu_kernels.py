@@ -103,7 +103,7 @@ def test_qkv_post(dtype, H, Hkv, D, page):
     pos = torch.tensor([0, 3, 7, 15, 31, 100], device=DEV, dtype=torch.int32)
     slots = torch.tensor([0, 1, 2, page + 1, page + 2, -1], device=DEV, dtype=torch.int64)  # the last token is not cached
     table = rope_table(128, D, theta).to(DEV)
-    kc = torch.zeros(nblocks, Hkv, page, D, device=DEV, dtype=dtype)
+    kc = torch.zeros(ops().k_cache_shape(nblocks, Hkv, page, D), device=DEV, dtype=dtype)
     vc = torch.zeros(nblocks, Hkv, D, page, device=DEV, dtype=dtype)
     qkv = qkv_in.clone()
     ops().qkv_post(qkv, T, heads=H, kv_heads=Hkv, head_dim=D, q_off=0, k_off=H * D, v_off=(H + Hkv) * D, q_gain=wq,
@@ -121,7 +121,7 @@ def test_qkv_post(dtype, H, Hkv, D, page):
         if s >= 0:
             want_k[s // page, :, s % page, :] = k[t]
             want_v[s // page, :, :, s % page] = v[t]
-    torch.testing.assert_close(kc.double().cpu(), want_k, **tol(dtype))
+    torch.testing.assert_close(ops().k_cache_rows(kc).double().cpu(), want_k, **tol(dtype))
     assert torch.equal(vc.double().cpu(), want_v)  # v is copied, not computed
 
 
@@ -182,7 +182,7 @@ def paged_case(dtype, H, Hkv, D, page, hist, new, seed=0, spike=None):
     cu = torch.tensor([0] + list(torch.tensor(new).cumsum(0)), dtype=torch.int32)
     meta = dict(bt=bt.to(DEV), cu=cu.to(DEV), sl=torch.tensor(total, dtype=torch.int32, device=DEV))
     q_all = torch.cat(qs).reshape(sum(new), H * D).to(DEV)
-    return q_all, kc.to(DEV), vc.to(DEV), meta, outs
+    return q_all, ops().k_cache_pack(kc).to(DEV), vc.to(DEV), meta, outs
 
 
 def expected_attention(outs, hist, scale, window):
@@ -455,7 +455,7 @@ def test_qkv_post_many_tokens_writes_v_transposed(start):
     slots[40] = -1
     slots_t = torch.tensor(slots, device=DEV, dtype=torch.int64)
     table = rope_table(128, D, 1e6).to(DEV)
-    kc = torch.zeros(nblocks, Hkv, page, D, device=DEV, dtype=torch.bfloat16)
+    kc = torch.zeros(ops().k_cache_shape(nblocks, Hkv, page, D), device=DEV, dtype=torch.bfloat16)
     vc = torch.zeros(nblocks, Hkv, D, page, device=DEV, dtype=torch.bfloat16)
     qkv = qkv_in.clone()
     ops().qkv_post(qkv, T, heads=H, kv_heads=Hkv, head_dim=D, q_off=0, k_off=H * D, v_off=(H + Hkv) * D, q_gain=None,
@@ -470,7 +470,7 @@ def test_qkv_post_many_tokens_writes_v_transposed(start):
     k = plain.rope_neox(qkv_in[:, H * D:(H + Hkv) * D].double().cpu().view(T, Hkv, D), plain.rope_angles(pos.tolist(), D, 1e6))
     for t, s in enumerate(slots):
         if s >= 0:
-            torch.testing.assert_close(kc[s // page, :, s % page, :].double().cpu(), k[t], rtol=2e-2, atol=2e-2)
+            torch.testing.assert_close(ops().k_cache_rows(kc)[s // page, :, s % page, :].double().cpu(), k[t], rtol=2e-2, atol=2e-2)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

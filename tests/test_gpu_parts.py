@@ -8,6 +8,7 @@ import pytest
 import torch
 
 import plain_qwen3 as plain
+from dinfer_amd.kernels import ops
 
 pytestmark = pytest.mark.gpu
 DEV = torch.device("cuda", 0)
@@ -105,7 +106,7 @@ def test_attention_part(dtype, window):
     mx.bind(context(dtype, page=page))
     lens = [13, 9]
     b = whole_batch(lens, page=page)
-    kc = torch.zeros(64, Hkv, page, D, device=DEV, dtype=dtype)
+    kc = torch.zeros(ops.k_cache_shape(64, Hkv, page, D), device=DEV, dtype=dtype)
     vc = torch.zeros(64, Hkv, D, page, device=DEV, dtype=dtype)
     x = torch.randn(64, Hd, device=DEV).to(dtype)
     out = mx.forward(x, b, CacheView(0, kc, vc, owner=True))[:sum(lens)].double().cpu()
@@ -137,7 +138,7 @@ def test_block_part(dtype):
     blk.bind(context(dtype, page=page))
     n = 10
     b = whole_batch([n], page=page)
-    kc = torch.zeros(64, Hkv, page, D, device=DEV, dtype=dtype)
+    kc = torch.zeros(ops.k_cache_shape(64, Hkv, page, D), device=DEV, dtype=dtype)
     vc = torch.zeros(64, Hkv, D, page, device=DEV, dtype=dtype)
     h0 = torch.randn(64, Hd, device=DEV).to(dtype)
     prev = torch.randn(64, Hd, device=DEV).to(dtype)       # the previous layer's branch, not yet added
