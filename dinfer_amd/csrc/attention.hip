@@ -107,11 +107,14 @@ struct Tile {
   const bf16* kc;
   const bf16* vc;
   int hk, Hkv, k_lo, k_hi;
+  int page_stride, head_off;  // elements from page to page, and from the page's start to this kv head
   float scale_log2e;
 
   __device__ __forceinline__ void init(const bf16* kc_, const bf16* vc_, const int32_t* bt, int max_blocks, int hk_,
                                        int Hkv_, int ps, int k_lo_, int k_hi_, float scale_log2e_) {
     kc = kc_; vc = vc_; hk = hk_; Hkv = Hkv_; k_lo = k_lo_; k_hi = k_hi_; scale_log2e = scale_log2e_;
+    page_stride = Hkv_ * ps * DT * 16;  // the host checks that this fits 31 bits
+    head_off = hk_ * ps * DT * 16;
     pages.init(bt, max_blocks, ps, k_lo_ & ~31);
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
@@ -124,12 +127,10 @@ struct Tile {
 
   // Loads are unconditional: a key outside [k_lo, k_hi) is replaced by the nearest key inside, which
   // lies in a page the request holds, so straight-line code with all loads in flight at once. What
-  // was loaded for such a key never counts: its score is masked, and compute() zeroes its value.
-  __device__ __forceinline__ void load(Frags<DT>& f, int kb) {
+  // was loaded for such a key never counts: its score is masked, and accumulate() zeroes its value.
+  __device__ __forceinline__ void load_k(Frags<DT>& f, int kb) {
     constexpr int D = DT * 16;
     const int lane = threadIdx.x & 63, i16 = lane & 15, g4 = lane >> 4;
-    const int ps = pages.ps;
-    pages.ensure(kb);
     const int last = k_hi - 1;
     // K rows of this lane: keys kg_row + (i16 & 3) and + 4, in one page (page size % 8 == 0)
     int key0 = kb + 8 * (i16 >> 2) + (i16 & 3), key1 = key0 + 4;
@@ -138,9 +139,9 @@ struct Tile {
     const int pg0 = pages.get(pages.page_of(key0)), pg1 = pages.get(pages.page_of(key1));
     // K pages are [Hkv][D / 8][page][8]: the 16-byte pieces of consecutive keys lie next to each other,
     // so the four lanes of a quad (four consecutive keys, one piece index) read 64 contiguous bytes
-    const bf16* kr0 = kc + ((int64_t)pg0 * Hkv + hk) * ps * D + pages.offset_of(key0) * 8;
-    const bf16* kr1 = kc + ((int64_t)pg1 * Hkv + hk) * ps * D + pages.offset_of(key1) * 8;
-    const int piece = ps * 8;
+    const bf16* kr0 = kc + ((int64_t)pg0 * page_stride + (head_off + pages.offset_of(key0) * 8));
+    const bf16* kr1 = kc + ((int64_t)pg1 * page_stride + (head_off + pages.offset_of(key1) * 8));
+    const int piece = pages.ps * 8;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       int c = ks * 4 + g4;
@@ -150,23 +151,29 @@ struct Tile {
       f.k[1][ks] = *(const bf16x8*)(kr1 + c * piece);
       if (DT % 2 == 1 && ks == KS - 1 && !dv) f.k[0][ks] = f.k[1][ks] = zero8();
     }
-    // V^T rows of this lane: d = 16 dt + i16, keys kg .. kg + 7 (one page)
-    int kg = kb + 8 * g4;
-    const int g_lo = k_lo & ~7, g_hi = last & ~7;
-    kg = kg < g_lo ? g_lo : (kg > g_hi ? g_hi : kg);
-    const int pgv = pages.get(pages.page_of(kg));
-    const bf16* vrow = vc + (((int64_t)pgv * Hkv + hk) * D + i16) * ps + pages.offset_of(kg);
-#pragma unroll
-    for (int d = 0; d < DT; ++d) f.v[d] = *(const bf16x8*)(vrow + (int64_t)d * 16 * ps);
   }
 
-  // MASK: some key of the block is invisible to some column, or lies outside [k_lo, k_hi)
-  template <bool MASK>
-  __device__ __forceinline__ void compute(const Frags<DT>& f, const bf16x8 (&qf)[NT][KS], int kb,
-                                          const int (&col_lo)[NT], const int (&col_hi)[NT]) {
-    constexpr bool need_mask = MASK;
-    const int lane = threadIdx.x & 63, g4 = lane >> 4;
-    f32x4 s[NT][2];
+  __device__ __forceinline__ void load_v(Frags<DT>& f, int kb) {
+    const int lane = threadIdx.x & 63, i16 = lane & 15, g4 = lane >> 4;
+    const int ps = pages.ps;
+    // V^T rows of this lane: d = 16 dt + i16, keys kg .. kg + 7 (one page)
+    int kg = kb + 8 * g4;
+    const int g_lo = k_lo & ~7, g_hi = (k_hi - 1) & ~7;
+    kg = kg < g_lo ? g_lo : (kg > g_hi ? g_hi : kg);
+    const int pgv = pages.get(pages.page_of(kg));
+    const bf16* vrow = vc + ((int64_t)pgv * page_stride + (head_off + i16 * ps + pages.offset_of(kg)));
+#pragma unroll
+    for (int d = 0; d < DT; ++d) f.v[d] = *(const bf16x8*)(vrow + d * 16 * ps);
+  }
+
+  __device__ __forceinline__ void load(Frags<DT>& f, int kb) {
+    pages.ensure(kb);
+    load_k(f, kb);
+    load_v(f, kb);
+  }
+
+  // S^T of one block: s[t][a] holds, for column i16 of tile t, the keys kb + 8 g4 + 4 a + {0..3}
+  __device__ __forceinline__ void scores(const Frags<DT>& f, const bf16x8 (&qf)[NT][KS], f32x4 (&s)[NT][2]) {
 #pragma unroll
     for (int t = 0; t < NT; ++t) s[t][0] = s[t][1] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -176,9 +183,15 @@ struct Tile {
         s[t][0] = mfma16(f.k[0][ks], qf[t][ks], s[t][0]);
         s[t][1] = mfma16(f.k[1][ks], qf[t][ks], s[t][1]);
       }
-    // online softmax per column; this lane holds keys kb + 8 g4 + {0..7} of column i16
-    const int kg = kb + 8 * g4;
-    bf16x8 pf[NT];
+  }
+
+  // Online softmax per column; this lane holds keys kb + 8 g4 + {0..7} of column i16. Returns the
+  // weights as the B operand of the second product.
+  // MASK: some key of the block is invisible to some column, or lies outside [k_lo, k_hi)
+  template <bool MASK>
+  __device__ __forceinline__ void softmax(const f32x4 (&s)[NT][2], bf16x8 (&pf)[NT], int kb, const int (&col_lo)[NT],
+                                          const int (&col_hi)[NT]) {
+    const int kg = kb + 8 * ((threadIdx.x & 63) >> 4);
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       // raw scores; the running maximum m is kept in raw units too, and the scale is folded into
@@ -189,7 +202,7 @@ struct Tile {
         x[r] = s[t][0][r];
         x[4 + r] = s[t][1][r];
       }
-      if (need_mask) {
+      if (MASK) {
 #pragma unroll
         for (int e = 0; e < 8; ++e)
           if (kg + e < col_lo[t] || kg + e >= col_hi[t]) x[e] = -INFINITY;
@@ -220,11 +233,16 @@ struct Tile {
       m[t] = m_new;
       l[t] += ps_;  // partial over this lane's keys; lane groups are summed at the end
     }
-    // O^T += V^T . P
+  }
+
+  // O^T += V^T . P
+  template <bool MASK>
+  __device__ __forceinline__ void accumulate(const Frags<DT>& f, const bf16x8 (&pf)[NT], int kb) {
+    const int kg = kb + 8 * ((threadIdx.x & 63) >> 4);
 #pragma unroll
     for (int d = 0; d < DT; ++d) {
       bf16x8 vf = f.v[d];
-      if (need_mask) {
+      if (MASK) {
         // a stale slot may hold anything; its weight is 0, but 0 * inf would poison the sum
 #pragma unroll
         for (int e = 0; e < 8; ++e)
@@ -235,19 +253,32 @@ struct Tile {
     }
   }
 
+  template <bool MASK>
+  __device__ __forceinline__ void compute(const Frags<DT>& f, const bf16x8 (&qf)[NT][KS], int kb,
+                                          const int (&col_lo)[NT], const int (&col_hi)[NT]) {
+    f32x4 s[NT][2];
+    bf16x8 pf[NT];
+    scores(f, qf, s);
+    softmax<MASK>(s, pf, kb, col_lo, col_hi);
+    accumulate<MASK>(f, pf, kb);
+  }
+
   // All key blocks of [k_lo, k_hi); mask(kb) says whether block kb needs per-key masking.
-  // PREFETCH: the next block's loads are issued before the current block is computed (two sets of
-  // fragments in registers); without it one set, and latency is hidden by more waves per SIMD.
-  // TWO_BODIES: blocks that need no masking run a body without it (more code and registers, fewer
-  // instructions per block); otherwise every block runs the masking body.
-  template <bool PREFETCH, bool TWO_BODIES, class MaskFn>
+  // TWO_BODIES: blocks that need no masking run a body without it (more code, fewer instructions
+  // per block); otherwise every block runs the masking body.
+  // PIPELINED: the next block's K is loaded as soon as the scores are issued, and its V as soon as
+  // the second product is: each set of registers is refilled the moment its last reader has gone,
+  // so the loads are in flight during the softmax and the other product at no cost in registers.
+  // Otherwise a block's loads are issued right before its use and other waves hide the latency.
+  template <bool PIPELINED, bool TWO_BODIES, class MaskFn>
   __device__ __forceinline__ void walk(const bf16x8 (&qf)[NT][KS], const int (&col_lo)[NT], const int (&col_hi)[NT],
                                        MaskFn mask) {
     int kb = k_lo & ~31;
     if (kb >= k_hi) return;
-    if (!PREFETCH) {
+    Frags<DT> f;
+    if (!PIPELINED) {
+#pragma nounroll
       for (; kb < k_hi; kb += 32) {
-        Frags<DT> f;
         load(f, kb);
         if (!TWO_BODIES || mask(kb))
           compute<true>(f, qf, kb, col_lo, col_hi);
@@ -256,18 +287,24 @@ struct Tile {
       }
       return;
     }
-    Frags<DT> f0, f1;
-    load(f0, kb);
-    while (true) {
-      const bool more1 = kb + 32 < k_hi;
-      if (more1) load(f1, kb + 32);
-      if (!TWO_BODIES || mask(kb)) compute<true>(f0, qf, kb, col_lo, col_hi); else compute<false>(f0, qf, kb, col_lo, col_hi);
-      if (!more1) break;
-      const bool more2 = kb + 64 < k_hi;
-      if (more2) load(f0, kb + 64);
-      if (!TWO_BODIES || mask(kb + 32)) compute<true>(f1, qf, kb + 32, col_lo, col_hi); else compute<false>(f1, qf, kb + 32, col_lo, col_hi);
-      if (!more2) break;
-      kb += 64;
+    load(f, kb);
+#pragma nounroll
+    for (; kb < k_hi; kb += 32) {
+      f32x4 s[NT][2];
+      bf16x8 pf[NT];
+      scores(f, qf, s);
+      // past the last block there is nothing to read ahead: read the last block again (never used)
+      const int nb = kb + 32 < k_hi ? kb + 32 : kb;
+      pages.ensure(nb);
+      load_k(f, nb);
+      if (!TWO_BODIES || mask(kb)) {
+        softmax<true>(s, pf, kb, col_lo, col_hi);
+        accumulate<true>(f, pf, kb);
+      } else {
+        softmax<false>(s, pf, kb, col_lo, col_hi);
+        accumulate<false>(f, pf, kb);
+      }
+      load_v(f, nb);
     }
   }
 
@@ -280,10 +317,15 @@ struct Tile {
   }
 };
 
-// Measured on MI355X at head size 128 (2,048-token prompt): one set of fragments with two waves per
-// SIMD beats prefetching with one wave (123 us against 132 us a layer), and 32 query rows per wave
-// beat 16 (more waves, 168 us) and 64 (one wave per SIMD, 182 us).
-constexpr bool FLASH_PREFETCH = false;
+// Flash kernel. A workgroup owns QT x 16 query rows of one head; its four waves share the rows and
+// deal the key blocks among themselves in four contiguous runs, each wave keeping its own running
+// (maximum, sum, output); at the end waves 1..3 hand theirs to wave 0 through LDS, which combines
+// them and stores the rows. So every key block is read by one wave only, and a long row tile (many
+// keys under a causal mask) is four short pieces of work instead of one long one: with a few
+// thousand workgroups of unequal length issued longest first, the chip stays evenly busy.
+// Measured on MI355X at head size 128 (one 2,048-token prompt, 32 heads): 122 us for the former
+// one-wave-per-tile kernel, where the longest tile set the time.
+constexpr bool FLASH_PIPELINED = false;
 
 template <int DT, int QT, bool P2>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) attn_flash_kernel(
@@ -293,8 +335,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))
     int window, int H, int Hkv, int ps, int skip_single) {
   constexpr int D = DT * 16;
   constexpr int KS = (DT + 1) / 2;
-  constexpr int QW = 16 * QT;   // query rows per wave
-  constexpr int QB = QW * 4;    // per workgroup
+  constexpr int QW = 16 * QT;  // query rows per workgroup
+  __shared__ f32x4 part_o[3][QT][DT][64];
+  __shared__ float part_m[3][QT][64], part_l[3][QT][64];
   // Block order: the head index runs fastest and visits kv heads round-robin, so that the
   // workgroups an XCD receives (linear id modulo 8) share kv heads, and with them the L2 lines
   // of K and V. Late query tiles (most keys) are issued first.
@@ -307,8 +350,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))
   const int q_len = cu_seqlens[b + 1] - q_begin;
   const int hist = seq_lens[b] - q_len;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, i16 = lane & 15, g4 = lane >> 4;
-  const int q0 = tile * QB + wave * QW;
-  if (q0 >= q_len) return;  // no workgroup barrier below
+  const int q0 = tile * QW;
+  if (q0 >= q_len) return;                // the whole workgroup: nobody is left waiting at the barrier below
   if (skip_single && q_len == 1) return;  // single rows go to the split-K kernel
   const int32_t* bt = block_table + (int64_t)b * max_blocks;
 
@@ -328,18 +371,58 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))
     col_hi[t] = pos + 1;
     col_lo[t] = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
   }
+  // the keys any row of the tile sees, and this wave's run of 32-key blocks among them
   const int p_first = hist + q0;
   const int p_last = hist + (q0 + QW < q_len ? q0 + QW : q_len) - 1;
-  const int k_hi = p_last + 1;
-  const int k_lo = window > 0 ? (p_first - window + 1 > 0 ? p_first - window + 1 : 0) : 0;
+  const int all_hi = p_last + 1;
+  const int all_lo = window > 0 ? (p_first - window + 1 > 0 ? p_first - window + 1 : 0) : 0;
+  const int blk_first = all_lo >> 5, blk_end = (all_hi + 31) >> 5;
+  const int per = (blk_end - blk_first + 3) >> 2;
+  const int blk0 = blk_first + wave * per;
+  const int blk1 = blk0 + per < blk_end ? blk0 + per : blk_end;
+  const int k_lo = blk0 * 32 > all_lo ? blk0 * 32 : all_lo;
+  const int k_hi = blk1 * 32 < all_hi ? blk1 * 32 : all_hi;
 
   Tile<DT, QT, P2> tl;
   tl.init(kc, vc, bt, (int)max_blocks, hk, Hkv, ps, k_lo, k_hi, scale_log2e);
-  tl.template walk<FLASH_PREFETCH, true>(qf, col_lo, col_hi, [&](int kb) {
-    return kb + 31 > p_first || kb < k_lo || (window > 0 && kb < p_last - window + 1);
+  tl.template walk<FLASH_PIPELINED, true>(qf, col_lo, col_hi, [&](int kb) {
+    return kb + 31 > p_first || kb < all_lo || (window > 0 && kb < p_last - window + 1);
   });
+
+  if (wave > 0) {
+#pragma unroll
+    for (int t = 0; t < QT; ++t) {
+      part_m[wave - 1][t][lane] = tl.m[t];
+      part_l[wave - 1][t][lane] = tl.l[t];
+#pragma unroll
+      for (int d = 0; d < DT; ++d) part_o[wave - 1][t][d][lane] = tl.o[t][d];
+    }
+  }
+  __syncthreads();
+  if (wave > 0) return;
 #pragma unroll
   for (int t = 0; t < QT; ++t) {
+    // every wave keeps a lane's share in the same places, so the parts combine lane by lane:
+    // o = sum_r 2^(c (m_r - M)) o_r, likewise l (still a partial over the lane's keys)
+    float mr[3], M = tl.m[t];
+#pragma unroll
+    for (int r = 0; r < 3; ++r) {
+      mr[r] = part_m[r][t][lane];
+      M = fmaxf(M, mr[r]);
+    }
+    const float mc = (M == -INFINITY ? 0.f : M) * scale_log2e;
+    const float a0 = exp2_raw(fmaf(tl.m[t], scale_log2e, -mc));  // an empty part has m = -inf: weight 0
+    float lsum = tl.l[t] * a0;
+#pragma unroll
+    for (int d = 0; d < DT; ++d) tl.o[t][d] *= a0;
+#pragma unroll
+    for (int r = 0; r < 3; ++r) {
+      const float ar = exp2_raw(fmaf(mr[r], scale_log2e, -mc));
+      lsum += part_l[r][t][lane] * ar;
+#pragma unroll
+      for (int d = 0; d < DT; ++d) tl.o[t][d] += part_o[r][t][d][lane] * ar;
+    }
+    tl.l[t] = lsum;
     const float lt = tl.sum_l(t);
     const float inv = lt > 0.f ? 1.f / lt : 0.f;
     const int row = q0 + t * 16 + i16;
@@ -471,20 +554,22 @@ int launch_flash(const bf16* q, int64_t ld_q, bf16* out, int64_t ld_out, const b
                  const int32_t* bt, int64_t max_blocks, const int32_t* cu, const int32_t* sl, int num_reqs,
                  int max_q_len, float scale, int window, int H, int Hkv, int ps, int skip_single, hipStream_t stream) {
   const float sl2 = scale * LOG2E;
-  if (max_q_len > 64) {
-    constexpr int QB = 2 * 16 * 4;
-    const int tiles = (max_q_len + QB - 1) / QB;
+  const bool p2 = (ps & (ps - 1)) == 0;
+  // 32 rows per workgroup where the head size leaves room for two row tiles (registers, and the LDS the
+  // waves meet in), and the portions are longer than one tile; otherwise 16
+  if (DT <= 8 && max_q_len > 16) {
+    constexpr int QT = DT <= 8 ? 2 : 1;
+    const int tiles = (max_q_len + 16 * QT - 1) / (16 * QT);
     const int64_t blocks = (int64_t)tiles * H * num_reqs;
     if (blocks > 0x7fffffff) return ERR_UNSUPPORTED;
-    auto kernel = (ps & (ps - 1)) == 0 ? attn_flash_kernel<DT, 2, true> : attn_flash_kernel<DT, 2, false>;
+    auto kernel = p2 ? attn_flash_kernel<DT, QT, true> : attn_flash_kernel<DT, QT, false>;
     kernel<<<(unsigned)blocks, 256, 0, stream>>>(q, ld_q, out, ld_out, kc, vc, bt, max_blocks, cu, sl, tiles, sl2,
                                                  window, H, Hkv, ps, skip_single);
   } else {
-    constexpr int QB = 16 * 4;
-    const int tiles = (max_q_len + QB - 1) / QB;
+    const int tiles = (max_q_len + 15) / 16;
     const int64_t blocks = (int64_t)tiles * H * num_reqs;
     if (blocks > 0x7fffffff) return ERR_UNSUPPORTED;
-    auto kernel = (ps & (ps - 1)) == 0 ? attn_flash_kernel<DT, 1, true> : attn_flash_kernel<DT, 1, false>;
+    auto kernel = p2 ? attn_flash_kernel<DT, 1, true> : attn_flash_kernel<DT, 1, false>;
     kernel<<<(unsigned)blocks, 256, 0, stream>>>(q, ld_q, out, ld_out, kc, vc, bt, max_blocks, cu, sl, tiles, sl2,
                                                  window, H, Hkv, ps, skip_single);
   }
@@ -523,7 +608,9 @@ extern "C" int dinfer_attn_mfma_supports(int head_dim, int page_size, int heads,
     case 32: case 48: case 64: case 96: case 128: case 256: break;
     default: return 0;
   }
-  return page_size > 0 && page_size % 8 == 0 && kv_heads > 0 && heads % kv_heads == 0 ? 1 : 0;
+  if (!(page_size > 0 && page_size % 8 == 0 && kv_heads > 0 && heads % kv_heads == 0)) return 0;
+  // the kernels keep the elements of one page (all kv heads) in 32-bit arithmetic
+  return (int64_t)kv_heads * page_size * head_dim < (int64_t)1 << 30 ? 1 : 0;
 }
 
 // skip_single: requests with one row are left to the split-K kernel.
