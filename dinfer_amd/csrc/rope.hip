@@ -360,7 +360,9 @@ extern "C" int dinfer_qkv_post(int dtype, void* qkv, int64_t tokens, int64_t ld,
                                int64_t v_off, const void* q_gain, const void* k_gain, int w_f32, float eps,
                                float w_offset, const int32_t* positions, const float* cos_sin, int rotary_dim,
                                int style, void* k_cache, void* v_cache, const int64_t* slot_mapping, int heads,
-                               int kv_heads, int head_dim, int page_size, hipStream_t stream) {
+                               int kv_heads, int head_dim, int page_size, int token_runs, hipStream_t stream) {
+  // token_runs: the tokens come in runs of consecutive positions of a request (prompt portions), so
+  // that gathering 8 tokens' values into 16-byte rows of the transposed V pages pays
   if (tokens <= 0) return OK;
   if (heads <= 0 || kv_heads <= 0 || head_dim <= 0 || page_size <= 0 || tokens > 0x7fffffff) return ERR_BAD_SHAPE;
   if (head_dim > MAX_D) return ERR_UNSUPPORTED;
@@ -378,7 +380,7 @@ extern "C" int dinfer_qkv_post(int dtype, void* qkv, int64_t tokens, int64_t ld,
     const int lph = head_dim / 8, hpw = 64 / lph;
     const dim3 vgrid((unsigned)tokens, (unsigned)((items + WAVES * hpw - 1) / (WAVES * hpw)));
     // many tokens: V goes to its transposed pages through the gathering kernel (16-byte stores)
-    const int skip_v = (slot_mapping && tokens >= 64 && page_size % 8 == 0 && ((uintptr_t)v_cache % 16) == 0) ? 1 : 0;
+    const int skip_v = (slot_mapping && token_runs && tokens >= 64 && page_size % 8 == 0 && ((uintptr_t)v_cache % 16) == 0) ? 1 : 0;
     if (skip_v)
       v_write_transposed_kernel<<<dim3((unsigned)((tokens + 8 * WAVES - 1) / (8 * WAVES)), (unsigned)kv_heads), WAVES * 64,
                                   0, stream>>>((const bf16*)qkv, ld, v_off, (bf16*)v_cache, slot_mapping, (int)tokens,

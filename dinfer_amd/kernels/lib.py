@@ -27,7 +27,7 @@ SIGNATURES = {
     "dinfer_rmsnorm": ("norm", [_I, _P, _P, _P, _P, _I, _P, _L, _L, _L, _L, _F, _F, _P]),
     "dinfer_qkv_post": (
         "rope",
-        [_I, _P, _L, _L, _L, _L, _L, _P, _P, _I, _F, _F, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _P],
+        [_I, _P, _L, _L, _L, _L, _L, _P, _P, _I, _F, _F, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _P],
     ),
     "dinfer_attn_paged_ref": (
         "attention_ref",

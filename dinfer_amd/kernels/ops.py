@@ -160,11 +160,12 @@ def qkv_post(qkv: torch.Tensor, tokens: int, *, heads: int, kv_heads: int, head_
              v_off: int, q_gain: torch.Tensor | None, k_gain: torch.Tensor | None, eps: float, gain_offset: float,
              positions: torch.Tensor, cos_sin: torch.Tensor | None, rotary_dim: int, rope_style: int,
              k_cache: torch.Tensor | None, v_cache: torch.Tensor | None, slot_mapping: torch.Tensor | None,
-             page_size: int) -> None:
+             page_size: int, token_runs: bool = True) -> None:
     """Per-head q/k norm, rotation, q written back in place, k and v written to the cache pages.
 
     k_cache and v_cache in the page layouts above; slot_mapping int64 [T] (None: nothing is written
-    to the cache).
+    to the cache). token_runs: the tokens come in runs of consecutive positions (prompt portions, not
+    single decoded tokens); it only chooses the faster of two ways of writing V.
     """
     _need_gpu(qkv, q_gain, k_gain, positions, cos_sin, k_cache, v_cache, slot_mapping)
     ld = _rows(qkv)
@@ -186,7 +187,7 @@ def qkv_post(qkv: torch.Tensor, tokens: int, *, heads: int, kv_heads: int, head_
     lib.call("dinfer_qkv_post", dtype_code(qkv.dtype), qkv.data_ptr(), tokens, ld, q_off, k_off, v_off,
              _ptr(q_gain), _ptr(k_gain), wf32, float(eps), float(gain_offset), positions.data_ptr(), _ptr(cos_sin),
              rotary_dim, rope_style, _ptr(k_cache), _ptr(v_cache), _ptr(slot_mapping), heads, kv_heads, head_dim,
-             page_size, _stream())
+             page_size, int(token_runs), _stream())
 
 
 def attn_paged_ref(q: torch.Tensor, out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,

@@ -81,7 +81,8 @@ class Attention(Mixer):
             eps=qn.eps if qn else 0.0, gain_offset=qn.weight_offset if qn else 0.0,
             positions=batch.positions, cos_sin=self.position.table(), rotary_dim=self.position.rotary_dim,
             rope_style=self.position.style, k_cache=cache.k, v_cache=cache.v,
-            slot_mapping=batch.slot_mapping[g] if cache.owner else None, page_size=self.page_size)
+            slot_mapping=batch.slot_mapping[g] if cache.owner else None, page_size=self.page_size,
+            token_runs=batch.max_q_len >= 8)
         attn_kernels.paged_attention(
             self.qkv_buf, self.attn_buf, cache.k, cache.v, batch, g, self.attn_ws, scale=self.scale,
             window=self.window or 0, heads=self.heads, kv_heads=self.kv_heads, head_dim=self.head_dim,
