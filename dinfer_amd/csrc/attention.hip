@@ -6,9 +6,11 @@
 //   A (16 x 32): lane l holds A[l % 16][8 * (l / 16) .. + 8]
 //   B (32 x 16): lane l holds B[8 * (l / 16) .. + 8][l % 16]
 //   D (16 x 16): lane l holds D[4 * (l / 16) + r][l % 16], r = 0..3
-// K pages [Hkv][page][D] give A = K rows straight from memory (contraction over
-// d); V pages [Hkv][D][page] (transposed) give A = V^T rows straight from memory
-// (contraction over keys). Nothing is staged through LDS.
+// K pages [Hkv][D / 8][page][8] give A = 8-element pieces of K rows straight from
+// memory (contraction over d; the pieces of consecutive keys are contiguous, so
+// a quad of lanes reads 64 contiguous bytes); V pages [Hkv][D][page] (transposed)
+// give A = V^T rows straight from memory (contraction over keys). K and V are
+// not staged through LDS.
 //
 // A block of 32 keys is scored by two MFMA chains (a = 0, 1). Row i of chain a
 // is key  kb + 8 * (i / 4) + 4 * a + (i % 4),  so lane group g = l / 16 ends up
@@ -17,9 +19,10 @@
 // A query (a column, l % 16) keeps its running maximum, sum and output column in
 // the same lanes through both products.
 //
-//   flash:  query rows with or without history, causal, optional window; one
-//           wave owns QT x 16 query rows of one head and walks its keys in
-//           blocks of 32 (online softmax in base 2).
+//   flash:  query rows with or without history, causal, optional window; a
+//           workgroup owns QT x 16 query rows of one head, its four waves walk a
+//           quarter of the keys each in blocks of 32 (online softmax in base 2)
+//           and combine their results in LDS.
 //   decode: all requests bring one row; the G query heads of a kv head are the
 //           16 columns, so K and V are read once per group; the keys are split
 //           over workgroups, each writing (m, l, o) partials; a merge kernel
