@@ -269,45 +269,20 @@ struct Tile {
   // All key blocks of [k_lo, k_hi); mask(kb) says whether block kb needs per-key masking.
   // TWO_BODIES: blocks that need no masking run a body without it (more code, fewer instructions
   // per block); otherwise every block runs the masking body.
-  // PIPELINED: the next block's K is loaded as soon as the scores are issued, and its V as soon as
-  // the second product is: each set of registers is refilled the moment its last reader has gone,
-  // so the loads are in flight during the softmax and the other product at no cost in registers.
-  // Otherwise a block's loads are issued right before its use and other waves hide the latency.
-  template <bool PIPELINED, bool TWO_BODIES, class MaskFn>
+  // A block's loads are issued right before its use and other waves hide the latency: reading a
+  // block ahead was measured and does not pay (neither with a second set of registers nor by
+  // refilling each fragment as soon as its last reader has issued).
+  template <bool TWO_BODIES, class MaskFn>
   __device__ __forceinline__ void walk(const bf16x8 (&qf)[NT][KS], const int (&col_lo)[NT], const int (&col_hi)[NT],
                                        MaskFn mask) {
-    int kb = k_lo & ~31;
-    if (kb >= k_hi) return;
     Frags<DT> f;
-    if (!PIPELINED) {
 #pragma nounroll
-      for (; kb < k_hi; kb += 32) {
-        load(f, kb);
-        if (!TWO_BODIES || mask(kb))
-          compute<true>(f, qf, kb, col_lo, col_hi);
-        else
-          compute<false>(f, qf, kb, col_lo, col_hi);
-      }
-      return;
-    }
-    load(f, kb);
-#pragma nounroll
-    for (; kb < k_hi; kb += 32) {
-      f32x4 s[NT][2];
-      bf16x8 pf[NT];
-      scores(f, qf, s);
-      // past the last block there is nothing to read ahead: read the last block again (never used)
-      const int nb = kb + 32 < k_hi ? kb + 32 : kb;
-      pages.ensure(nb);
-      load_k(f, nb);
-      if (!TWO_BODIES || mask(kb)) {
-        softmax<true>(s, pf, kb, col_lo, col_hi);
-        accumulate<true>(f, pf, kb);
-      } else {
-        softmax<false>(s, pf, kb, col_lo, col_hi);
-        accumulate<false>(f, pf, kb);
-      }
-      load_v(f, nb);
+    for (int kb = k_lo & ~31; kb < k_hi; kb += 32) {
+      load(f, kb);
+      if (!TWO_BODIES || mask(kb))
+        compute<true>(f, qf, kb, col_lo, col_hi);
+      else
+        compute<false>(f, qf, kb, col_lo, col_hi);
     }
   }
 
@@ -328,8 +303,6 @@ struct Tile {
 // thousand workgroups of unequal length issued longest first, the chip stays evenly busy.
 // Measured on MI355X at head size 128 (one 2,048-token prompt, 32 heads): 122 us for the former
 // one-wave-per-tile kernel, where the longest tile set the time.
-constexpr bool FLASH_PIPELINED = false;
-
 template <int DT, int QT, bool P2>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))) attn_flash_kernel(
     const bf16* __restrict__ q, int64_t ld_q, bf16* __restrict__ out, int64_t ld_out, const bf16* __restrict__ kc,
@@ -388,7 +361,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))
 
   Tile<DT, QT, P2> tl;
   tl.init(kc, vc, bt, (int)max_blocks, hk, Hkv, ps, k_lo, k_hi, scale_log2e);
-  tl.template walk<FLASH_PIPELINED, true>(qf, col_lo, col_hi, [&](int kb) {
+  tl.template walk<true>(qf, col_lo, col_hi, [&](int kb) {
     return kb + 31 > p_first || kb < all_lo || (window > 0 && kb < p_last - window + 1);
   });
 
@@ -489,7 +462,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 8)))
   const int col_lo[1] = {k_lo}, col_hi[1] = {k_hi};
   Tile<DT, 1, P2> tl;
   tl.init(kc, vc, bt, (int)max_blocks, hk, Hkv, ps, k_lo, k_hi, scale_log2e);
-  tl.template walk<false, false>(qf, col_lo, col_hi, [&](int kb) { return kb < k_lo || kb + 32 > k_hi; });
+  tl.template walk<false>(qf, col_lo, col_hi, [&](int kb) { return kb < k_lo || kb + 32 > k_hi; });
   const float lt = tl.sum_l(0);
   if (i16 < G) {
     float* pp = part + (((int64_t)b * H + hk * G + i16) * splits + sp) * (D + 4);

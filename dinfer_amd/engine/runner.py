@@ -47,7 +47,7 @@ class ModelRunner:
         # decode rows may ride on top of the prompt budget (service.rs:206-210)
         self.max_tokens = options.max_num_batched_tokens + (options.max_num_seqs if options.decode_exempt_from_budget else 0)
         self.ctx = BuildContext(device, self.dtype, self.max_tokens, self.max_rows, self.page_size,
-                                options.max_num_seqs)
+                                options.max_num_seqs, max_seq_len=options.max_model_len)
         model.bind(self.ctx)
         self._build_caches()
         self.batch = StepBatch(device, self.max_tokens, options.max_num_seqs, self.max_rows,

@@ -12,7 +12,8 @@ import torch
 from . import ops
 
 TARGET_WAVES = 1024   # split-K aims at about this many waves (measured: more, shorter waves cost more than they hide)
-MAX_SPLITS = 32
+MAX_SPLITS = 128      # the kernels take up to 256
+MIN_KEYS_PER_SPLIT = 512   # of the longest request the engine admits, beyond 32 parts
 
 
 class Workspace:
@@ -20,6 +21,11 @@ class Workspace:
 
     def __init__(self, ctx, heads: int, kv_heads: int, head_dim: int):
         self.max_reqs = ctx.max_reqs
+        # measured on MI355X (head 128, 8 kv heads): one request of 2k-4k keys is fastest with 32 parts,
+        # of 32k with 64, of 128k with 128; the count may not depend on the lengths of a step (a captured
+        # graph must stay valid), so it is bounded by the longest request the engine admits
+        longest = ctx.max_seq_len or 4096
+        self.max_splits = min(MAX_SPLITS, max(32, longest // MIN_KEYS_PER_SPLIT))
         self.mfma = (ctx.dtype == torch.bfloat16 and ops.attn_mfma_supports(head_dim, ctx.page_size, heads, kv_heads))
         self.split_k = self.mfma and heads // kv_heads <= 16
         self.part = None
@@ -31,7 +37,7 @@ class Workspace:
 
     def splits(self, num_reqs: int) -> int:
         """Parts per request: a function of the batch size only, so a captured graph stays valid."""
-        return max(1, min(MAX_SPLITS, TARGET_WAVES // (num_reqs * self.kv_heads)))
+        return max(1, min(self.max_splits, TARGET_WAVES // (num_reqs * self.kv_heads)))
 
 
 def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k_cache, v_cache, batch, group: int, ws: Workspace, *,

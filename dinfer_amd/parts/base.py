@@ -44,9 +44,12 @@ class BuildContext:
     """What a part may know about the engine it is built into."""
 
     def __init__(self, device, dtype: torch.dtype, max_tokens: int, max_rows: int, page_size: int,
-                 max_reqs: int = 1):
+                 max_reqs: int = 1, max_seq_len: int | None = None):
+        """max_tokens / max_rows / max_reqs: the largest step; max_seq_len: the longest request
+        (None: unknown), for parts whose launch shapes are sized for it."""
         self.device, self.dtype = device, dtype
         self.max_tokens, self.max_rows, self.page_size, self.max_reqs = max_tokens, max_rows, page_size, max_reqs
+        self.max_seq_len = max_seq_len
         self.workspace = Workspace(device, dtype, max_tokens)
 
 
