@@ -88,6 +88,15 @@ struct Pages {
   __device__ __forceinline__ int get(int page) const { return __shfl(reg, page - base, 64); }
 };
 
+// 16 bytes of cache pages; stream: past the caches (the bytes are used once)
+template <bool STREAM>
+__device__ __forceinline__ bf16x8 ld16(const bf16* p) {
+  if constexpr (STREAM)
+    return __builtin_nontemporal_load((const bf16x8*)p);
+  else
+    return *(const bf16x8*)p;
+}
+
 template <int DT>
 struct Frags {
   static constexpr int KS = (DT + 1) / 2;
@@ -101,7 +110,8 @@ struct Frags {
 //   k_lo, k_hi  the keys this wave may touch at all (held pages, written slots)
 // load() issues the loads of one block, compute() consumes them; walk() keeps the next block's
 // loads in flight while the current one is computed.
-template <int DT, int NT, bool P2>
+// STREAM: K and V are read with non-temporal loads (each byte is used once: many requests, keys read once).
+template <int DT, int NT, bool P2, bool STREAM = false>
 struct Tile {
   static constexpr int KS = (DT + 1) / 2;  // 32-wide steps over the head dimension
   f32x4 o[NT][DT];
@@ -150,8 +160,8 @@ struct Tile {
       int c = ks * 4 + g4;
       const bool dv = c * 8 < D;  // D % 32 == 16: the upper half of the last step is padding
       if (!dv) c = 0;
-      f.k[0][ks] = *(const bf16x8*)(kr0 + c * piece);
-      f.k[1][ks] = *(const bf16x8*)(kr1 + c * piece);
+      f.k[0][ks] = ld16<STREAM>(kr0 + c * piece);
+      f.k[1][ks] = ld16<STREAM>(kr1 + c * piece);
       if (DT % 2 == 1 && ks == KS - 1 && !dv) f.k[0][ks] = f.k[1][ks] = zero8();
     }
   }
@@ -166,7 +176,7 @@ struct Tile {
     const int pgv = pages.get(pages.page_of(kg));
     const bf16* vrow = vc + ((int64_t)pgv * page_stride + (head_off + i16 * ps + pages.offset_of(kg)));
 #pragma unroll
-    for (int d = 0; d < DT; ++d) f.v[d] = *(const bf16x8*)(vrow + d * 16 * ps);
+    for (int d = 0; d < DT; ++d) f.v[d] = ld16<STREAM>(vrow + d * 16 * ps);
   }
 
   __device__ __forceinline__ void load(Frags<DT>& f, int kb) {
@@ -428,7 +438,7 @@ __device__ __forceinline__ void split_range(int seq, int window, int splits, int
 }
 
 // One wave per (split, kv head, request). part: [B, H, splits, D + 4] float = (m in base-2 units, l, -, -, o[D]).
-template <int DT, bool P2>
+template <int DT, bool P2, bool STREAM>
 __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 8))) attn_decode_kernel(
     const bf16* __restrict__ q, int64_t ld_q, float* __restrict__ part, const bf16* __restrict__ kc,
     const bf16* __restrict__ vc, const int32_t* __restrict__ block_table, int64_t max_blocks,
@@ -460,7 +470,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 8)))
     }
   }
   const int col_lo[1] = {k_lo}, col_hi[1] = {k_hi};
-  Tile<DT, 1, P2> tl;
+  Tile<DT, 1, P2, STREAM> tl;
   tl.init(kc, vc, bt, (int)max_blocks, hk, Hkv, ps, k_lo, k_hi, scale_log2e);
   tl.template walk<false>(qf, col_lo, col_hi, [&](int kb) { return kb < k_lo || kb + 32 > k_hi; });
   const float lt = tl.sum_l(0);
@@ -556,7 +566,11 @@ template <int DT>
 int launch_decode(const bf16* q, int64_t ld_q, bf16* out, int64_t ld_out, float* part, const bf16* kc, const bf16* vc,
                   const int32_t* bt, int64_t max_blocks, const int32_t* cu, const int32_t* sl, int num_reqs,
                   int splits, float scale, int window, int H, int Hkv, int ps, hipStream_t stream) {
-  auto kernel = (ps & (ps - 1)) == 0 ? attn_decode_kernel<DT, true> : attn_decode_kernel<DT, false>;
+  // many requests: the keys of a step exceed the caches and each is used once, so they are read past
+  // them (measured at 64 requests of 2k-4k keys: 10% faster; at 8 or fewer, slightly slower)
+  const bool p2 = (ps & (ps - 1)) == 0, stream_kv = num_reqs >= 32;
+  auto kernel = p2 ? (stream_kv ? attn_decode_kernel<DT, true, true> : attn_decode_kernel<DT, true, false>)
+                   : (stream_kv ? attn_decode_kernel<DT, false, true> : attn_decode_kernel<DT, false, false>);
   kernel<<<dim3((unsigned)splits, (unsigned)Hkv, (unsigned)num_reqs), 64, 0, stream>>>(
       q, ld_q, part, kc, vc, bt, max_blocks, cu, sl, splits, scale * LOG2E, window, H, Hkv, ps);
   const int D = DT * 16;
