@@ -3,13 +3,20 @@
 // the LM head, where time is the time to stream W from HBM once.
 //
 // v_mfma_f32_16x16x32_bf16 with the weight as the A operand: a tile is 16 weight
-// rows (n) x 16 tokens (m), contracted over k. Lane l = (i = l % 16, g = l / 16)
-// loads 32 contiguous bytes W[n0 + i][kk + 16 g .. + 16] and feeds them to two
-// MFMAs; the activations are loaded with the same k mapping, so a wave reads
-// 128 contiguous bytes of each of its 16 rows per step, and the waves of a
-// workgroup take consecutive runs of k of the same rows (split-K inside the
-// workgroup). Partial sums meet in LDS and are added in wave order, then stored
-// once. No atomics: the result of a given launch shape is reproducible.
+// rows (n) x 16 tokens (m), contracted over k in steps of 64.
+//
+// Loads are shaped for the memory path, not for the MFMA: lane l reads the
+// 16-byte piece l % 8 of row l / 8, so that eight lanes read one whole 128-byte
+// line and an instruction touches 8 lines (with the MFMA's own lane order, one
+// row per lane, it touches 64 line-quads and the load-return path of the CU was
+// busy 75% of the time, measured). Each wave turns a tile into MFMA order through
+// a 2.3 KB strip of LDS of its own (rows padded to 144 bytes: both the writes and
+// the reads are free of bank conflicts); a wave's LDS operations complete in
+// order, so the strip needs no barrier. Activations go the same way.
+//
+// The waves of a workgroup take consecutive runs of k of the same rows (split-K
+// inside the workgroup). Partial sums meet in LDS and are added in wave order,
+// then stored once. No atomics: the result of a given launch shape is reproducible.
 //
 //   MT = ceil(M / 16) token tiles share every weight fragment (registers),
 //   RT weight-row tiles share every activation fragment.
@@ -31,6 +38,23 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
+// Orders a wave's LDS writes before its reads of what other lanes wrote (and the reverse): the hardware
+// runs a wave's LDS operations in order, this keeps the compiler from moving them across.
+__device__ __forceinline__ void wave_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+}
+
+// 16 bytes of the weight; STREAM: read past the caches (a large weight is read once per launch, and
+// whole lines at a time: measured 10% faster from about 40 MB on, slightly slower below)
+template <bool STREAM>
+__device__ __forceinline__ bf16x8 ld_weight(const bf16* p) {
+  if constexpr (STREAM)
+    return __builtin_nontemporal_load((const bf16x8*)p);
+  else
+    return *(const bf16x8*)p;
+}
+
 template <class O>
 __device__ __forceinline__ void store4(O* p, f32x4 v);
 template <>
@@ -46,34 +70,45 @@ __device__ __forceinline__ void store4<bf16>(bf16* p, f32x4 v) {
 // GATED (RT == 2): W is [2N, K], rows [0, N) the gate and [N, 2N) the up projection; the workgroup's
 // two row tiles are gate rows n0.. and up rows N + n0.., and the epilogue stores
 // silu(gate) * up into C [M, N]: the activation costs no pass of its own.
-template <int MT, int RT, class O, bool GATED = false>
+template <int MT, int RT, class O, bool GATED, bool STREAM>
 __global__ void __launch_bounds__(1024) gemm_small_m_kernel(const bf16* __restrict__ A, int64_t lda,
                                                             const bf16* __restrict__ W, int64_t ldw,
                                                             O* __restrict__ C, int64_t ldc, int M, int N, int K) {
   static_assert(!GATED || RT == 2, "the gated form pairs one gate tile with one up tile");
   // 64-wide k steps in flight per wave: as many as the register file takes at 16 waves a workgroup
   constexpr int UNROLL = MT <= 2 ? (4 / RT > 0 ? 4 / RT : 1) : (2 / RT > 0 ? 2 / RT : 1);
-  extern __shared__ float red[];  // [waves][RT * MT][64 lanes][4]
+  constexpr int ROW_BYTES = 144;              // 64 k of a row and 16 bytes of padding
+  constexpr int STRIP_BYTES = 16 * ROW_BYTES;  // one tile of 16 rows
+  extern __shared__ __attribute__((aligned(16))) char smem[];  // a strip per wave; afterwards [waves][RT * MT][64 lanes][4] sums
+  float* red = (float*)smem;
   const int nw = blockDim.x >> 6;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, i16 = lane & 15, g4 = lane >> 4;
+  const int lrow = lane >> 3, lpiece = lane & 7;  // what this lane loads: piece lpiece of rows lrow and lrow + 8
   const int n0 = GATED ? blockIdx.x * 16 : blockIdx.x * 16 * RT;
+  char* strip = smem + wave * STRIP_BYTES;
+  char* put = strip + lrow * ROW_BYTES + lpiece * 16;  // where this lane's loads go (rows lrow, + 8)
+  const char* get = strip + i16 * ROW_BYTES + g4 * 16;  // its MFMA operands: row i16, pieces g4 and 4 + g4
 
-  const bf16* wp[RT];
+  const bf16* wp[RT][2];
 #pragma unroll
-  for (int r = 0; r < RT; ++r) {
-    int n = GATED ? n0 + i16 : n0 + r * 16 + i16;
-    if (n >= N) n = N - 1;  // rows past the end are computed and dropped
-    if (GATED && r == 1) n += N;
-    wp[r] = W + (int64_t)n * ldw + 16 * g4;
-  }
-  const bf16* ap[MT];
-  bool arow[MT];
+  for (int r = 0; r < RT; ++r)
 #pragma unroll
-  for (int t = 0; t < MT; ++t) {
-    const int m = t * 16 + i16;
-    arow[t] = m < M;
-    ap[t] = A + (int64_t)(arow[t] ? m : 0) * lda + 16 * g4;
-  }
+    for (int h = 0; h < 2; ++h) {
+      int n = (GATED ? n0 : n0 + r * 16) + lrow + 8 * h;
+      if (n >= N) n = N - 1;  // rows past the end are computed and dropped
+      if (GATED && r == 1) n += N;
+      wp[r][h] = W + (int64_t)n * ldw + 8 * lpiece;
+    }
+  const bf16* ap[MT][2];
+  bool arow[MT][2];
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int m = t * 16 + lrow + 8 * h;
+      arow[t][h] = m < M;
+      ap[t][h] = A + (int64_t)(arow[t][h] ? m : 0) * lda + 8 * lpiece;
+    }
   f32x4 acc[RT][MT];
 #pragma unroll
   for (int r = 0; r < RT; ++r)
@@ -86,33 +121,49 @@ __global__ void __launch_bounds__(1024) gemm_small_m_kernel(const bf16* __restri
   const int s_begin = wave * per_wave;
   const int s_end = s_begin + per_wave < steps ? s_begin + per_wave : steps;
   for (int s0 = s_begin; s0 < s_end; s0 += UNROLL) {
-    bf16x8 wf[UNROLL][RT][2], af[UNROLL][MT][2];
+    bf16x8 wraw[UNROLL][RT][2], araw[UNROLL][MT][2];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       const int kk = (s0 + u) * 64;
-      const int k = kk + 16 * g4;
-      const bool ok0 = k < K && (s0 + u) < s_end, ok1 = k + 8 < K && (s0 + u) < s_end;
-#pragma unroll
-      for (int r = 0; r < RT; ++r) {
-        wf[u][r][0] = ok0 ? *(const bf16x8*)(wp[r] + kk) : zero8();
-        wf[u][r][1] = ok1 ? *(const bf16x8*)(wp[r] + kk + 8) : zero8();
-      }
-#pragma unroll
-      for (int t = 0; t < MT; ++t) {
-        af[u][t][0] = (ok0 && arow[t]) ? *(const bf16x8*)(ap[t] + kk) : zero8();
-        af[u][t][1] = (ok1 && arow[t]) ? *(const bf16x8*)(ap[t] + kk + 8) : zero8();
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < UNROLL; ++u)
+      const bool ok = kk + 8 * lpiece < K && (s0 + u) < s_end;
 #pragma unroll
       for (int r = 0; r < RT; ++r)
 #pragma unroll
+        for (int h = 0; h < 2; ++h) wraw[u][r][h] = ok ? ld_weight<STREAM>(wp[r][h] + kk) : zero8();
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) araw[u][t][h] = (ok && arow[t][h]) ? *(const bf16x8*)(ap[t][h] + kk) : zero8();
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      // through the strip, tile by tile: what every lane loaded goes in by rows, the MFMA operands come out
+      bf16x8 af[MT][2];
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        *(bf16x8*)put = araw[u][t][0];
+        *(bf16x8*)(put + 8 * ROW_BYTES) = araw[u][t][1];
+        wave_sync();
+        af[t][0] = *(const bf16x8*)get;
+        af[t][1] = *(const bf16x8*)(get + 64);
+        wave_sync();
+      }
+#pragma unroll
+      for (int r = 0; r < RT; ++r) {
+        *(bf16x8*)put = wraw[u][r][0];
+        *(bf16x8*)(put + 8 * ROW_BYTES) = wraw[u][r][1];
+        wave_sync();
+        const bf16x8 wf0 = *(const bf16x8*)get, wf1 = *(const bf16x8*)(get + 64);
+        wave_sync();
+#pragma unroll
         for (int t = 0; t < MT; ++t) {
-          acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][r][0], af[u][t][0], acc[r][t], 0, 0, 0);
-          acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][r][1], af[u][t][1], acc[r][t], 0, 0, 0);
+          acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf0, af[t][0], acc[r][t], 0, 0, 0);
+          acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf1, af[t][1], acc[r][t], 0, 0, 0);
         }
+      }
+    }
   }
+  __syncthreads();  // the strips are done with: the same memory now takes the sums
 
   // partial sums of the waves meet in LDS
   f32x4* slot = (f32x4*)red + ((int64_t)wave * RT * MT) * 64 + lane;
@@ -152,12 +203,23 @@ __global__ void __launch_bounds__(1024) gemm_small_m_kernel(const bf16* __restri
   }
 }
 
+inline bool streams_weight(int64_t rows, int64_t K) { return rows * K * (int64_t)sizeof(bf16) >= (int64_t)40 << 20; }
+
+// LDS of a workgroup: a strip per wave while streaming, then the partial sums of every wave
+inline size_t lds_bytes(int waves, int rt, int mt) {
+  const size_t strips = (size_t)waves * 16 * 144, sums = (size_t)waves * rt * mt * 64 * sizeof(f32x4);
+  return strips > sums ? strips : sums;
+}
+
 template <int MT, int RT, class O>
 int launch(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, O* C, int64_t ldc, int M, int N, int K, int waves,
            hipStream_t stream) {
   const int row_tiles = (N + 16 * RT - 1) / (16 * RT);
-  const size_t lds = (size_t)waves * RT * MT * 64 * sizeof(f32x4);
-  gemm_small_m_kernel<MT, RT, O><<<(unsigned)row_tiles, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
+  const size_t lds = lds_bytes(waves, RT, MT);
+  if (streams_weight(N, K))
+    gemm_small_m_kernel<MT, RT, O, false, true><<<(unsigned)row_tiles, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
+  else
+    gemm_small_m_kernel<MT, RT, O, false, false><<<(unsigned)row_tiles, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
   return launch_status();
 }
 
@@ -165,8 +227,11 @@ template <int MT>
 int launch_gated(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, bf16* C, int64_t ldc, int M, int N, int K,
                  int waves, hipStream_t stream) {
   const int col_tiles = (N + 15) / 16;
-  const size_t lds = (size_t)waves * 2 * MT * 64 * sizeof(f32x4);
-  gemm_small_m_kernel<MT, 2, bf16, true><<<(unsigned)col_tiles, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
+  const size_t lds = lds_bytes(waves, 2, MT);
+  if (streams_weight(2 * (int64_t)N, K))
+    gemm_small_m_kernel<MT, 2, bf16, true, true><<<(unsigned)col_tiles, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
+  else
+    gemm_small_m_kernel<MT, 2, bf16, true, false><<<(unsigned)col_tiles, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
   return launch_status();
 }
 
@@ -197,18 +262,17 @@ extern "C" int dinfer_gemm_small_m(int out_f32, const void* A, int64_t lda, cons
     return ERR_BAD_SHAPE;
   const int mt = (int)(M + 15) / 16;
   int rt = row_tiles_per_block, nw = waves;
-  if (rt == 0) rt = mt >= 2 ? 2 : ((N >= 6144 && M > 4) ? 2 : 1);  // measured on MI355X
+  // measured on MI355X (K = 4096 and 12288, N from 4096 to 151936): one row tile and 8 waves a workgroup,
+  // two row tiles and 4 waves from N = 8192 on when there are more than a few tokens
+  if (rt == 0) rt = mt >= 2 ? 2 : ((N >= 8192 && M > 4) ? 2 : 1);
   if (nw == 0) {
-    // about 2048 waves in flight, each with at least two k steps
-    const int64_t tiles = (N + 16 * rt - 1) / (16 * rt);
-    nw = 4;
-    while (nw < 16 && tiles * nw < (rt == 1 ? 2048 : 768)) nw *= 2;
+    nw = (rt == 1 || N < 8192) ? 8 : 4;
     const int64_t steps = (K + 63) / 64;
-    while (nw > 1 && steps < 2 * nw) nw /= 2;
+    while (nw > 1 && steps < 2 * nw) nw /= 2;  // every wave at least two k steps
   }
-  while (nw > 1 && (size_t)nw * rt * mt * 64 * sizeof(f32x4) > 64 * 1024) nw /= 2;
+  while (nw > 1 && lds_bytes(nw, rt, mt) > 64 * 1024) nw /= 2;
   if (nw < 1 || nw > 16) return ERR_BAD_SHAPE;
-  if ((size_t)nw * rt * mt * 64 * sizeof(f32x4) > 64 * 1024) return ERR_UNSUPPORTED;
+  if (lds_bytes(nw, rt, mt) > 64 * 1024) return ERR_UNSUPPORTED;
   if (out_f32)
     return dispatch<float>((const bf16*)A, lda, (const bf16*)W, ldw, (float*)C, ldc, (int)M, (int)N, (int)K, rt, nw,
                            stream);
@@ -235,7 +299,7 @@ extern "C" int dinfer_gemm_small_m_gated(const void* A, int64_t lda, const void*
     const int64_t steps = (K + 63) / 64;
     while (nw > 1 && steps < 2 * nw) nw /= 2;
   }
-  if (nw < 1 || nw > 16 || (size_t)nw * 2 * mt * 64 * sizeof(f32x4) > 64 * 1024) return ERR_BAD_SHAPE;
+  if (nw < 1 || nw > 16 || lds_bytes(nw, 2, mt) > 64 * 1024) return ERR_BAD_SHAPE;
   if (mt == 1)
     return launch_gated<1>((const bf16*)A, lda, (const bf16*)W, ldw, (bf16*)C, ldc, (int)M, (int)N, (int)K, nw, stream);
   return launch_gated<2>((const bf16*)A, lda, (const bf16*)W, ldw, (bf16*)C, ldc, (int)M, (int)N, (int)K, nw, stream);
