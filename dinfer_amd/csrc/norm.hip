@@ -61,12 +61,22 @@ __global__ void __launch_bounds__(256) rmsnorm_bf16x8_kernel(const bf16* __restr
   bf16x8* o = (bf16x8*)(out + r * width);
   const int n8 = (int)(width / 8);
   float v[ITERS][8];
+  float g[ITERS][8];  // the gains: loaded with the row, not after the sum (one memory round trip less)
   float ss = 0.f;
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
     const int i = it * 256 + threadIdx.x;
     if (i < n8) {
       const bf16x8 xv = xr[i];
+      if (wf32) {
+        const float* wp = (const float*)w + (int64_t)i * 8;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) g[it][j] = wp[j] + w_offset;
+      } else {
+        const bf16x8 wv = ((const bf16x8*)w)[i];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) g[it][j] = (float)wv[j] + w_offset;
+      }
       if (rr) {
         const bf16x8 rv = rr[i];
         bf16x8 s;
@@ -91,15 +101,8 @@ __global__ void __launch_bounds__(256) rmsnorm_bf16x8_kernel(const bf16* __restr
     const int i = it * 256 + threadIdx.x;
     if (i < n8) {
       bf16x8 y;
-      if (wf32) {
-        const float* wp = (const float*)w + (int64_t)i * 8;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) y[j] = (bf16)(v[it][j] * inv * (wp[j] + w_offset));
-      } else {
-        const bf16x8 wv = ((const bf16x8*)w)[i];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) y[j] = (bf16)(v[it][j] * inv * ((float)wv[j] + w_offset));
-      }
+      for (int j = 0; j < 8; ++j) y[j] = (bf16)(v[it][j] * inv * g[it][j]);
       o[i] = y;
     }
   }
