@@ -263,8 +263,9 @@ extern "C" int dinfer_gemm_small_m(int out_f32, const void* A, int64_t lda, cons
   const int mt = (int)(M + 15) / 16;
   int rt = row_tiles_per_block, nw = waves;
   // measured on MI355X (K = 4096 and 12288, N from 4096 to 151936): one row tile and 8 waves a workgroup,
-  // two row tiles and 4 waves from N = 8192 on when there are more than a few tokens
-  if (rt == 0) rt = mt >= 2 ? 2 : ((N >= 8192 && M > 4) ? 2 : 1);
+  // two row tiles and 4 waves from N = 8192 on when there are more than a few tokens (four row tiles for a
+  // vocabulary-sized N at 17 to 32 tokens)
+  if (rt == 0) rt = mt >= 2 ? ((mt == 2 && N >= 65536) ? 4 : 2) : ((N >= 8192 && M > 4) ? 2 : 1);
   if (nw == 0) {
     nw = (rt == 1 || N < 8192) ? 8 : 4;
     const int64_t steps = (K + 63) / 64;
