@@ -20,8 +20,11 @@ class BlockPool:
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
-        if h:
-            native.fn("dh_pool_destroy")(h)
+        try:
+            if h:
+                native.fn("dh_pool_destroy")(h)
+        except Exception:  # the interpreter is shutting down: the process ends anyway
+            pass
 
     @property
     def num_free(self) -> int:

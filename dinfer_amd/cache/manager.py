@@ -81,8 +81,11 @@ class CacheManager:
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
-        if h:
-            native.fn("dh_cache_destroy")(h)
+        try:
+            if h:
+                native.fn("dh_cache_destroy")(h)
+        except Exception:  # the interpreter is shutting down: the process ends anyway
+            pass
 
     # ---- request numbers -------------------------------------------------------------------------
     def handle(self, req_id, create: bool = False, pin: bool = False) -> int:

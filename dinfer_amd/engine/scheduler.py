@@ -97,8 +97,11 @@ class Scheduler:
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
-        if h:
-            native.fn("dh_sched_destroy")(h)
+        try:
+            if h:
+                native.fn("dh_sched_destroy")(h)
+        except Exception:  # the interpreter is shutting down: the process ends anyway
+            pass
 
     # ---- intake --------------------------------------------------------------------------------
     def add_request(self, req: Request) -> None:
