@@ -1,7 +1,8 @@
 #!/usr/bin/env python3
 """In-process throughput of the engine on one MI355X: Qwen3-8B-shaped random weights.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L] [--shape 8b|14b|32b]
+                    [--prompt P] [--context C]
 
 Prints ONE JSON line. `value` is decoded tokens per second at the default batch (8), each
 request with a 2,048-token prompt in a 4,096-token context; a "step" is one decode step
@@ -31,7 +32,13 @@ sys.path.insert(0, str(Path(__file__).resolve().parent))
 SIZES = dict(vocab_size=151936, hidden_size=4096, intermediate_size=12288, num_hidden_layers=36,
              num_attention_heads=32, num_key_value_heads=8, head_dim=128, rms_norm_eps=1e-6, rope_theta=1e6,
              max_position_embeddings=40960, tie_word_embeddings=False)
-PROMPT, CONTEXT = 2048, 4096
+# further sizes of the same architecture (BASELINE.json configs[3] and [4]); `--shape` picks one
+SHAPES = {
+    "8b": {},
+    "14b": dict(hidden_size=5120, intermediate_size=17408, num_hidden_layers=40, num_attention_heads=40),
+    "32b": dict(hidden_size=5120, intermediate_size=25600, num_hidden_layers=64, num_attention_heads=64),
+}
+DEFAULT_PROMPT, DEFAULT_CONTEXT = 2048, 4096
 HBM_PEAK = 8.0e12
 MFMA_PEAK = {"bfloat16": 2.5e15, "float32": 157.3e12}
 
@@ -56,6 +63,9 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     ap.add_argument("--no-hip-graph", action="store_true")
     ap.add_argument("--skip-prefill", action="store_true", help="do not time the 2,048-token prefill (profiling decode)")
+    ap.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="layer sizes (default: Qwen3-8B)")
+    ap.add_argument("--prompt", type=int, default=DEFAULT_PROMPT, help="prompt tokens per request (and of the timed prefill)")
+    ap.add_argument("--context", type=int, default=DEFAULT_CONTEXT, help="max_model_len the engine is built for")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py measures one GPU only (this engine does not use a second one); got --gpus {a.gpus}")
@@ -65,7 +75,11 @@ def main() -> int:
     from dinfer_amd import Engine, SamplingParams
     from dinfer_amd.config.qwen3 import Qwen3Config
 
-    sizes = dict(SIZES)
+    sizes = {**SIZES, **SHAPES[a.shape]}
+    PROMPT, CONTEXT = a.prompt, a.context
+    if not 0 < PROMPT < CONTEXT:
+        print("--prompt must lie below --context")
+        return 2
     full_layers = sizes["num_hidden_layers"]
     if a.layers:
         sizes["num_hidden_layers"] = a.layers
@@ -137,12 +151,12 @@ def main() -> int:
             points[f"decode_b{b}"] = round(b / d, 1)
 
     line = {
-        "metric": "decode tok/s (Qwen3-8B shape, batch 8, 2048-token prompts, context 4096)",
+        "metric": f"decode tok/s (Qwen3-{a.shape.upper()} shape, batch {a.batch}, {PROMPT}-token prompts, context {CONTEXT})",
         "value": round(a.batch / dt, 1), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if a.dtype == "bfloat16" else "fp32", "data": "synthetic",
         "config": {
-            "model": "Qwen3-8B shape, random weights", "global_batch": a.batch, "seq_len": CONTEXT,
+            "model": f"Qwen3-{a.shape.upper()} shape, random weights", "global_batch": a.batch, "seq_len": CONTEXT,
             "prompt_len": PROMPT, "parallelism": "single GPU", "layers": sizes["num_hidden_layers"],
             "layers_of_config": full_layers, "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads,
             "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size,
