@@ -62,15 +62,19 @@ class _PoolView:
 
 
 class CacheManager:
-    def __init__(self, groups: list[GroupSpec], max_seqs: int):
+    def __init__(self, groups: list[GroupSpec], max_seqs: int, prefix_caching: bool = False):
+        """prefix_caching: full pages are named after the tokens of the prefix they end (needs groups that
+        keep every key, one page size); ``lookup`` and ``commit`` use the names."""
         self.groups = list(groups)
+        self.prefix_caching = bool(prefix_caching)
         if len(self.groups) > native.MAX_GROUPS:
             raise ValueError(f"{len(self.groups)} cache groups; at most {native.MAX_GROUPS} are supported")
         n = len(self.groups)
         arr = lambda vals: (_I32 * max(n, 1))(*vals)
         self._h = native.created("dh_cache_create", n, arr([g.page_size for g in self.groups]),
                                  arr([g.num_blocks for g in self.groups]),
-                                 arr([-1 if g.window is None else g.window for g in self.groups]), int(max_seqs))
+                                 arr([-1 if g.window is None else g.window for g in self.groups]), int(max_seqs),
+                                 int(self.prefix_caching))
         self.max_seqs = max_seqs
         self.pools = [_PoolView(self, g) for g in range(n)]
         self._handles: dict = {}          # request id -> the number the core knows it by
@@ -157,6 +161,21 @@ class CacheManager:
         native.checked("dh_cache_free", self._h, self.handle(req_id))
         if req_id not in self._pinned:
             del self._handles[req_id]
+
+    # ---- prefix cache --------------------------------------------------------------------------
+    def lookup(self, req_id, tokens: list) -> int:
+        """For an admitted request that holds no page yet: takes the cached pages that match the start of
+        its tokens (never all of them: the last token is always computed). Returns the tokens covered."""
+        arr = (_I32 * max(len(tokens), 1))(*tokens)
+        got = native.fn("dh_cache_lookup")(self._h, self.handle(req_id), arr, len(tokens))
+        if got < 0:
+            raise native.error(int(got), f"request {req_id!r}: ")
+        return int(got)
+
+    def commit(self, req_id, tokens: list, num_computed: int) -> None:
+        """After a step: names the pages that tokens[:num_computed] fill completely."""
+        arr = (_I32 * max(len(tokens), 1))(*tokens)
+        native.checked("dh_cache_commit", self._h, self.handle(req_id), arr, num_computed)
 
     # ---- views for the step --------------------------------------------------------------------
     def block_table(self, req_id, group: int) -> list[int]:

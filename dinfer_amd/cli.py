@@ -21,6 +21,11 @@ def _engine_flags(p: argparse.ArgumentParser) -> None:
     p.add_argument("--block-size", type=int, default=16, help="tokens per cache page")
     p.add_argument("--gpu-memory-utilization", type=float, default=0.9)
     p.add_argument("--no-decode-exempt", action="store_true", help="decode rows count against the token budget")
+    p.add_argument("--enable-prefix-caching", dest="prefix_caching", action="store_true",
+                   help="keep the pages of finished requests by their tokens; a prompt with the same start reuses them")
+    p.add_argument("--no-prefix-caching", dest="prefix_caching", action="store_false",
+                   help="do not reuse pages between requests (the default here)")
+    p.set_defaults(prefix_caching=False)
     p.add_argument("--long-prefill-token-threshold", type=int, default=0,
                    help="most prompt tokens of one request per step (0: no limit)")
     p.add_argument("--prefill-tokens-per-step", type=int, default=0,
@@ -36,6 +41,7 @@ def _options(a):
         dtype=a.dtype, max_model_len=a.max_model_len, max_num_seqs=a.max_num_seqs,
         max_num_batched_tokens=a.max_num_batched_tokens, num_blocks=a.num_blocks, block_size=a.block_size,
         gpu_memory_utilization=a.gpu_memory_utilization, decode_exempt_from_budget=not a.no_decode_exempt,
+        enable_prefix_caching=a.prefix_caching,
         long_prefill_token_threshold=a.long_prefill_token_threshold,
         prefill_tokens_per_step=a.prefill_tokens_per_step, hip_graph=not a.no_graph, device=a.device)
 

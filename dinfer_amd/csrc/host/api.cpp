@@ -92,12 +92,12 @@ int32_t dh_pool_check(void* pool) {
 
 // ---- cache manager
 void* dh_cache_create(int32_t n_groups, const int32_t* page_sizes, const int32_t* num_blocks, const int32_t* windows,
-                      int32_t max_seqs) {
+                      int32_t max_seqs, int32_t prefix_cache) {
     void* out = nullptr;
     guarded([&] {
         std::vector<GroupSpec> groups;
         for (int g = 0; g < n_groups; ++g) groups.push_back({page_sizes[g], num_blocks[g], windows[g]});
-        out = new CacheManager(std::move(groups), max_seqs);
+        out = new CacheManager(std::move(groups), max_seqs, prefix_cache != 0);
         return 0;
     });
     return out;
@@ -160,6 +160,14 @@ int32_t dh_cache_free_list(void* cache, int32_t group, int32_t* out, int32_t cap
 int32_t dh_cache_check(void* cache) {
     return guarded([&] { C(cache)->check(); return 0; });
 }
+int64_t dh_cache_lookup(void* cache, int64_t rid, const int32_t* tokens, int64_t n) {
+    int64_t got = 0;
+    const int32_t rc = guarded([&] { got = C(cache)->lookup(rid, tokens, n); return 0; });
+    return rc < 0 ? rc : got;
+}
+int32_t dh_cache_commit(void* cache, int64_t rid, const int32_t* tokens, int64_t num_computed) {
+    return guarded([&] { C(cache)->commit(rid, tokens, num_computed); return 0; });
+}
 
 // ---- batch
 int32_t dh_batch_fill(void* cache, const dh_batch_buffers* buf, int32_t n, const int64_t* rids, const int32_t* starts,
@@ -183,9 +191,14 @@ int32_t dh_batch_fill(void* cache, const dh_batch_buffers* buf, int32_t n, const
 
 // ---- scheduler
 void* dh_sched_create(const dh_sched_options* opt, void* cache, const int32_t* eos, int32_t n_eos) {
-    SchedOptions o;
-    std::memcpy(&o, opt, sizeof(o));
-    return new SchedulerBox(o, C(cache), eos, n_eos);
+    void* out = nullptr;
+    guarded([&] {
+        SchedOptions o;
+        std::memcpy(&o, opt, sizeof(o));
+        out = new SchedulerBox(o, C(cache), eos, n_eos);
+        return 0;
+    });
+    return out;
 }
 void dh_sched_destroy(void* sched) { delete S(sched); }
 
@@ -214,7 +227,7 @@ int32_t dh_sched_request_info(void* sched, int64_t rid, dh_request_info* out) {
     return guarded([&] {
         const Request* r = S(sched)->sched.get(rid);
         if (!r) throw Error(ERR_KEY, "the scheduler does not know the request");
-        *out = {r->num_prompt, r->num_tokens(), r->num_computed, r->status, r->reason, r->preemptions};
+        *out = {r->num_prompt, r->num_tokens(), r->num_computed, r->status, r->reason, r->preemptions, r->num_cached};
         return 0;
     });
 }

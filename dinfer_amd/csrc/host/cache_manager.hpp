@@ -15,6 +15,16 @@
 // keys all lie before the window of the request's next token; its block-table entry becomes
 // -1 and is never read again.
 //
+// Prefix cache (optional; crates/core/src/kv/hash.rs:20-60, kv/manager.rs:150-199,288-335). A full page
+// of a request's tokens gets a name: a hash of the tokens in it chained to the name of the page
+// before it, so a name stands for the whole prefix up to and including that page. commit() names
+// the pages a step has filled; lookup() gives a new request the longest run of named pages that
+// matches the start of its prompt (never all of it: the last token is always computed), so those
+// tokens need not be computed again. A named page that nobody holds waits at the tail of the
+// free list and is handed out last. Names are checked against the stored tokens and the
+// parent's name, so two prefixes whose hashes collide are still told apart. Only for groups
+// that keep every key (a window group gives pages back while the request lives).
+//
 // State slots (in the manner of crates/layers/src/exec.rs:253-333). Each live request holds
 // one index in [0, max_seqs) for its whole life. A slot handed out is reported by
 // take_fresh_slots() so that the engine zero-fills its state before the first step that uses it.
@@ -38,14 +48,28 @@ struct GroupSpec {
 
 class CacheManager {
 public:
-    CacheManager(std::vector<GroupSpec> groups, int max_seqs) : groups_(std::move(groups)), max_seqs_(max_seqs) {
+    CacheManager(std::vector<GroupSpec> groups, int max_seqs, bool prefix_cache = false)
+        : groups_(std::move(groups)), max_seqs_(max_seqs), prefix_cache_(prefix_cache) {
         if (max_seqs <= 0) throw Error(ERR_VALUE, "max_seqs must be positive");
         for (const GroupSpec& g : groups_) {
             if (g.page_size <= 0) throw Error(ERR_VALUE, "a page holds at least one token");
             pools_.emplace_back(g.num_blocks);
         }
         for (int s = max_seqs - 1; s >= 0; --s) free_slots_.push_back(s);
+        if (prefix_cache_) {
+            if (groups_.empty()) throw Error(ERR_VALUE, "a prefix cache needs a cache group");
+            for (const GroupSpec& g : groups_) {
+                if (g.window >= 0) throw Error(ERR_VALUE, "the prefix cache needs groups that keep every key");
+                if (g.page_size != groups_[0].page_size)
+                    throw Error(ERR_VALUE, "the prefix cache needs one page size in all groups");
+                named_tokens_.emplace_back(static_cast<size_t>(g.num_blocks) * g.page_size, 0);
+                named_parent_.emplace_back(g.num_blocks, 0);
+                named_check_.emplace_back(g.num_blocks, 0);
+            }
+        }
     }
+
+    bool prefix_cache() const { return prefix_cache_; }
 
     int num_groups() const { return static_cast<int>(groups_.size()); }
     int max_seqs() const { return max_seqs_; }
@@ -148,6 +172,68 @@ public:
         reqs_.erase(it);
     }
 
+    // ---- prefix cache
+    // For a request that holds no page yet: takes the longest run of named pages matching the start of
+    // tokens[0, n), at most (n - 1) / page_size of them, and returns how many tokens they cover.
+    int64_t lookup(int64_t rid, const int32_t* tokens, int64_t n) {
+        Req& r = find(rid);
+        if (!prefix_cache_) return 0;
+        for (const auto& t : r.tables)
+            if (!t.empty()) throw Error(ERR_RUNTIME, "a prefix is looked up before the request holds pages");
+        const int ps = groups_[0].page_size;
+        const int64_t most = n > 0 ? (n - 1) / ps : 0;
+        uint64_t name = 0, chk = 0;
+        int64_t got = 0;
+        std::vector<int32_t> hit(groups_.size());
+        for (; got < most; ++got) {
+            uint64_t nn, nc;
+            name_page(name, chk, tokens + got * ps, ps, &nn, &nc);
+            bool all = true;
+            for (size_t g = 0; g < groups_.size() && all; ++g) {
+                const int b = pools_[g].find(nn);
+                all = b >= 0 && named_check_[g][b] == nc && named_parent_[g][b] == name &&
+                      std::equal(tokens + got * ps, tokens + (got + 1) * ps, named_tokens_[g].begin() + static_cast<size_t>(b) * ps);
+                hit[g] = b;
+            }
+            if (!all) break;
+            for (size_t g = 0; g < groups_.size(); ++g) {
+                pools_[g].touch(hit[g]);
+                r.tables[g].push_back(hit[g]);
+            }
+            name = nn;
+            chk = nc;
+        }
+        r.num_named = got;
+        r.last_name = name;
+        r.last_check = chk;
+        r.num_tokens = got * ps;
+        return got * ps;
+    }
+
+    // After a step: the pages that tokens[0, num_computed) fill completely get their names.
+    void commit(int64_t rid, const int32_t* tokens, int64_t num_computed) {
+        if (!prefix_cache_) return;
+        Req& r = find(rid);
+        const int ps = groups_[0].page_size;
+        const int64_t full = num_computed / ps;
+        for (; r.num_named < full; ++r.num_named) {
+            const int64_t i = r.num_named;
+            uint64_t nn, nc;
+            name_page(r.last_name, r.last_check, tokens + i * ps, ps, &nn, &nc);
+            for (size_t g = 0; g < groups_.size(); ++g) {
+                const int b = r.tables[g].at(i);
+                // if another page carries the name already, this one stays nameless (its content is a duplicate)
+                if (!pools_[g].has_name(b) && pools_[g].set_name(b, nn)) {
+                    named_check_[g][b] = nc;
+                    named_parent_[g][b] = r.last_name;
+                    std::copy(tokens + i * ps, tokens + (i + 1) * ps, named_tokens_[g].begin() + static_cast<size_t>(b) * ps);
+                }
+            }
+            r.last_name = nn;
+            r.last_check = nc;
+        }
+    }
+
     // ---- views for the step
     const std::vector<int32_t>& block_table(int64_t rid, int g) const { return find(rid).tables.at(g); }
 
@@ -172,22 +258,28 @@ public:
         for (size_t g = 0; g < groups_.size(); ++g) {
             const BlockPool& pool = pools_[g];
             pool.check();
-            std::vector<uint8_t> seen(pool.num_blocks(), 0);
-            int n_seen = 0;
+            // a page is in as many block tables as it has references (more than one only for shared prefixes)
+            std::vector<int32_t> uses(pool.num_blocks(), 0);
             for (const auto& kv : reqs_) {
                 for (int32_t b : kv.second.tables[g]) {
                     if (b < 0) continue;
                     std::string where = "group " + std::to_string(g) + ": page " + std::to_string(b);
                     if (b >= pool.num_blocks()) throw Error(ERR_ASSERT, where + " does not exist");
-                    if (seen[b]) throw Error(ERR_ASSERT, where + " is in two block tables");
                     if (!pool.is_held(b)) throw Error(ERR_ASSERT, where + " of a live request is on the free list");
-                    seen[b] = 1;
-                    ++n_seen;
+                    if (++uses[b] > 1 && !prefix_cache_) throw Error(ERR_ASSERT, where + " is in two block tables");
                 }
             }
-            if (n_seen + pool.num_free() != pool.num_blocks())
+            int held = 0;
+            for (int b = 0; b < pool.num_blocks(); ++b) {
+                if (uses[b] != pool.ref_count(b))
+                    throw Error(ERR_ASSERT, "group " + std::to_string(g) + ": page " + std::to_string(b) + " is in " +
+                                                std::to_string(uses[b]) + " block tables and has " +
+                                                std::to_string(pool.ref_count(b)) + " references");
+                held += uses[b] > 0;
+            }
+            if (held + pool.num_free() != pool.num_blocks())
                 throw Error(ERR_ASSERT, "group " + std::to_string(g) + ": " +
-                                            std::to_string(pool.num_blocks() - pool.num_free() - n_seen) + " pages are lost");
+                                            std::to_string(pool.num_blocks() - pool.num_free() - held) + " pages are lost");
         }
         std::vector<uint8_t> slot_seen(max_seqs_, 0);
         size_t n = 0;
@@ -206,6 +298,8 @@ private:
         std::vector<std::vector<int32_t>> tables;
         int64_t num_tokens = 0;  // tokens for which pages have been allocated
         int slot = -1;
+        int64_t num_named = 0;   // leading pages that carry a name (or were tried)
+        uint64_t last_name = 0, last_check = 0;  // of page num_named - 1
     };
 
     const Req& find(int64_t rid) const {
@@ -220,6 +314,30 @@ private:
     int max_seqs_;
     std::vector<int> free_slots_, fresh_slots_;
     std::unordered_map<int64_t, Req> reqs_;
+    // Two independent 64-bit hashes of (the parent's two, the page's tokens): one is the name, the other
+    // is kept beside the page and compared on a hit.
+    static uint64_t mix(uint64_t x) {
+        x += 0x9e3779b97f4a7c15ull;
+        x = (x ^ (x >> 30)) * 0xbf58476d1ce4e5b9ull;
+        x = (x ^ (x >> 27)) * 0x94d049bb133111ebull;
+        return x ^ (x >> 31);
+    }
+    static void name_page(uint64_t parent, uint64_t parent_check, const int32_t* tokens, int n, uint64_t* name,
+                          uint64_t* check) {
+        uint64_t a = mix(parent ^ 0x243f6a8885a308d3ull), b = mix(parent_check ^ 0x13198a2e03707344ull);
+        for (int i = 0; i < n; ++i) {
+            const uint64_t t = static_cast<uint32_t>(tokens[i]);
+            a = mix(a ^ t);
+            b = mix(b + (t << 1 | 1) * 0xa4093822299f31d0ull);
+        }
+        *name = a;
+        *check = b;
+    }
+
+    bool prefix_cache_ = false;
+    std::vector<std::vector<int32_t>> named_tokens_;   // per group: [page][page_size] tokens of named pages
+    std::vector<std::vector<uint64_t>> named_parent_;  // per group: the name of the page before
+    std::vector<std::vector<uint64_t>> named_check_;   // per group: the second hash
     std::vector<int> need_;
     std::vector<int32_t> scratch_;
 };

@@ -24,9 +24,10 @@ int32_t dh_pool_free_list(void* pool, int32_t* out, int32_t capacity);   /* retu
 int32_t dh_pool_is_held(void* pool, int32_t page);
 int32_t dh_pool_check(void* pool);
 
-/* ---- cache manager. windows[g] < 0: the group keeps every key */
+/* ---- cache manager. windows[g] < 0: the group keeps every key. prefix_cache: pages are named after the
+ * tokens they hold, so that a later request with the same start need not compute them again */
 void* dh_cache_create(int32_t n_groups, const int32_t* page_sizes, const int32_t* num_blocks, const int32_t* windows,
-                      int32_t max_seqs);
+                      int32_t max_seqs, int32_t prefix_cache);
 void dh_cache_destroy(void* cache);
 int32_t dh_cache_has(void* cache, int64_t rid);
 int32_t dh_cache_can_admit(void* cache);
@@ -43,6 +44,10 @@ int32_t dh_cache_slot_mapping(void* cache, int64_t rid, int32_t group, int64_t s
 int32_t dh_cache_num_free(void* cache, int32_t group);
 int32_t dh_cache_free_list(void* cache, int32_t group, int32_t* out, int32_t capacity);
 int32_t dh_cache_check(void* cache);
+/* prefix cache: tokens of the request from its first; lookup returns how many of them are covered by cached pages
+ * (the request must be admitted and hold no page yet); commit names the pages that tokens[0, num_computed) fill */
+int64_t dh_cache_lookup(void* cache, int64_t rid, const int32_t* tokens, int64_t n);
+int32_t dh_cache_commit(void* cache, int64_t rid, const int32_t* tokens, int64_t num_computed);
 
 /* ---- the flat batch of a step, written into the caller's pinned buffer */
 #define DH_MAX_GROUPS 8
@@ -72,13 +77,13 @@ int32_t dh_batch_fill(void* cache, const dh_batch_buffers* buf, int32_t n, const
 /* ---- scheduler */
 typedef struct {
     int32_t max_num_batched_tokens, max_num_seqs, max_model_len, prefill_tokens_per_step,
-        long_prefill_token_threshold, enable_chunked_prefill, decode_exempt_from_budget;
+        long_prefill_token_threshold, enable_chunked_prefill, decode_exempt_from_budget, enable_prefix_caching;
 } dh_sched_options;
 
 typedef struct { int64_t id; int32_t start, num_new, samples; } dh_scheduled;
 typedef struct { int64_t id; int32_t token, reason; } dh_update_result;
 /* status: 0 waiting, 1 running, 2 preempted, 3 finished. reason: 0 none, 1 stop, 2 length, 3 abort */
-typedef struct { int32_t num_prompt, num_tokens, num_computed, status, reason, preemptions; } dh_request_info;
+typedef struct { int32_t num_prompt, num_tokens, num_computed, status, reason, preemptions, num_cached; } dh_request_info;
 
 void* dh_sched_create(const dh_sched_options* opt, void* cache, const int32_t* eos, int32_t n_eos);
 void dh_sched_destroy(void* sched);

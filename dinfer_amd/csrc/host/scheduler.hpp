@@ -38,6 +38,7 @@ struct SchedOptions {
     int32_t long_prefill_token_threshold;  // 0: no cap
     int32_t enable_chunked_prefill;
     int32_t decode_exempt_from_budget;
+    int32_t enable_prefix_caching;  // needs a cache manager built with a prefix cache
 };
 
 enum Status : int32_t { WAITING = 0, RUNNING = 1, PREEMPTED = 2, FINISHED = 3 };
@@ -54,6 +55,7 @@ struct Request {
     bool ignore_eos = false;
     std::vector<int32_t> stop_ids;
     int32_t preemptions = 0;
+    int32_t num_cached = 0;  // tokens of the prompt found in the prefix cache at the last admission
 
     int32_t num_tokens() const { return static_cast<int32_t>(tokens.size()); }
     int32_t num_output() const { return num_tokens() - num_prompt; }
@@ -81,7 +83,10 @@ struct UpdateResult {
 class Scheduler {
 public:
     Scheduler(const SchedOptions& opt, CacheManager* cache, const int32_t* eos, int n_eos)
-        : opt_(opt), cache_(cache), eos_(eos, eos + n_eos) {}
+        : opt_(opt), cache_(cache), eos_(eos, eos + n_eos) {
+        if (opt_.enable_prefix_caching && !cache_->prefix_cache())
+            throw Error(ERR_VALUE, "prefix caching is asked for but the cache manager was built without it");
+    }
 
     // ---- intake
     void add(std::unique_ptr<Request> req) {
@@ -176,16 +181,22 @@ public:
         if (!preempted_any) {
             while (budget > 0 && !waiting_.empty() && static_cast<int>(running_.size()) < opt_.max_num_seqs) {
                 Request* r = waiting_.front();
+                if (!cache_->can_admit()) break;
+                cache_->admit(r->id);
+                // a prefix of the prompt (or, after a preemption, of prompt and outputs) may be in the cache
+                // still: those tokens are not computed again (:564-570)
+                if (opt_.enable_prefix_caching && r->num_computed == 0) {
+                    r->num_cached = static_cast<int32_t>(cache_->lookup(r->id, r->tokens.data(), r->num_tokens()));
+                    r->num_computed = r->num_cached;
+                }
                 const int64_t remaining = r->num_tokens() - r->num_computed;
                 int64_t n = remaining;
                 if (threshold && n > threshold) n = threshold;
                 n = std::min(n, std::min(budget, quota));
                 if (n < remaining && !opt_.enable_chunked_prefill) n = 0;
-                if (n <= 0) break;
-                if (!cache_->can_admit()) break;
-                cache_->admit(r->id);
-                if (!cache_->allocate(r->id, r->num_computed, n)) {
-                    cache_->free(r->id);  // no pages now: wait
+                if (n <= 0 || !cache_->allocate(r->id, r->num_computed, n)) {
+                    cache_->free(r->id);  // no budget or no pages now: wait (what was found stays cached)
+                    if (opt_.enable_prefix_caching) r->num_computed = r->num_cached = 0;
                     break;
                 }
                 waiting_.pop_front();
@@ -215,6 +226,7 @@ public:
             if (it == reqs_.end() || it->second->status != RUNNING) continue;  // preempted or aborted meanwhile
             Request* r = it->second.get();
             cache_->release_passed(r->id, r->num_computed);
+            if (opt_.enable_prefix_caching) cache_->commit(r->id, r->tokens.data(), r->num_computed);
             int32_t tok = -1;
             Reason reason = NO_REASON;
             if (s.samples) {

@@ -28,6 +28,7 @@ class Request:
         self._status = WAITING
         self._finish_reason: str | None = None
         self._num_preemptions = 0
+        self._num_cached = 0
 
     def __repr__(self) -> str:
         return (f"Request(id={self.id!r}, prompt={self.num_prompt}, outputs={self.num_output}, "
@@ -57,10 +58,17 @@ class Request:
         info = self._live()
         return info.preemptions if info else self._num_preemptions
 
+    @property
+    def num_cached_tokens(self) -> int:
+        """Tokens found in the prefix cache when the request was last admitted (not computed again)."""
+        info = self._live()
+        return info.num_cached if info else self._num_cached
+
     def _detach(self, info) -> None:
         """Keeps the last state when the scheduler lets the request go."""
         self._num_computed, self._status = info.num_computed, STATUS_NAMES[info.status]
         self._finish_reason, self._num_preemptions = REASON_NAMES[info.reason], info.preemptions
+        self._num_cached = info.num_cached
         self._owner = None
 
     # ---- tokens

@@ -127,7 +127,7 @@ class ModelRunner:
                                f"pages, the pool has {num_blocks}")
         self.num_blocks = int(num_blocks)
         self.group_specs = [GroupSpec(self.page_size, self.num_blocks, window=k[3]) for k in keys]
-        self.cache = CacheManager(self.group_specs, opt.max_num_seqs)
+        self.cache = CacheManager(self.group_specs, opt.max_num_seqs, prefix_caching=opt.enable_prefix_caching)
         self.cache_views: list[CacheView] = []
         self.state_tensors: list[torch.Tensor] = []
         own: dict[int, CacheView] = {}

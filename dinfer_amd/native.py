@@ -30,7 +30,7 @@ class BatchFacts(Structure):
 class SchedOptions(Structure):
     _fields_ = [(n, _I) for n in ("max_num_batched_tokens", "max_num_seqs", "max_model_len", "prefill_tokens_per_step",
                                   "long_prefill_token_threshold", "enable_chunked_prefill",
-                                  "decode_exempt_from_budget")]
+                                  "decode_exempt_from_budget", "enable_prefix_caching")]
 
 
 class Scheduled(Structure):
@@ -42,7 +42,8 @@ class UpdateResult(Structure):
 
 
 class RequestInfo(Structure):
-    _fields_ = [(n, _I) for n in ("num_prompt", "num_tokens", "num_computed", "status", "reason", "preemptions")]
+    _fields_ = [(n, _I) for n in ("num_prompt", "num_tokens", "num_computed", "status", "reason", "preemptions",
+                                  "num_cached")]
 
 
 _SIGNATURES = {
@@ -54,7 +55,9 @@ _SIGNATURES = {
     "dh_pool_free_list": (_I, [_P, _P, _I]),
     "dh_pool_is_held": (_I, [_P, _I]),
     "dh_pool_check": (_I, [_P]),
-    "dh_cache_create": (_P, [_I, _P, _P, _P, _I]),
+    "dh_cache_create": (_P, [_I, _P, _P, _P, _I, _I]),
+    "dh_cache_lookup": (_L, [_P, _L, _P, _L]),
+    "dh_cache_commit": (_I, [_P, _L, _P, _L]),
     "dh_cache_destroy": (None, [_P]),
     "dh_cache_has": (_I, [_P, _L]),
     "dh_cache_can_admit": (_I, [_P]),

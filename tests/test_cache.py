@@ -149,3 +149,98 @@ def test_random_orders_keep_the_invariants(seed, window):
         m.free(rid)
     m.check()
     assert m.num_free(0) == 40 and m.num_free(1) == 40
+
+
+# ---- prefix cache ----------------------------------------------------------------------------------
+def pmgr(blocks=8, page=4, seqs=4):
+    return CacheManager([GroupSpec(page, blocks)], seqs, prefix_caching=True)
+
+
+def run_request(m, rid, tokens, keep=False):
+    """Admits, looks the prefix up, allocates and commits the rest; returns the tokens found cached."""
+    m.admit(rid)
+    got = m.lookup(rid, tokens)
+    assert m.allocate(rid, got, len(tokens) - got)
+    m.commit(rid, tokens, len(tokens))
+    if not keep:
+        m.free(rid)
+    m.check()
+    return got
+
+
+def test_prefix_is_found_again_but_never_the_whole_prompt():
+    """kv/manager.rs:150-199: full pages only, and at most (n - 1) / page of them."""
+    m = pmgr()
+    a = list(range(100, 110))                       # 10 tokens: two full pages and a half
+    assert run_request(m, "a", a) == 0
+    assert run_request(m, "b", a) == 8              # both full pages
+    assert run_request(m, "c", a[:8]) == 4          # 8 tokens: the last one must be computed, so one page
+    assert run_request(m, "d", a[:5] + [7] + a[6:]) == 4   # differs inside the second page
+    assert run_request(m, "e", [1] + a[1:]) == 0    # differs in the first page: nothing, though later pages match
+
+
+def test_shared_pages_have_two_holders():
+    m = pmgr()
+    a = list(range(20))
+    run_request(m, "a", a, keep=True)
+    assert run_request(m, "b", a[:13] + [99], keep=True) == 12
+    ta, tb = m.block_table("a", 0), m.block_table("b", 0)
+    assert ta[:3] == tb[:3] and ta[3] != tb[3]
+    m.free("a")
+    m.check()
+    assert m.block_table("b", 0) == tb and m.num_free() == 8 - 4   # b still holds the shared pages
+    m.free("b")
+    m.check()
+    assert m.num_free() == 8
+
+
+def test_named_pages_are_evicted_last_and_oldest_first():
+    """kv/block_pool.rs:160-182: nameless pages return to the head, named ones to the tail; a request is
+    freed last page first, so its tail is evicted before its head (kv/manager.rs:338-345)."""
+    m = pmgr(blocks=6)
+    a = list(range(50, 62))                         # three full pages: 0, 1, 2
+    run_request(m, "a", a + [1])                    # and one token in page 3 (nameless)
+    assert m.pools[0].free_list() == [3, 4, 5, 2, 1, 0]
+    m.admit("x")
+    assert m.allocate("x", 0, 16)                   # takes 3, 4, 5 and the youngest-freed named page, 2
+    assert m.block_table("x", 0) == [3, 4, 5, 2]
+    m.free("x")                                     # nameless now: back at the head, last page first
+    assert m.pools[0].free_list() == [2, 5, 4, 3, 1, 0]
+    assert run_request(m, "b", a + [1], keep=True) == 8     # pages 0 and 1 are still named, 2 is not
+    m.check()
+
+
+def test_random_prefix_traffic_keeps_the_invariants():
+    rng = random.Random(3)
+    m = CacheManager([GroupSpec(4, 24), GroupSpec(4, 30)], 4, prefix_caching=True)
+    stems = [[rng.randrange(50) for _ in range(40)] for _ in range(3)]
+    live, hits = {}, 0
+    for step in range(500):
+        if live and (len(live) == 4 or rng.random() < 0.4):
+            rid = rng.choice(list(live))
+            m.free(rid)
+            del live[rid]
+        else:
+            toks = rng.choice(stems)[:rng.randrange(1, 40)] + [rng.randrange(50) for _ in range(rng.randrange(0, 6))]
+            rid = f"r{step}"
+            m.admit(rid)
+            got = m.lookup(rid, toks)
+            assert got % 4 == 0 and got < len(toks)
+            hits += got
+            if m.allocate(rid, got, len(toks) - got):
+                m.commit(rid, toks, len(toks))
+                assert m.slot_mapping(rid, 0, 0, len(toks)) and m.slot_mapping(rid, 1, 0, len(toks))
+                live[rid] = toks
+            else:
+                m.free(rid)
+        m.check()
+    assert hits > 500
+    for rid in list(live):
+        m.free(rid)
+    m.check()
+    assert m.num_free(0) == 24 and m.num_free(1) == 30
+
+
+def test_prefix_cache_refuses_window_groups():
+    with pytest.raises(ValueError, match="every key"):
+        CacheManager([GroupSpec(4, 8, 6)], 2, prefix_caching=True)

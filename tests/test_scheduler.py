@@ -233,3 +233,102 @@ def test_random_loads_keep_every_rule():
             assert r.status == "finished" and r.finish_reason == LENGTH and r.num_output == r.sampling.max_tokens, r
         assert s.cache.num_free() == blocks and not s.requests
     assert preemptions > 10
+
+
+# ---- prefix caching ---------------------------------------------------------------------------------
+def mkp(max_seqs, budget, blocks, **kw):
+    kw = {"max_model_len": 4096, "decode_exempt_from_budget": False, "enable_prefix_caching": True, **kw}
+    opt = EngineOptions(max_num_seqs=max_seqs, max_num_batched_tokens=budget, block_size=16, num_blocks=blocks, **kw)
+    cache = CacheManager([GroupSpec(16, blocks)], max_seqs, prefix_caching=True)
+    return Scheduler(opt, cache, eos_token_ids=[2])
+
+
+def same_prompt(i, n, max_tokens):
+    return Request(i, list(range(500, 500 + n)), SamplingParams(max_tokens=max_tokens))
+
+
+def test_second_request_with_the_same_prompt_skips_the_cached_pages():
+    """sched/mod.rs:564-570 with kv/manager.rs:150-199: 40 tokens, pages of 16: the second request finds
+    32 tokens cached and feeds 8."""
+    s = mkp(4, 100, 16)
+    r1, r2 = same_prompt(1, 40, 3), same_prompt(2, 40, 2)
+    s.add_request(r1)
+    assert step(s, {1: 7})[0] == [(1, 40)]
+    s.add_request(r2)
+    sched, out, _ = step(s, {1: 7, 2: 7})
+    assert sched == [(1, 1), (2, 8)] and out.scheduled[1].start == 32
+    assert r2.num_cached_tokens == 32 and r1.num_cached_tokens == 0
+    t1, t2 = s.cache.block_table(1, 0), s.cache.block_table(2, 0)
+    assert t1[:2] == t2[:2] and t1[2] != t2[2]
+    step(s, {1: 7, 2: 7})
+    assert not s.has_unfinished() and s.cache.num_free() == 16
+
+
+def test_a_prompt_that_is_cached_whole_still_computes_its_last_token():
+    s = mkp(4, 100, 16)
+    s.add_request(same_prompt(1, 32, 1))
+    step(s, {1: 7})
+    r2 = same_prompt(2, 32, 1)
+    s.add_request(r2)
+    sched, out, _ = step(s, {2: 7})
+    assert sched == [(2, 16)] and out.scheduled[0].start == 16 and r2.num_cached_tokens == 16
+
+
+def test_preempted_request_finds_its_own_pages_again():
+    """Without a prefix cache a preempted request replays everything (sched/mod.rs:979-991); with it, the
+    pages that were not handed out meanwhile are still there."""
+    s = mkp(4, 100, 5)
+    r1, r2 = req(1, 32, 20), req(2, 31, 40)
+    s.add_request(r1)
+    s.add_request(r2)
+    assert step(s, {1: 5, 2: 5})[0] == [(1, 32), (2, 31)]          # pages 0, 1 and 2, 3; page 4 is free
+    assert step(s, {1: 5, 2: 5})[0] == [(1, 1), (2, 1)]            # request 1 takes page 4, request 2 fills page 3
+    # request 2 needs a page and is the last one running: it is skipped while request 1 goes on ...
+    for _ in range(15):
+        sched, out, _ = step(s, {1: 5})
+        assert sched == [(1, 1)] and not out.preempted
+    # ... until request 1 needs a page itself: request 2 is preempted, its two full pages go to the tail
+    sched, out, _ = step(s, {1: 5})
+    assert sched == [(1, 1)] and out.preempted == [2] and r2.num_computed == 0
+    while r1.status != "finished":
+        step(s, {1: 5})
+    # request 1 took the younger of the two pages (the tail of request 2 is evicted first); the other is found again
+    sched, out, _ = step(s, {2: 5})
+    assert sched == [(2, 33 - 16)] and out.scheduled[0].start == 16 and r2.num_cached_tokens == 16
+    assert r2.num_preemptions == 1
+
+
+def test_random_loads_with_prefix_caching_keep_every_rule():
+    import random
+    cached = 0
+    for seed in range(6):
+        rng = random.Random(100 + seed)
+        budget, max_seqs, blocks = rng.choice([8, 24, 64]), rng.choice([2, 3, 5]), rng.choice([8, 12, 20])
+        s = mkp(max_seqs, budget, blocks, decode_exempt_from_budget=bool(seed % 2), max_model_len=blocks * 16)
+        stems = [[rng.randrange(1000) + 10 for _ in range(70)] for _ in range(2)]
+        todo = []
+        for i in range(14):
+            p = rng.choice(stems)[:rng.randrange(1, 60)] + [rng.randrange(1000) + 10 for _ in range(rng.randrange(0, 4))]
+            mt = rng.randrange(1, 20)
+            if len(p) + mt <= blocks * 16 - 16:
+                todo.append(Request(i, p, SamplingParams(max_tokens=mt)))
+        everyone = list(todo)
+        steps = 0
+        while todo or s.has_unfinished():
+            steps += 1
+            assert steps < 5000
+            while todo and rng.random() < 0.4:
+                s.add_request(todo.pop())
+            out = s.schedule()
+            charged = sum(x.num_new for x in out.scheduled
+                          if not (s.opt.decode_exempt_from_budget and x.num_new == 1 and x.start > 0))
+            assert charged <= budget and len(s.running) <= max_seqs
+            for x in out.scheduled:
+                assert x.num_new >= 1 and x.samples == (x.start + x.num_new == x.request.num_tokens)
+            s.update(out, {x.request.id: 3 for x in out.scheduled if x.samples})
+            s.cache.check()
+        for r in everyone:
+            assert r.status == "finished" and r.num_output == r.sampling.max_tokens, r
+            cached += r.num_cached_tokens
+        assert s.cache.num_free() == blocks and not s.requests
+    assert cached > 200
