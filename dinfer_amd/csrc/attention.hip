@@ -141,19 +141,24 @@ struct Tile {
   // Loads are unconditional: a key outside [k_lo, k_hi) is replaced by the nearest key inside, which
   // lies in a page the request holds, so straight-line code with all loads in flight at once. What
   // was loaded for such a key never counts: its score is masked, and accumulate() zeroes its value.
+  // CLAMP = false: the block lies wholly inside [k_lo, k_hi), so no key needs replacing.
+  template <bool CLAMP>
   __device__ __forceinline__ void load_k(Frags<DT>& f, int kb) {
     constexpr int D = DT * 16;
     const int lane = threadIdx.x & 63, i16 = lane & 15, g4 = lane >> 4;
     const int last = k_hi - 1;
-    // K rows of this lane: keys kg_row + (i16 & 3) and + 4, in one page (page size % 8 == 0)
+    // K rows of this lane: keys kg_row + (i16 & 3) and + 4: one aligned group of 8, so one page (page size % 8 == 0)
     int key0 = kb + 8 * (i16 >> 2) + (i16 & 3), key1 = key0 + 4;
-    key0 = key0 < k_lo ? k_lo : (key0 > last ? last : key0);
-    key1 = key1 < k_lo ? k_lo : (key1 > last ? last : key1);
-    const int pg0 = pages.get(pages.page_of(key0)), pg1 = pages.get(pages.page_of(key1));
+    if (CLAMP) {
+      key0 = key0 < k_lo ? k_lo : (key0 > last ? last : key0);
+      key1 = key1 < k_lo ? k_lo : (key1 > last ? last : key1);
+    }
+    const int pg0 = pages.get(pages.page_of(key0));
+    const int pg1 = CLAMP ? pages.get(pages.page_of(key1)) : pg0;  // clamping may move the two into different pages
     // K pages are [Hkv][D / 8][page][8]: the 16-byte pieces of consecutive keys lie next to each other,
     // so the four lanes of a quad (four consecutive keys, one piece index) read 64 contiguous bytes
     const bf16* kr0 = kc + ((int64_t)pg0 * page_stride + (head_off + pages.offset_of(key0) * 8));
-    const bf16* kr1 = kc + ((int64_t)pg1 * page_stride + (head_off + pages.offset_of(key1) * 8));
+    const bf16* kr1 = CLAMP ? kc + ((int64_t)pg1 * page_stride + (head_off + pages.offset_of(key1) * 8)) : kr0 + 32;
     const int piece = pages.ps * 8;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -166,23 +171,27 @@ struct Tile {
     }
   }
 
+  template <bool CLAMP>
   __device__ __forceinline__ void load_v(Frags<DT>& f, int kb) {
     const int lane = threadIdx.x & 63, i16 = lane & 15, g4 = lane >> 4;
     const int ps = pages.ps;
     // V^T rows of this lane: d = 16 dt + i16, keys kg .. kg + 7 (one page)
     int kg = kb + 8 * g4;
-    const int g_lo = k_lo & ~7, g_hi = (k_hi - 1) & ~7;
-    kg = kg < g_lo ? g_lo : (kg > g_hi ? g_hi : kg);
+    if (CLAMP) {
+      const int g_lo = k_lo & ~7, g_hi = (k_hi - 1) & ~7;
+      kg = kg < g_lo ? g_lo : (kg > g_hi ? g_hi : kg);
+    }
     const int pgv = pages.get(pages.page_of(kg));
     const bf16* vrow = vc + ((int64_t)pgv * page_stride + (head_off + i16 * ps + pages.offset_of(kg)));
 #pragma unroll
     for (int d = 0; d < DT; ++d) f.v[d] = ld16<STREAM>(vrow + d * 16 * ps);
   }
 
+  template <bool CLAMP>
   __device__ __forceinline__ void load(Frags<DT>& f, int kb) {
     pages.ensure(kb);
-    load_k(f, kb);
-    load_v(f, kb);
+    load_k<CLAMP>(f, kb);
+    load_v<CLAMP>(f, kb);
   }
 
   // S^T of one block: s[t][a] holds, for column i16 of tile t, the keys kb + 8 g4 + 4 a + {0..3}
@@ -288,11 +297,13 @@ struct Tile {
     Frags<DT> f;
 #pragma nounroll
     for (int kb = k_lo & ~31; kb < k_hi; kb += 32) {
-      load(f, kb);
-      if (!TWO_BODIES || mask(kb))
+      if (!TWO_BODIES || mask(kb)) {
+        load<true>(f, kb);
         compute<true>(f, qf, kb, col_lo, col_hi);
-      else
+      } else {
+        load<false>(f, kb);
         compute<false>(f, qf, kb, col_lo, col_hi);
+      }
     }
   }
 
