@@ -9,7 +9,7 @@
 //   s_j = scale * <q, k_j>;  P = softmax(s);  o = sum_j P_j v_j   (all float)
 //
 // K and V are read from the cache pages through the request's block table
-// (K page [Hkv][page][D], V page [Hkv][D][page]); the step's own tokens were
+// (K page [Hkv][D / 8][page][8], V page [Hkv][D][page]); the step's own tokens were
 // written there before this kernel runs.
 //
 // Reference behaviour: crates/kernels/cuda/gqa.cu:1037-1118 (plain paged

@@ -11,7 +11,7 @@
 //
 // Cache pages (chosen for MFMA operand loads on gfx950: both operands of
 // Q.K^T and P.V want 8 consecutive elements of the contraction dimension):
-//   K page  [Hkv][page][D]   a key's head is one contiguous row of D
+//   K page  [Hkv][D / 8][page][8]   the 8-element pieces of consecutive keys are contiguous
 //   V page  [Hkv][D][page]   transposed: for one d, the page's keys are contiguous
 // A token's slot is block * page + offset; a negative slot writes nothing.
 //
