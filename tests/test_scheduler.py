@@ -332,3 +332,38 @@ def test_random_loads_with_prefix_caching_keep_every_rule():
             cached += r.num_cached_tokens
         assert s.cache.num_free() == blocks and not s.requests
     assert cached > 200
+
+
+def test_request_ids_can_be_used_again_and_aborts_free_everything():
+    s = mk(4, 100, 16)
+    a = req(1, 20, 5)
+    s.add_request(a)
+    import pytest
+    with pytest.raises(KeyError):
+        s.add_request(req(1, 3, 1))                  # the id is live
+    step(s, {1: 9})
+    s.abort(1)                                       # while running
+    assert a.status == "finished" and a.finish_reason == "abort" and not s.has_unfinished()
+    assert s.cache.num_free() == 16 and not s.cache.has(1)
+    b = req(1, 7, 2)                                 # the same id again, a different request
+    s.add_request(b)
+    s.add_request(req(2, 5, 2))
+    s.abort(2)                                       # while waiting
+    assert [r.id for r in s.waiting] == [1]
+    assert step(s, {1: 9})[0] == [(1, 7)] and b.num_computed == 7 and a.num_computed == 20
+    s.abort(99)                                      # unknown: nothing happens
+    step(s, {1: 9})
+    assert not s.has_unfinished() and s.cache.num_free() == 16
+    s.cache.check()
+
+
+def test_abort_between_schedule_and_update_drops_the_sample():
+    s = mk(4, 100, 16)
+    s.add_request(req(1, 4, 5))
+    s.add_request(req(2, 4, 5))
+    out = s.schedule()
+    s.abort(1)
+    res = s.update(out, {1: 7, 2: 8})                # the token for request 1 is ignored
+    assert [(r.id, t) for r, t, _ in res] == [(2, 8)]
+    s.cache.check()
+    assert s.cache.num_free() == 15
