@@ -24,8 +24,8 @@ def _engine_flags(p: argparse.ArgumentParser) -> None:
     p.add_argument("--enable-prefix-caching", dest="prefix_caching", action="store_true",
                    help="keep the pages of finished requests by their tokens; a prompt with the same start reuses them")
     p.add_argument("--no-prefix-caching", dest="prefix_caching", action="store_false",
-                   help="do not reuse pages between requests (the default here)")
-    p.set_defaults(prefix_caching=False)
+                   help="do not reuse pages between requests (default: reuse where every layer keeps all its keys)")
+    p.set_defaults(prefix_caching=None)
     p.add_argument("--long-prefill-token-threshold", type=int, default=0,
                    help="most prompt tokens of one request per step (0: no limit)")
     p.add_argument("--prefill-tokens-per-step", type=int, default=0,

@@ -20,7 +20,10 @@ class EngineOptions:
     long_prefill_token_threshold: int = 0    # per-request cap on a prompt portion (0: none)
     prefill_tokens_per_step: int = 0         # cap on all prompt tokens of a step (0: none)
     enable_chunked_prefill: bool = True
-    enable_prefix_caching: bool = False  # pages keep the tokens they hold; a later request with the same start reuses them
+    # pages keep the tokens they hold and a later request with the same start reuses them; None: on where every
+    # layer keeps all its keys (a window layer gives pages back while the request lives), as --no-prefix-caching
+    # of the reference implies (bins/dinfer/src/main.rs:30-131: the cache is on unless switched off)
+    enable_prefix_caching: bool | None = None
     hip_graph: bool = True              # replay decode steps from captured HIP graphs
     device: int = 0
     max_logits_rows: int | None = None  # None: max_num_seqs; replay and tests ask for more

@@ -127,7 +127,14 @@ class ModelRunner:
                                f"pages, the pool has {num_blocks}")
         self.num_blocks = int(num_blocks)
         self.group_specs = [GroupSpec(self.page_size, self.num_blocks, window=k[3]) for k in keys]
-        self.cache = CacheManager(self.group_specs, opt.max_num_seqs, prefix_caching=opt.enable_prefix_caching)
+        prefix = opt.enable_prefix_caching
+        if prefix is None:
+            # reusing pages is only the whole truth where the pages are: no layer drops keys, none keeps state of its own
+            prefix = (bool(keys) and all(g.window is None for g in self.group_specs)
+                      and not any(isinstance(n, StateSpec) for n in needs))
+        elif prefix and any(isinstance(n, StateSpec) for n in needs):
+            raise ValueError("the prefix cache cannot restore a layer's own state: switch it off for this model")
+        self.cache = CacheManager(self.group_specs, opt.max_num_seqs, prefix_caching=prefix)
         self.cache_views: list[CacheView] = []
         self.state_tensors: list[torch.Tensor] = []
         own: dict[int, CacheView] = {}

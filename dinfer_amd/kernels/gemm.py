@@ -33,8 +33,6 @@ def matmul_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int) -> to
     if m <= SMALL_M and w.shape[1] % 8 == 0:
         return ops.gemm_small_m(a, w, out, m)
     if out.dtype == torch.float32:
-        if m <= SMALL_M and w.shape[1] % 8 == 0:
-            return ops.gemm_small_m(a, w, out, m)  # float logits straight from the accumulators
         tmp = torch.mm(a[:m], w.t())
         ops.widen(tmp, out, m * w.shape[0]) if out.is_contiguous() else out[:m].copy_(tmp)
         return out
