@@ -197,7 +197,8 @@ def test_prefix_caching_changes_nothing_but_the_work(model_dirs, dtype):
     tails = prompts_for(name, [3, 11, 1, 25], 22)
     prompts = [stem + t for t in tails]
     sp = SamplingParams(max_tokens=6, temperature=0.0, ignore_eos=True)
-    plain_eng = engine(model_dirs[name], name, dtype=dtype)
+    plain_eng = engine(model_dirs[name], name, dtype=dtype, enable_prefix_caching=False)
+    assert not plain_eng.runner.cache.prefix_caching
     want = [plain_eng.generate([p], sp)[0] for p in prompts] + plain_eng.generate(prompts, sp)
     eng = engine(model_dirs[name], name, dtype=dtype, enable_prefix_caching=True)
     got, cached = [], []
@@ -219,3 +220,13 @@ def test_prefix_caching_changes_nothing_but_the_work(model_dirs, dtype):
         assert same >= 0.8 * sum(len(g) for g in got), (got, want)
     eng.runner.cache.check()
     assert eng.runner.cache.num_free(0) == 128
+
+
+def test_prefix_cache_is_on_where_every_layer_keeps_its_keys(model_dirs):
+    """Left to itself the engine reuses pages between requests, except for a model with window layers (their
+    pages go back while the request lives); asking for it there is an error, not a silent no."""
+    assert engine(model_dirs["A"], "A").runner.cache.prefix_caching
+    assert not engine(model_dirs["C"], "C").runner.cache.prefix_caching
+    assert not engine(model_dirs["A"], "A", enable_prefix_caching=False).runner.cache.prefix_caching
+    with pytest.raises(ValueError, match="keep every key"):
+        engine(model_dirs["C"], "C", enable_prefix_caching=True)
