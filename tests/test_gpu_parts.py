@@ -287,3 +287,197 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
     finally:
         unregister_architecture("ToyStateLM")
         MIXERS.unregister("toy_decay")
+
+
+# ---- a toy feed-forward with routing, another position encoding, and a layer that reads another's cache ------
+def register_routed_toy():
+    from dinfer_amd.config import ModelConfig, key, register_architecture
+    from dinfer_amd.parts import (FEED_FORWARDS, POSITION_ENCODINGS, FeedForward, LayerSpec, ModelSpec,
+                                  PositionEncoding, RunEntry, TensorSpec, part)
+
+    class RoutedFF(FeedForward):
+        """Every token goes to its top_k of E small gated experts; router logits and their softmax in float32,
+        the chosen weights renormalised to sum 1."""
+
+        def __init__(self, hidden, experts, top_k, intermediate):
+            self.hidden, self.E, self.k, self.inter = hidden, experts, top_k, intermediate
+
+        def tensors(self):
+            t = {"router.weight": TensorSpec((self.E, self.hidden))}
+            for e in range(self.E):
+                t[f"experts.{e}.gate.weight"] = TensorSpec((self.inter, self.hidden))
+                t[f"experts.{e}.up.weight"] = TensorSpec((self.inter, self.hidden))
+                t[f"experts.{e}.down.weight"] = TensorSpec((self.hidden, self.inter))
+            return t
+
+        def load(self, get):
+            self.router = get("router.weight").float()
+            self.w = [tuple(get(f"experts.{e}.{n}.weight", compute=True).float() for n in ("gate", "up", "down"))
+                      for e in range(self.E)]
+
+        def bind(self, ctx):
+            self.out = ctx.workspace.buffer("routed_out", self.hidden)
+
+        def forward(self, x, batch):
+            T = batch.num_tokens
+            xf = x[:T].float()
+            p = torch.softmax(xf @ self.router.T, dim=-1)
+            top, idx = p.topk(self.k, dim=-1)
+            top = top / top.sum(dim=-1, keepdim=True)
+            y = torch.zeros_like(xf)
+            for e, (g, u, d) in enumerate(self.w):
+                wgt = (top * (idx == e)).sum(dim=-1, keepdim=True)       # 0 for tokens that did not choose e
+                y += wgt * ((torch.nn.functional.silu(xf @ g.T) * (xf @ u.T)) @ d.T)
+            self.out[:T] = y.to(self.out.dtype)
+            return self.out
+
+    class SlowedRotary(PositionEncoding):
+        """Rotation of the first rotary_dim dims in interleaved pairs (2i, 2i + 1) by position / factor."""
+
+        def __init__(self, head_dim, theta, max_positions, rotary_dim, factor):
+            self.rotary_dim, self.style = rotary_dim, 1
+            self.theta, self.max_positions, self.factor = theta, max_positions, factor
+
+        def bind(self, ctx):
+            i = torch.arange(self.rotary_dim // 2, dtype=torch.float64)
+            ang = (torch.arange(self.max_positions, dtype=torch.float64) / self.factor)[:, None] \
+                * (self.theta ** (-2.0 * i / self.rotary_dim))[None, :]
+            self._table = torch.cat([ang.cos(), ang.sin()], dim=1).float().to(ctx.device)
+
+        def table(self):
+            return self._table
+
+    @dataclass(frozen=True)
+    class RoutedConfig(ModelConfig):
+        vocab_size: int = key(int)
+        hidden_size: int = key(int)
+        ARCHITECTURE = "ToyRoutedLM"
+
+    def build_spec(c):
+        norm = part("rmsnorm", eps=1e-5)
+        slowed = part("toy_slowed_rotary", theta=100.0, max_positions=128, rotary_dim=16, factor=4.0)
+        layers = [
+            LayerSpec(part("prenorm"), part("attention", heads=3, kv_heads=1, head_dim=32, position=slowed),
+                      part("toy_routed", experts=4, top_k=2, intermediate=24), norm, "layers.0."),
+            LayerSpec(part("prenorm"), part("attention", heads=2, kv_heads=2, head_dim=16, position=part("none"), window=12),
+                      part("gated_mlp", intermediate=40), norm, "layers.1."),
+        ]
+        # the third entry runs layer 0 again on the keys and values the first entry wrote (it writes none)
+        run = [RunEntry(0), RunEntry(1), RunEntry(0, cache=0)]
+        return ModelSpec("ToyRoutedLM", c.vocab_size, c.hidden_size, 128, layers, run, norm, "norm.", "embed.weight",
+                         "head.weight", tie_embeddings=False)
+
+    FEED_FORWARDS.register("toy_routed", RoutedFF)
+    POSITION_ENCODINGS.register("toy_slowed_rotary", SlowedRotary)
+    register_architecture("ToyRoutedLM", RoutedConfig, build_spec)
+    return RoutedConfig
+
+
+def routed_toy_plain(w, ids):
+    """The routed toy model for one whole sequence, straight torch in float64."""
+    W = {k: v.double() for k, v in w.items()}
+    T = len(ids)
+    h = W["embed.weight"][ids]
+
+    def slowed_rope(x):                      # x [T, heads, 32]: dims 0..15 in pairs (2i, 2i + 1), the rest untouched
+        i = torch.arange(8, dtype=torch.float64)
+        ang = (torch.arange(T, dtype=torch.float64) / 4.0)[:, None] * (100.0 ** (-2.0 * i / 16))[None, :]
+        c, s = ang.cos()[:, None, :], ang.sin()[:, None, :]
+        a, b = x[..., 0:16:2], x[..., 1:16:2]
+        y = x.clone()
+        y[..., 0:16:2], y[..., 1:16:2] = a * c - b * s, b * c + a * s
+        return y
+
+    def routed(p, x):
+        pr = torch.softmax(x @ W[p + "router.weight"].T, dim=-1)
+        y = torch.zeros_like(x)
+        for t in range(T):
+            top = sorted(range(4), key=lambda e: (-float(pr[t, e]), e))[:2]
+            tot = sum(pr[t, e] for e in top)
+            for e in top:
+                q = p + f"experts.{e}."
+                y[t] += pr[t, e] / tot * plain.swiglu_mlp(x[t:t + 1], W[q + "gate.weight"], W[q + "up.weight"], W[q + "down.weight"])[0]
+        return y
+
+    def layer0(h, kv):
+        p = "layers.0."
+        x = plain.rms_norm(h, W[p + "input_layernorm.weight"], 1e-5)
+        q = slowed_rope((x @ W[p + "self_attn.q_proj.weight"].T).view(T, 3, 32))
+        if kv is None:
+            kv = (slowed_rope((x @ W[p + "self_attn.k_proj.weight"].T).view(T, 1, 32)),
+                  (x @ W[p + "self_attn.v_proj.weight"].T).view(T, 1, 32))
+        o = plain.causal_attention(q, kv[0], kv[1], 32 ** -0.5)
+        h = h + o.reshape(T, 96) @ W[p + "self_attn.o_proj.weight"].T
+        return h + routed(p + "mlp.", plain.rms_norm(h, W[p + "post_attention_layernorm.weight"], 1e-5)), kv
+
+    def layer1(h):
+        p = "layers.1."
+        x = plain.rms_norm(h, W[p + "input_layernorm.weight"], 1e-5)
+        q, k, v = ((x @ W[p + f"self_attn.{n}_proj.weight"].T).view(T, 2, 16) for n in "qkv")
+        h = h + plain.causal_attention(q, k, v, 16 ** -0.5, window=12).reshape(T, 32) @ W[p + "self_attn.o_proj.weight"].T
+        x = plain.rms_norm(h, W[p + "post_attention_layernorm.weight"], 1e-5)
+        return h + plain.swiglu_mlp(x, W[p + "mlp.gate_proj.weight"], W[p + "mlp.up_proj.weight"], W[p + "mlp.down_proj.weight"])
+
+    h, kv = layer0(h, None)
+    h, _ = layer0(layer1(h), kv)
+    return plain.rms_norm(h, W["norm.weight"], 1e-5) @ W["head.weight"].T
+
+
+def test_toy_routing_position_encoding_and_shared_cache(tmp_path):
+    """A feed-forward that routes, a position encoding of another kind and a run order in which a layer runs
+    twice, the second time on the first time's cache: all defined here, no file of the framework changed.
+    Two page groups (every key; a window of 12), replayed whole, in portions and token by token."""
+    from safetensors.torch import load_file
+    from dinfer_amd.config import EngineOptions, unregister_architecture
+    from dinfer_amd.engine.batch import Entry
+    from dinfer_amd.engine.runner import ModelRunner
+    from dinfer_amd.parts import FEED_FORWARDS, POSITION_ENCODINGS
+    from dinfer_amd.weights import write_random_model
+    RoutedConfig = register_routed_toy()
+    try:
+        cfg = RoutedConfig.from_dict(dict(vocab_size=113, hidden_size=40, architectures=["ToyRoutedLM"]))
+        write_random_model(cfg, tmp_path, seed=9, dtype="float32")
+        w = load_file(str(tmp_path / "model.safetensors"))
+        assert "layers.0.mlp.experts.3.down.weight" in w and "layers.0.mlp.router.weight" in w
+        # make the router decisive, so that float32 and float64 choose the same experts
+        from safetensors.torch import save_file
+        w["layers.0.mlp.router.weight"] = w["layers.0.mlp.router.weight"] * 40.0
+        save_file(w, str(tmp_path / "model.safetensors"))
+        opt = EngineOptions(dtype="float32", max_model_len=128, max_num_seqs=3, max_num_batched_tokens=64,
+                            block_size=8, num_blocks=24, max_logits_rows=64)
+        r = ModelRunner.from_dir(tmp_path, opt)
+        assert len(r.group_specs) == 2 and len(r.cache_views) == 3 and not r.cache_views[2].owner
+        assert not r.cache.prefix_caching                      # a window group: pages do not outlive their use
+        rng = random.Random(3)
+        seqs = {k: [rng.randrange(113) for _ in range(n)] for k, n in (("a", 50), ("b", 37), ("c", 22))}
+        want = {k: routed_toy_plain(w, v) for k, v in seqs.items()}
+        plan = [[("a", 50)], [("b", 7), ("c", 2)], [("b", 1), ("c", 9)], [("b", 13), ("c", 1)], [("b", 16), ("c", 10)]]
+        fed = {k: 0 for k in seqs}
+
+        def run(st):
+            entries = []
+            for k, n in st:
+                assert r.reserve(k, fed[k], n)
+                entries.append(Entry(k, seqs[k][fed[k]:fed[k] + n], fed[k], list(range(n))))
+            logits = r.step(entries).double().cpu()
+            i = 0
+            for e in entries:
+                n = len(e.tokens)
+                torch.testing.assert_close(logits[i:i + n], want[e.req_id][e.start:e.start + n], rtol=2e-4, atol=2e-5)
+                i += n
+                fed[e.req_id] += n
+                r.advance(e.req_id, fed[e.req_id])
+                if fed[e.req_id] == len(seqs[e.req_id]):
+                    r.finish(e.req_id)
+
+        for st in plan:
+            run(st)
+        fed["a"] = 0                                          # again, token by token, in pages used before
+        for _ in range(len(seqs["a"])):
+            run([("a", 1)])
+        r.cache.check()
+        assert r.cache.num_free(0) == 24 and r.cache.num_free(1) == 24
+    finally:
+        unregister_architecture("ToyRoutedLM")
+        FEED_FORWARDS.unregister("toy_routed")
+        POSITION_ENCODINGS.unregister("toy_slowed_rotary")
