@@ -31,6 +31,7 @@ enum : int {
   ERR_BAD_SHAPE = 2,
   ERR_UNSUPPORTED = 3,
   ERR_LAUNCH = 4,
+  ERR_WORKSPACE = 5,
 };
 
 __device__ __forceinline__ float to_f32(float v) { return v; }

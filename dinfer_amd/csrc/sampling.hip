@@ -307,6 +307,486 @@ __global__ void __launch_bounds__(256) penalties_kernel(float* __restrict__ logi
   }
 }
 
+
+// ---- the same rule in a few passes over many workgroups -----------------------------------------
+// One workgroup per row needs about a hundred passes over the row for top-k and top-p (two
+// bisections) and walks the running sum 1024 entries at a time: 0.25 to 2.7 ms at a vocabulary of
+// 152k, however few the rows. Here a row is cut into segments of 2048 entries, one workgroup each:
+//   1. max:      the segment's largest z                          -> the row's maximum M
+//   2. hist:     per segment the mass sum exp(z - M) of the entries that survive min_p; for rows with
+//                top-k / top-p a histogram of (M - z) in bins of 1/64: count and mass (fixed point,
+//                integer atomics: the sums do not depend on the order of arrival)
+//   3. cut, extract: from the histogram, the bin that must hold the k-th largest entry, or the entry at
+//                which the mass reaches p; every entry of that bin and of the bins above goes to a list
+//   4. final:    one workgroup per row sorts the list (a few dozen to a few thousand entries), finds
+//                both thresholds exactly as the definitions say, and draws among what is left in
+//                vocabulary order; rows without top-k / top-p draw through the segment masses.
+// A row whose list would not fit (a flat distribution with a wide nucleus), or whose list turns out
+// too short for p, takes the one-workgroup path above inside step 4: slower, same rule.
+struct SampleRow {
+  float temperature;
+  int32_t top_k;
+  float top_p, min_p;
+  uint64_t seed, offset;
+};
+static_assert(sizeof(SampleRow) == 32, "rows are packed by the caller");
+
+constexpr int SEG = 2048;          // entries per segment
+constexpr int SEG_THREADS = 256;
+constexpr int NB = 2048;           // bins below the maximum
+constexpr float BINS_PER_UNIT = 64.f;
+constexpr int CAP = 4096;          // most entries of a row's list
+constexpr float MASS_ONE = 1099511627776.f;  // 2^40: fixed-point unit of the histogram's mass
+
+struct Plan {
+  bool active, do_k, do_p;
+  float inv_t, min_p, top_p;
+  int top_k;
+};
+__device__ __forceinline__ Plan plan_of(const SampleRow& r, int vocab) {
+  Plan p;
+  p.active = r.temperature > 1e-5f;
+  p.inv_t = p.active ? 1.f / r.temperature : 0.f;
+  p.min_p = r.min_p;
+  p.top_p = r.top_p;
+  p.top_k = r.top_k;
+  p.do_k = r.top_k > 0 && r.top_k < vocab;
+  p.do_p = r.top_p < 1.f && r.top_p > 0.f;
+  return p;
+}
+__device__ __forceinline__ bool survives(float z, float M, float min_p) {
+  return z > -INFINITY && !(min_p > 0.f && expf(z - M) < min_p);
+}
+__device__ __forceinline__ int bin_of(float z, float M) {
+  const float d = (M - z) * BINS_PER_UNIT;
+  return d < (float)(NB - 1) ? (int)d : NB - 1;
+}
+// ascending keys = descending z, ties by ascending index
+__device__ __forceinline__ uint32_t ordered_bits(float z) {
+  const uint32_t b = __float_as_uint(z);
+  return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+__device__ __forceinline__ float from_ordered_bits(uint32_t o) {
+  return __uint_as_float((o & 0x80000000u) ? (o & 0x7fffffffu) : ~o);
+}
+__device__ __forceinline__ uint64_t key_of(float z, int i) { return ((uint64_t)(~ordered_bits(z)) << 32) | (uint32_t)i; }
+__device__ __forceinline__ float key_value(uint64_t k) { return from_ordered_bits(~(uint32_t)(k >> 32)); }
+
+struct Scratch {
+  float* seg_max;                  // [rows][segs]
+  float* seg_mass;                 // [rows][segs]
+  unsigned long long* hist_mass;   // [rows][NB]
+  uint32_t* hist_count;            // [rows][NB]
+  unsigned long long* cand;        // [rows][CAP]
+  uint32_t* n_cand;                // [rows]
+  uint32_t* generic;               // [rows]: 1 = the list would not fit
+  int32_t* cut;                    // [rows]: the lowest bin on the list
+};
+inline size_t scratch_bytes(int64_t rows, int64_t segs) {
+  return (size_t)rows * ((size_t)segs * 8 + (size_t)NB * 12 + (size_t)CAP * 8 + 12);
+}
+inline Scratch carve(void* base, int64_t rows, int64_t segs) {
+  Scratch s;
+  char* p = (char*)base;
+  s.hist_mass = (unsigned long long*)p; p += (size_t)rows * NB * 8;
+  s.cand = (unsigned long long*)p;      p += (size_t)rows * CAP * 8;
+  s.hist_count = (uint32_t*)p;          p += (size_t)rows * NB * 4;
+  s.seg_max = (float*)p;                p += (size_t)rows * segs * 4;
+  s.seg_mass = (float*)p;               p += (size_t)rows * segs * 4;
+  s.n_cand = (uint32_t*)p;              p += (size_t)rows * 4;
+  s.generic = (uint32_t*)p;             p += (size_t)rows * 4;
+  s.cut = (int32_t*)p;
+  return s;
+}
+
+__device__ float row_max_of_segments(const float* seg_max, int segs, float* red) {
+  float m = -INFINITY;
+  for (int s = threadIdx.x; s < segs; s += blockDim.x) m = fmaxf(m, seg_max[s]);
+  return block_max(m, red);
+}
+
+__global__ void __launch_bounds__(SEG_THREADS) sample_max_kernel(const float* __restrict__ logits, int64_t ld,
+                                                                 const SampleRow* __restrict__ rows, Scratch sc,
+                                                                 int vocab, int segs) {
+  __shared__ float red[16];
+  const int r = blockIdx.y, s = blockIdx.x;
+  const Plan pl = plan_of(rows[r], vocab);
+  if (!pl.active) return;
+  if (pl.do_k || pl.do_p)
+    for (int b = s * SEG_THREADS + threadIdx.x; b < NB; b += segs * SEG_THREADS) {
+      sc.hist_count[(int64_t)r * NB + b] = 0u;
+      sc.hist_mass[(int64_t)r * NB + b] = 0ull;
+    }
+  if (s == 0 && threadIdx.x == 0) {
+    sc.n_cand[r] = 0u;
+    sc.generic[r] = 0u;
+  }
+  const float* row = logits + (int64_t)r * ld;
+  float m = -INFINITY;
+  for (int i = s * SEG + threadIdx.x; i < min(vocab, (s + 1) * SEG); i += SEG_THREADS) m = fmaxf(m, row[i] * pl.inv_t);
+  m = block_max(m, red);
+  if (threadIdx.x == 0) sc.seg_max[(int64_t)r * segs + s] = m;
+}
+
+__global__ void __launch_bounds__(SEG_THREADS) sample_hist_kernel(const float* __restrict__ logits, int64_t ld,
+                                                                  const SampleRow* __restrict__ rows, Scratch sc,
+                                                                  int vocab, int segs) {
+  __shared__ float red[16];
+  __shared__ uint32_t count[NB];
+  __shared__ unsigned long long mass[NB];
+  const int r = blockIdx.y, s = blockIdx.x;
+  const Plan pl = plan_of(rows[r], vocab);
+  if (!pl.active) return;
+  const bool filtered = pl.do_k || pl.do_p;
+  const float M = row_max_of_segments(sc.seg_max + (int64_t)r * segs, segs, red);
+  if (filtered) {
+    for (int b = threadIdx.x; b < NB; b += SEG_THREADS) {
+      count[b] = 0u;
+      mass[b] = 0ull;
+    }
+    __syncthreads();
+  }
+  const float* row = logits + (int64_t)r * ld;
+  float local = 0.f;
+  for (int i = s * SEG + threadIdx.x; i < min(vocab, (s + 1) * SEG); i += SEG_THREADS) {
+    const float z = row[i] * pl.inv_t;
+    if (!survives(z, M, pl.min_p)) continue;
+    const float e = expf(z - M);
+    local += e;
+    if (filtered) {
+      const int b = bin_of(z, M);
+      atomicAdd(&count[b], 1u);
+      atomicAdd(&mass[b], (unsigned long long)(e * MASS_ONE));
+    }
+  }
+  local = block_sum(local, red);
+  if (threadIdx.x == 0) sc.seg_mass[(int64_t)r * segs + s] = local;
+  if (filtered) {
+    __syncthreads();
+    for (int b = threadIdx.x; b < NB; b += SEG_THREADS)
+      if (count[b]) {
+        atomicAdd(&sc.hist_count[(int64_t)r * NB + b], count[b]);
+        atomicAdd(&sc.hist_mass[(int64_t)r * NB + b], mass[b]);
+      }
+  }
+}
+
+// Step 3a, one workgroup per row: the lowest bin whose entries must be on the list, and how many entries
+// that makes (more than CAP: the row takes the one-workgroup path).
+__global__ void __launch_bounds__(SEG_THREADS) sample_cut_kernel(const SampleRow* __restrict__ rows, Scratch sc, int vocab) {
+  constexpr int PER = NB / SEG_THREADS;  // consecutive bins per thread
+  __shared__ uint32_t tc[SEG_THREADS];
+  __shared__ unsigned long long tm[SEG_THREADS];
+  __shared__ int cut_bin;
+  const int r = blockIdx.x;
+  const Plan pl = plan_of(rows[r], vocab);
+  if (!pl.active || !(pl.do_k || pl.do_p)) return;
+  // running count and mass from the top bin down
+  uint32_t c[PER];
+  unsigned long long m[PER];
+  uint32_t csum = 0;
+  unsigned long long msum = 0;
+#pragma unroll
+  for (int e = 0; e < PER; ++e) {
+    c[e] = sc.hist_count[(int64_t)r * NB + threadIdx.x * PER + e];
+    m[e] = sc.hist_mass[(int64_t)r * NB + threadIdx.x * PER + e];
+    csum += c[e];
+    msum += m[e];
+  }
+  tc[threadIdx.x] = csum;
+  tm[threadIdx.x] = msum;
+  if (threadIdx.x == 0) cut_bin = NB - 1;
+  __syncthreads();
+  uint32_t cbefore = 0, ctotal = 0;
+  unsigned long long mbefore = 0, mtotal = 0;
+  for (int t = 0; t < SEG_THREADS; ++t) {
+    if (t == threadIdx.x) {
+      cbefore = ctotal;
+      mbefore = mtotal;
+    }
+    ctotal += tc[t];
+    mtotal += tm[t];
+  }
+  // the first bin at which the count reaches k, or else (top-p alone) the one after the bin at which
+  // the mass reaches p of all of it: one bin of margin for the rounding of the sums in step 4
+  const double want_mass = (double)pl.top_p * (double)mtotal;
+  int found = NB;
+  {
+    uint32_t cc = cbefore;
+    unsigned long long mm = mbefore;
+#pragma unroll
+    for (int e = 0; e < PER; ++e) {
+      cc += c[e];
+      mm += m[e];
+      const bool hit = pl.do_k ? cc >= (uint32_t)pl.top_k : (double)mm >= want_mass;
+      if (hit && found == NB) found = threadIdx.x * PER + e;
+    }
+  }
+  if (found < NB) atomicMin(&cut_bin, pl.do_k ? found : min(found + 1, NB - 1));
+  __syncthreads();
+  const int cut = cut_bin;
+  uint32_t cc = cbefore;
+#pragma unroll
+  for (int e = 0; e < PER; ++e) {
+    cc += c[e];
+    if (threadIdx.x * PER + e == cut) {
+      sc.cut[r] = cut;
+      sc.generic[r] = cc > (uint32_t)CAP ? 1u : 0u;
+    }
+  }
+}
+
+// Step 3b: every surviving entry of the bins down to the cut goes to the row's list.
+__global__ void __launch_bounds__(SEG_THREADS) sample_extract_kernel(const float* __restrict__ logits, int64_t ld,
+                                                                     const SampleRow* __restrict__ rows, Scratch sc,
+                                                                     int vocab, int segs) {
+  __shared__ float red[16];
+  const int r = blockIdx.y, s = blockIdx.x;
+  const Plan pl = plan_of(rows[r], vocab);
+  if (!pl.active || !(pl.do_k || pl.do_p) || sc.generic[r]) return;
+  const float M = row_max_of_segments(sc.seg_max + (int64_t)r * segs, segs, red);
+  const int cut = sc.cut[r];
+  const float* row = logits + (int64_t)r * ld;
+  for (int i = s * SEG + threadIdx.x; i < min(vocab, (s + 1) * SEG); i += SEG_THREADS) {
+    const float z = row[i] * pl.inv_t;
+    if (!survives(z, M, pl.min_p) || bin_of(z, M) > cut) continue;
+    const uint32_t slot = atomicAdd(&sc.n_cand[r], 1u);
+    if (slot < (uint32_t)CAP) sc.cand[(int64_t)r * CAP + slot] = key_of(z, i);
+  }
+}
+
+// Inclusive running sum over the workgroup's threads in thread order; every thread gets its own.
+__device__ float block_scan(float v, float* wave_tot) {
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  float incl = v;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const float up = __shfl_up(incl, o, 64);
+    if (lane >= o) incl += up;
+  }
+  __syncthreads();
+  if (lane == 63) wave_tot[w] = incl;
+  __syncthreads();
+  float before = 0.f;
+  for (int k = 0; k < w; ++k) before += wave_tot[k];
+  return before + incl;
+}
+
+// ascending bitonic sort of n_pow2 keys in LDS
+__device__ void sort_keys(unsigned long long* keys, int n_pow2) {
+  for (int k = 2; k <= n_pow2; k <<= 1)
+    for (int j = k >> 1; j > 0; j >>= 1) {
+      for (int t = threadIdx.x; t < n_pow2 / 2; t += BLOCK) {
+        const int i = (t / j) * 2 * j + (t % j), l = i + j;
+        const bool asc = (i & k) == 0;
+        const unsigned long long a = keys[i], b = keys[l];
+        if ((a > b) == asc) {
+          keys[i] = b;
+          keys[l] = a;
+        }
+      }
+      __syncthreads();
+    }
+}
+
+struct FinalShared {
+  Red red;
+  float fred[NWAVE];
+  float wave_tot[NWAVE];
+  DrawShared draw;
+  int pick;
+  int edge;
+  float carry, before;
+};
+
+// The one-workgroup form of the whole chain for this row (its z goes to `z`).
+__device__ int generic_row(const float* row, float* z, int vocab, const Plan& pl, uint64_t seed, uint64_t offset,
+                           FinalShared& sh) {
+  for (int i = threadIdx.x; i < vocab; i += BLOCK) z[i] = row[i] * pl.inv_t;
+  __syncthreads();
+  row_min_p(z, vocab, pl.min_p, sh.fred);
+  row_topk_topp(z, vocab, pl.top_k, pl.top_p, sh.fred);
+  return row_draw(z, vocab, seed, offset, sh.fred, sh.draw);
+}
+
+// Number of leading keys (sorted by descending value) whose value is >= t.
+__device__ int count_at_least(const unsigned long long* keys, int n, float t, FinalShared& sh) {
+  __syncthreads();
+  if (threadIdx.x == 0) sh.edge = 0;
+  __syncthreads();
+  for (int j = threadIdx.x; j < n; j += BLOCK)
+    if (key_value(keys[j]) >= t && (j + 1 == n || key_value(keys[j + 1]) < t)) sh.edge = j + 1;
+  __syncthreads();
+  return sh.edge;
+}
+
+__global__ void __launch_bounds__(BLOCK) sample_final_kernel(const float* __restrict__ logits, int64_t ld,
+                                                             float* __restrict__ work,
+                                                             const SampleRow* __restrict__ rows, Scratch sc,
+                                                             int32_t* __restrict__ out, int vocab, int segs,
+                                                             int force_generic) {
+  __shared__ FinalShared sh;
+  __shared__ unsigned long long keys[CAP];
+  __shared__ float cum[CAP];
+  const int r = blockIdx.x;
+  const SampleRow sr = rows[r];
+  const Plan pl = plan_of(sr, vocab);
+  const float* row = logits + (int64_t)r * ld;
+  if (!pl.active) {
+    const int c = row_argmax(row, vocab, sh.red);
+    if (threadIdx.x == 0) out[r] = c;
+    return;
+  }
+  const bool filtered = pl.do_k || pl.do_p;
+  if (force_generic || (filtered && sc.generic[r])) {
+    const int c = generic_row(row, work + (int64_t)r * vocab, vocab, pl, sr.seed, sr.offset, sh);
+    if (threadIdx.x == 0) out[r] = c;
+    return;
+  }
+  const float M = row_max_of_segments(sc.seg_max + (int64_t)r * segs, segs, sh.fred);
+  const float u = philox_uniform(sr.seed, sr.offset);
+  const float* seg_mass = sc.seg_mass + (int64_t)r * segs;
+
+  if (!filtered) {
+    // the segment in which the running sum of the survivors' mass reaches u * total, then the entry in it
+    float total = 0.f;
+    for (int base = 0; base < segs; base += BLOCK) {
+      const int s = base + threadIdx.x;
+      const float c = total + block_scan(s < segs ? seg_mass[s] : 0.f, sh.wave_tot);
+      __syncthreads();
+      if (threadIdx.x == BLOCK - 1) sh.carry = c;
+      __syncthreads();
+      total = sh.carry;
+    }
+    // the first segment with survivors at which the running sum reaches the target
+    const float target = u * total;
+    if (threadIdx.x == 0) sh.pick = 0x7fffffff;
+    __syncthreads();
+    float before_all = 0.f;
+    for (int base = 0; base < segs; base += BLOCK) {
+      const int s = base + threadIdx.x;
+      const float mine = s < segs ? seg_mass[s] : 0.f;
+      const float c = before_all + block_scan(mine, sh.wave_tot);
+      if (mine > 0.f && c >= target) atomicMin(&sh.pick, s);
+      __syncthreads();
+      if (threadIdx.x == BLOCK - 1) sh.carry = c;
+      if (s == sh.pick) sh.before = c - mine;
+      __syncthreads();
+      before_all = sh.carry;
+      if (sh.pick != 0x7fffffff) break;
+    }
+    const int seg = sh.pick;
+    if (seg == 0x7fffffff) {  // no survivor at all: every logit is -inf (or the total is no number)
+      if (threadIdx.x == 0) out[r] = 0;
+      return;
+    }
+    const float local_target = target - sh.before;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      sh.pick = 0x7fffffff;
+      sh.edge = -1;
+    }
+    __syncthreads();
+    float run = 0.f;
+    for (int base = seg * SEG; base < min(vocab, (seg + 1) * SEG); base += BLOCK) {
+      const int i = base + threadIdx.x;
+      float e = 0.f;
+      if (i < min(vocab, (seg + 1) * SEG)) {
+        const float z = row[i] * pl.inv_t;
+        if (survives(z, M, pl.min_p)) e = expf(z - M);
+      }
+      const float c = run + block_scan(e, sh.wave_tot);
+      if (e > 0.f) {
+        atomicMax(&sh.edge, i);  // the last survivor, should rounding leave the target above the segment's sum
+        if (c >= local_target) atomicMin(&sh.pick, i);
+      }
+      __syncthreads();
+      if (threadIdx.x == BLOCK - 1) sh.carry = c;
+      __syncthreads();
+      run = sh.carry;
+    }
+    if (threadIdx.x == 0) out[r] = sh.pick != 0x7fffffff ? sh.pick : (sh.edge >= 0 ? sh.edge : 0);
+    return;
+  }
+
+  // the list, sorted by descending value
+  const int n = (int)min(sc.n_cand[r], (uint32_t)CAP);
+  int n2 = 64;
+  while (n2 < n) n2 <<= 1;
+  for (int j = threadIdx.x; j < n2; j += BLOCK) keys[j] = j < n ? sc.cand[(int64_t)r * CAP + j] : ~0ull;
+  __syncthreads();
+  sort_keys(keys, n2);
+  int kept = n;
+  if (pl.do_k && n > pl.top_k) kept = count_at_least(keys, n, key_value(keys[pl.top_k - 1]), sh);
+  if (pl.do_p) {
+    // running mass in sorted order; the denominator is the mass of what top-k left
+    float run = 0.f;
+    for (int base = 0; base < kept; base += BLOCK) {
+      const int j = base + threadIdx.x;
+      const float c = run + block_scan(j < kept ? expf(key_value(keys[j]) - M) : 0.f, sh.wave_tot);
+      if (j < kept) cum[j] = c;
+      __syncthreads();
+      if (threadIdx.x == BLOCK - 1) sh.carry = c;
+      __syncthreads();
+      run = sh.carry;
+    }
+    float denom = run;
+    if (!pl.do_k) {  // nothing was cut before: all survivors count, the list holds only the largest of them
+      float t = 0.f;
+      for (int s = threadIdx.x; s < segs; s += BLOCK) t += seg_mass[s];
+      denom = block_sum(t, sh.fred);
+    }
+    if (threadIdx.x == 0) sh.pick = 0x7fffffff;
+    __syncthreads();
+    const float want = pl.top_p * denom;
+    for (int j = threadIdx.x; j < kept; j += BLOCK)
+      if (cum[j] >= want) atomicMin(&sh.pick, j);
+    __syncthreads();
+    const int cross = sh.pick;
+    __syncthreads();
+    if (cross == 0x7fffffff) {
+      if (!pl.do_k) {  // the list is too short for p after all
+        const int c = generic_row(row, work + (int64_t)r * vocab, vocab, pl, sr.seed, sr.offset, sh);
+        if (threadIdx.x == 0) out[r] = c;
+        return;
+      }
+    } else {
+      kept = count_at_least(keys, kept, key_value(keys[cross]), sh);
+    }
+  }
+  // what is left, in vocabulary order
+  __syncthreads();
+  int k2 = 64;
+  while (k2 < kept) k2 <<= 1;
+  for (int j = threadIdx.x; j < max(k2, n2); j += BLOCK) {
+    const unsigned long long k = keys[j];
+    const unsigned long long v = j < kept ? ((k & 0xffffffffull) << 32) | (uint32_t)__float_as_uint(key_value(k)) : ~0ull;
+    if (j < k2) keys[j] = v;
+  }
+  __syncthreads();
+  sort_keys(keys, k2);
+  float run = 0.f;
+  for (int base = 0; base < kept; base += BLOCK) {
+    const int j = base + threadIdx.x;
+    const float c = run + block_scan(j < kept ? expf(__uint_as_float((uint32_t)keys[j]) - M) : 0.f, sh.wave_tot);
+    if (j < kept) cum[j] = c;
+    __syncthreads();
+    if (threadIdx.x == BLOCK - 1) sh.carry = c;
+    __syncthreads();
+    run = sh.carry;
+  }
+  const float target = u * run;
+  if (threadIdx.x == 0) sh.pick = 0x7fffffff;
+  __syncthreads();
+  for (int j = threadIdx.x; j < kept; j += BLOCK)
+    if (cum[j] >= target && expf(__uint_as_float((uint32_t)keys[j]) - M) > 0.f) atomicMin(&sh.pick, j);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const int j = sh.pick != 0x7fffffff ? sh.pick : kept - 1;
+    out[r] = kept > 0 ? (int)(keys[j] >> 32) : 0;
+  }
+}
+
 }  // namespace
 
 extern "C" int dinfer_argmax(const float* logits, int64_t ld, int32_t* out, int64_t rows, int64_t vocab,
@@ -337,5 +817,42 @@ extern "C" int dinfer_penalties(float* logits, int64_t ld, const int32_t* ids, c
   if (vocab <= 0 || ld < vocab || rows > 0x7fffffff) return ERR_BAD_SHAPE;
   penalties_kernel<<<(unsigned)rows, 256, 0, stream>>>(logits, ld, ids, counts, offsets, repetition, frequency,
                                                        presence, (int)vocab);
+  return launch_status();
+}
+
+
+// Bytes of scratch that dinfer_sample_rows needs for this many rows and this vocabulary.
+extern "C" int dinfer_sample_scratch_bytes(int64_t rows, int64_t vocab, int64_t* bytes) {
+  if (rows <= 0 || vocab <= 0 || !bytes) return ERR_BAD_SHAPE;
+  *bytes = (int64_t)scratch_bytes(rows, (vocab + SEG - 1) / SEG);
+  return OK;
+}
+
+// The same rule as dinfer_sample, rows packed as {float temperature; int32 top_k; float top_p; float min_p;
+// uint64 seed; uint64 offset} (32 bytes each), in five launches that spread a row over many workgroups.
+// work [rows, vocab] floats and scratch (dinfer_sample_scratch_bytes, 8-byte aligned) are device memory;
+// what they hold before and after does not matter. any_filter = 0 promises that no row has top-k or top-p (two
+// launches fewer); force_generic != 0: every row takes the one-workgroup path.
+extern "C" int dinfer_sample_rows(const float* logits, int64_t ld, float* work, void* scratch, int64_t scratch_size,
+                                  const void* rows_packed, int32_t* out, int64_t rows, int64_t vocab,
+                                  int any_filter, int force_generic, hipStream_t stream) {
+  if (rows <= 0) return OK;
+  if (vocab <= 0 || vocab > (1 << 24) || ld < vocab || rows > 65535) return ERR_BAD_SHAPE;
+  if (!work || !scratch || !rows_packed || ((uintptr_t)scratch & 7) || ((uintptr_t)rows_packed & 7)) return ERR_BAD_SHAPE;
+  const int64_t segs = (vocab + SEG - 1) / SEG;
+  if ((size_t)scratch_size < scratch_bytes(rows, segs)) return ERR_WORKSPACE;
+  const Scratch sc = carve(scratch, rows, segs);
+  const SampleRow* sr = (const SampleRow*)rows_packed;
+  if (!force_generic) {
+    const dim3 grid((unsigned)segs, (unsigned)rows);
+    sample_max_kernel<<<grid, SEG_THREADS, 0, stream>>>(logits, ld, sr, sc, (int)vocab, (int)segs);
+    sample_hist_kernel<<<grid, SEG_THREADS, 0, stream>>>(logits, ld, sr, sc, (int)vocab, (int)segs);
+    if (any_filter) {
+      sample_cut_kernel<<<(unsigned)rows, SEG_THREADS, 0, stream>>>(sr, sc, (int)vocab);
+      sample_extract_kernel<<<grid, SEG_THREADS, 0, stream>>>(logits, ld, sr, sc, (int)vocab, (int)segs);
+    }
+  }
+  sample_final_kernel<<<(unsigned)rows, BLOCK, 0, stream>>>(logits, ld, work, sr, sc, out, (int)vocab, (int)segs,
+                                                            force_generic);
   return launch_status();
 }

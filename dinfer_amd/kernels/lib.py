@@ -47,6 +47,8 @@ SIGNATURES = {
     "dinfer_gemm_small_m_gated": ("gemm", [_P, _L, _P, _L, _P, _L, _L, _L, _L, _I, _P]),
     "dinfer_argmax": ("sampling", [_P, _L, _P, _L, _L, _P]),
     "dinfer_sample": ("sampling", [_P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _P]),
+    "dinfer_sample_rows": ("sampling", [_P, _L, _P, _P, _L, _P, _P, _L, _L, _I, _I, _P]),
+    "dinfer_sample_scratch_bytes": ("sampling", [_L, _L, _P]),
     "dinfer_penalties": ("sampling", [_P, _L, _P, _P, _P, _P, _P, _P, _L, _L, _P]),
 }
 

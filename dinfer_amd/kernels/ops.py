@@ -6,6 +6,9 @@ the calls can be captured into a HIP graph like any other stream work.
 """
 from __future__ import annotations
 
+import ctypes
+
+import numpy as np
 import torch
 
 from . import lib
@@ -324,6 +327,34 @@ def sample(logits: torch.Tensor, work: torch.Tensor | None, out: torch.Tensor, r
         assert t is None or (t.dtype == dt and t.numel() >= rows)
     lib.call("dinfer_sample", logits.data_ptr(), _rows(logits), _ptr(work), _ptr(temperature), _ptr(top_k),
              _ptr(top_p), _ptr(min_p), _ptr(seeds), _ptr(offsets), out.data_ptr(), rows, vocab, _stream())
+    return out
+
+
+# One row of dinfer_sample_rows: what to do with a row of logits.
+SAMPLE_ROW = np.dtype([("temperature", "<f4"), ("top_k", "<i4"), ("top_p", "<f4"), ("min_p", "<f4"),
+                       ("seed", "<u8"), ("offset", "<u8")])
+
+
+def sample_scratch_bytes(rows: int, vocab: int) -> int:
+    n = ctypes.c_int64(0)
+    lib.call("dinfer_sample_scratch_bytes", rows, vocab, ctypes.addressof(n))
+    return n.value
+
+
+def sample_rows(logits: torch.Tensor, work: torch.Tensor, scratch: torch.Tensor, packed: torch.Tensor,
+                out: torch.Tensor, rows: int, any_filter: bool = True, force_generic: bool = False) -> torch.Tensor:
+    """One token per row by the rule of `sample`, a row spread over many workgroups. packed: uint8 device
+    tensor holding `rows` records of SAMPLE_ROW; work [rows, vocab] float32 and scratch (uint8,
+    sample_scratch_bytes) are the kernels' own memory between their launches. any_filter=False promises
+    that no row has top-k or top-p."""
+    _need_gpu(logits, work, scratch, packed, out)
+    vocab = logits.shape[1]
+    assert logits.dtype == torch.float32 and out.dtype == torch.int32 and out.numel() >= rows
+    assert work.dtype == torch.float32 and work.is_contiguous() and work.numel() >= rows * vocab
+    assert packed.dtype == torch.uint8 and packed.is_contiguous() and packed.numel() >= rows * SAMPLE_ROW.itemsize
+    assert scratch.dtype == torch.uint8 and scratch.is_contiguous()
+    lib.call("dinfer_sample_rows", logits.data_ptr(), _rows(logits), work.data_ptr(), scratch.data_ptr(),
+             scratch.numel(), packed.data_ptr(), out.data_ptr(), rows, vocab, int(any_filter), int(force_generic), _stream())
     return out
 
 

@@ -18,16 +18,27 @@ from ..kernels import ops
 from .params import SamplingParams
 
 
-def _i64(u: int) -> int:
-    """The int64 with the bits of the uint64 u."""
-    return u - (1 << 64) if u >= 1 << 63 else u
-
-
 class Sampler:
     def __init__(self, device, max_rows: int, vocab: int):
         self.device, self.max_rows, self.vocab = device, max_rows, vocab
         self.out = torch.empty(max_rows, dtype=torch.int32, device=device)
-        self.work: torch.Tensor | None = None  # [max_rows, vocab] float32, made on first non-greedy use
+        # made on first non-greedy use: [max_rows, vocab] float32 for rows that take the one-workgroup path,
+        # the kernels' scratch, and the rows' options (filled in pinned host memory, copied once per step)
+        self.work: torch.Tensor | None = None
+        self.scratch: torch.Tensor | None = None
+        self.rows_host: torch.Tensor | None = None
+        self.rows_dev: torch.Tensor | None = None
+
+    def _buffers(self) -> None:
+        if self.work is not None:
+            return
+        nbytes = self.max_rows * ops.SAMPLE_ROW.itemsize
+        self.work = torch.empty((self.max_rows, self.vocab), dtype=torch.float32, device=self.device)
+        self.scratch = torch.empty(ops.sample_scratch_bytes(self.max_rows, self.vocab), dtype=torch.uint8,
+                                   device=self.device)
+        self.rows_host = torch.empty(nbytes, dtype=torch.uint8, pin_memory=True)
+        self.rows_dev = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
+        self._rows_np = self.rows_host.numpy().view(ops.SAMPLE_ROW)
 
     def sample(self, logits: torch.Tensor, rows: list) -> list[int]:
         """rows: per logits row (SamplingParams, num_output_tokens, prompt_ids, output_ids, seed)."""
@@ -40,19 +51,15 @@ class Sampler:
             return self.out[:R].tolist()
         if any(p.has_penalties for p, *_ in rows):
             self._penalties(logits, rows)
-        if self.work is None:
-            self.work = torch.empty((self.max_rows, self.vocab), dtype=torch.float32, device=self.device)
-        dev = self.device
-        f32 = lambda xs: torch.tensor(xs, dtype=torch.float32, device=dev)
-        temperature = f32([p.temperature for p, *_ in rows])
-        top_k = torch.tensor([p.top_k for p, *_ in rows], dtype=torch.int32, device=dev)
-        top_p = f32([p.top_p for p, *_ in rows])
-        min_p = f32([p.min_p for p, *_ in rows])
-        seeds = torch.tensor([_i64(seed) for *_, seed in rows], dtype=torch.int64, device=dev)
-        offsets = torch.tensor([n_out for _, n_out, *_ in rows], dtype=torch.int64, device=dev)
-        ops.sample(logits, self.work, self.out, R, temperature=temperature, top_k=top_k, top_p=top_p, min_p=min_p,
-                   seeds=seeds, offsets=offsets)
-        return self.out[:R].tolist()
+        self._buffers()
+        rec = self._rows_np
+        for i, (p, n_out, _prompt, _output, seed) in enumerate(rows):
+            rec[i] = (p.temperature, p.top_k, p.top_p, p.min_p, seed & 0xFFFFFFFFFFFFFFFF, n_out)
+        n = R * ops.SAMPLE_ROW.itemsize
+        self.rows_dev[:n].copy_(self.rows_host[:n], non_blocking=True)
+        any_filter = any(p.top_k > 0 or p.top_p < 1.0 for p, *_ in rows)
+        ops.sample_rows(logits, self.work, self.scratch, self.rows_dev, self.out, R, any_filter=any_filter)
+        return self.out[:R].tolist()   # waits for the stream, and with it for the copy out of rows_host
 
     def _penalties(self, logits, rows) -> None:
         ids, cnts, offs = [], [], [0]

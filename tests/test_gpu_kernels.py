@@ -316,18 +316,33 @@ def test_argmax_ties_to_lowest_index():
     assert out.tolist() == want
 
 
-def draw(logits, temperature, seeds, offsets, **kw):
+PATHS = ["one_workgroup", "spread", "spread_forced_generic"]
+
+
+def draw(logits, temperature, seeds, offsets, path="spread", **kw):
+    """path: the kernel with one workgroup a row; the launches that spread a row over many workgroups (what the
+    sampler uses); the latter with every row sent down its built-in one-workgroup branch."""
+    import numpy as np
     R, V = logits.shape
     out = torch.empty(R, device=DEV, dtype=torch.int32)
     work = torch.empty(R, V, device=DEV)
     f = lambda xs, dt: torch.tensor(xs, device=DEV, dtype=dt)
-    ops().sample(logits, work, out, R, temperature=f(temperature, torch.float32), seeds=f(seeds, torch.int64),
-                 offsets=f(offsets, torch.int64),
-                 **{k: f(v, torch.int32 if k == "top_k" else torch.float32) for k, v in kw.items()})
+    if path == "one_workgroup":
+        ops().sample(logits, work, out, R, temperature=f(temperature, torch.float32), seeds=f(seeds, torch.int64),
+                     offsets=f(offsets, torch.int64),
+                     **{k: f(v, torch.int32 if k == "top_k" else torch.float32) for k, v in kw.items()})
+        return out.tolist()
+    rec = np.zeros(R, dtype=ops().SAMPLE_ROW)
+    rec["temperature"], rec["seed"], rec["offset"] = temperature, [x & (2**64 - 1) for x in seeds], offsets
+    rec["top_k"], rec["top_p"], rec["min_p"] = kw.get("top_k", -1), kw.get("top_p", 1.0), kw.get("min_p", 0.0)
+    packed = torch.from_numpy(rec.view(np.uint8)).to(DEV)
+    scratch = torch.empty(ops().sample_scratch_bytes(R, V), dtype=torch.uint8, device=DEV)
+    ops().sample_rows(logits, work, scratch, packed, out, R, force_generic=path == "spread_forced_generic")
     return out.tolist()
 
 
-def test_sample_follows_the_inverse_cdf_rule():
+@pytest.mark.parametrize("path", PATHS)
+def test_sample_follows_the_inverse_cdf_rule(path):
     """Each draw must be the token whose interval of the running sum holds u * total, with u from the
     plain Philox. Draws whose target lies within rounding of an interval's edge are not judged."""
     V = 331
@@ -335,7 +350,7 @@ def test_sample_follows_the_inverse_cdf_rule():
     temps = [0.7] * 64
     seeds = [12345 + i for i in range(64)]
     offsets = [i * 3 for i in range(64)]
-    got = draw(logits, temps, seeds, offsets)
+    got = draw(logits, temps, seeds, offsets, path)
     judged = 0
     for r in range(64):
         tok, slack = plain.sample_row(logits[r].cpu(), temps[r], seeds[r], offsets[r])
@@ -345,31 +360,34 @@ def test_sample_follows_the_inverse_cdf_rule():
     assert judged > 55
 
 
-def test_sample_does_not_depend_on_batch_position():
+@pytest.mark.parametrize("path", PATHS)
+def test_sample_does_not_depend_on_batch_position(path):
     V = 1000
     row = torch.randn(1, V, device=DEV)
     other = torch.randn(5, V, device=DEV)
-    alone = draw(row, [0.9], [777], [4])[0]
+    alone = draw(row, [0.9], [777], [4], path)[0]
     batch = torch.cat([other[:3], row, other[3:]])
-    mixed = draw(batch, [1.0, 0.0, 0.5, 0.9, 1.3, 0.0], [1, 2, 3, 777, 5, 6], [0, 0, 0, 4, 0, 0])
+    mixed = draw(batch, [1.0, 0.0, 0.5, 0.9, 1.3, 0.0], [1, 2, 3, 777, 5, 6], [0, 0, 0, 4, 0, 0], path)
     assert mixed[3] == alone
     assert mixed[1] == int(batch[1].argmax()) and mixed[5] == int(batch[5].argmax())  # greedy rows untouched
 
 
-def test_sample_frequencies_match_softmax():
+@pytest.mark.parametrize("path", PATHS[:2])
+def test_sample_frequencies_match_softmax(path):
     """100k draws of one 64-token row at temperature 0.8: L1 distance to softmax below 0.03
     (the reference's statistical test, crates/kernels/tests/ref_tests.rs:225-252)."""
     V, N = 64, 100_000
     row = torch.randn(V, device=DEV) * 2
     counts = torch.zeros(V)
     for chunk in range(N // 1000):
-        toks = draw(row.expand(1000, V).contiguous(), [0.8] * 1000, [42] * 1000, list(range(chunk * 1000, chunk * 1000 + 1000)))
+        toks = draw(row.expand(1000, V).contiguous(), [0.8] * 1000, [42] * 1000, list(range(chunk * 1000, chunk * 1000 + 1000)), path)
         counts += torch.bincount(torch.tensor(toks), minlength=V).float()
     want = torch.softmax(row.cpu() / 0.8, -1)
     assert (counts / N - want).abs().sum() < 0.03
 
 
-def test_sample_candidate_sets():
+@pytest.mark.parametrize("path", PATHS)
+def test_sample_candidate_sets(path):
     """min_p, top-k and top-p: every draw falls in the set the plain rule keeps."""
     V = 512
     logits = torch.randn(6, V, device=DEV) * 3
@@ -380,7 +398,7 @@ def test_sample_candidate_sets():
         keep = plain.candidate_mask(logits[r].cpu().double() / 0.9, **c)
         seen = set()
         for off in range(0, 200, 50):
-            toks = draw(logits[r].expand(50, V).contiguous(), [0.9] * 50, [9] * 50, list(range(off, off + 50)),
+            toks = draw(logits[r].expand(50, V).contiguous(), [0.9] * 50, [9] * 50, list(range(off, off + 50)), path,
                         top_k=[c["top_k"]] * 50, top_p=[c["top_p"]] * 50, min_p=[c["min_p"]] * 50)
             seen |= set(toks)
         outside = [t for t in seen if not keep[t]]
@@ -388,6 +406,70 @@ def test_sample_candidate_sets():
         assert len(outside) <= max(2, int(0.001 * keep.sum())), f"case {c}: drew {outside} outside the kept set"
         if c["top_k"] == 1:
             assert seen == {int(logits[r].argmax())}
+
+
+def test_sample_spread_over_workgroups_at_a_large_vocabulary():
+    """At a vocabulary of many segments (and no multiple of one): peaked rows, whose top-k / top-p sets are short
+    lists, and a flat row whose nucleus is too wide for a list and takes the built-in one-workgroup branch.
+    Every option alone and together; each judged draw is the plain rule's token."""
+    V = 151936 + 3
+    g = torch.Generator().manual_seed(5)
+    base = torch.randn(V, generator=g) * 2.0
+    peaked = base.clone()
+    peaked[torch.randperm(V, generator=g)[:40]] += torch.rand(40, generator=g) * 6 + 6     # a few dozen likely tokens
+    flat = base * 0.2
+    cases = [dict(), dict(min_p=0.02), dict(top_k=1), dict(top_k=20), dict(top_k=3000), dict(top_p=0.9), dict(top_p=0.3),
+             dict(top_k=50, top_p=0.95), dict(top_k=50, top_p=0.9, min_p=0.01), dict(top_k=V - 1), dict(top_p=0.999)]
+    rows, opts = [], []
+    for i, c in enumerate(cases):
+        for src in (peaked, flat):
+            rows.append(src)
+            opts.append({**dict(top_k=-1, top_p=1.0, min_p=0.0), **c})
+    logits = torch.stack(rows).to(DEV)
+    R = len(rows)
+    seeds, offsets, temps = [100 + i for i in range(R)], [i % 7 for i in range(R)], [0.8] * R
+    kw = {k: [o[k] for o in opts] for k in ("top_k", "top_p", "min_p")}
+    got = draw(logits, temps, seeds, offsets, "spread", **kw)
+    slow = draw(logits, temps, seeds, offsets, "one_workgroup", **kw)
+    judged = 0
+    for r in range(R):
+        tok, slack = plain.sample_row(logits[r].cpu(), temps[r], seeds[r], offsets[r], **opts[r])
+        keep = plain.candidate_mask(logits[r].cpu().double() / temps[r], **opts[r])
+        assert keep[got[r]], f"row {r} {opts[r]}: drew {got[r]} outside the kept set"
+        if slack > 1e-5:
+            judged += 1
+            assert got[r] == tok, f"row {r} {opts[r]}: drew {got[r]}, the rule says {tok} (one workgroup: {slow[r]})"
+        else:
+            # an interval narrower than 32-bit sums resolve (a flat row: 1 / V each): the target must lie
+            # within rounding of the drawn token's interval
+            z = logits[r].cpu().double() / temps[r]
+            pr = torch.where(keep, torch.exp(z - z[keep].max()), torch.zeros_like(z))
+            cum = pr.cumsum(-1)
+            target = plain.uniform(seeds[r], offsets[r]) * float(cum[-1])
+            lo, hi = float(cum[got[r]] - pr[got[r]]), float(cum[got[r]])
+            assert max(lo - target, target - hi, 0.0) < 2e-5 * float(cum[-1]), f"row {r} {opts[r]}: drew {got[r]}, rule {tok}"
+    assert judged >= R // 2
+
+
+def test_sample_paths_agree_on_random_options():
+    """The spread launches against the one-workgroup kernel over random rows and options: the same token, but for
+    the few draws whose target lies within rounding of an interval's edge (the sums are taken in another order)."""
+    V, R = 40000 + 17, 96
+    rng = random.Random(8)
+    logits = (torch.randn(R, V) * torch.tensor([rng.choice([0.3, 1.0, 3.0, 6.0]) for _ in range(R)])[:, None]).to(DEV)
+    logits[5, 100:200] = float("-inf")
+    logits[6, :] = 1.5                                                     # all equal: every filter keeps all ties
+    temps = [rng.choice([0.0, 0.3, 0.8, 1.0, 1.7]) for _ in range(R)]
+    kw = dict(top_k=[rng.choice([-1, -1, 1, 7, 64, 1000, 30000]) for _ in range(R)],
+              top_p=[rng.choice([1.0, 1.0, 0.95, 0.7, 0.1]) for _ in range(R)],
+              min_p=[rng.choice([0.0, 0.0, 0.05, 0.3]) for _ in range(R)])
+    seeds, offsets = [rng.getrandbits(64) - (1 << 63) for _ in range(R)], [rng.randrange(500) for _ in range(R)]
+    a = draw(logits, temps, seeds, offsets, "one_workgroup", **kw)
+    b = draw(logits, temps, seeds, offsets, "spread", **kw)
+    c = draw(logits, temps, seeds, offsets, "spread_forced_generic", **kw)
+    assert a == c
+    differ = [r for r in range(R) if a[r] != b[r]]
+    assert len(differ) <= 2, [(r, a[r], b[r], temps[r], {k: v[r] for k, v in kw.items()}) for r in differ]
 
 
 def test_penalties_match_plain_rule():
