@@ -787,6 +787,47 @@ __global__ void __launch_bounds__(BLOCK) sample_final_kernel(const float* __rest
   }
 }
 
+
+// ---- penalties from a history kept on the device ---------------------------------------------------
+// history [slots, vocab] int32: bit 30 = the token occurs in the request's prompt, the low bits count
+// its occurrences among the request's outputs. The host sends only what is new (a prompt once, then
+// the token of each step), so a step costs no pass over the request's tokens on the host.
+constexpr int32_t IN_PROMPT = 1 << 30;
+
+struct PenaltyRow {
+  int32_t slot;  // < 0: the row has no penalties
+  float repetition, frequency, presence;
+};
+static_assert(sizeof(PenaltyRow) == 16, "rows are packed by the caller");
+
+// entries [n][3] = (slot, token, kind): kind 0 marks a prompt token, kind 1 counts one more output
+__global__ void __launch_bounds__(256) history_add_kernel(int32_t* __restrict__ history, int64_t vocab,
+                                                          const int32_t* __restrict__ entries, int n, int slots) {
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= n) return;
+  const int slot = entries[3 * e], tok = entries[3 * e + 1], kind = entries[3 * e + 2];
+  if (slot < 0 || slot >= slots || tok < 0 || tok >= vocab) return;
+  int32_t* cell = history + (int64_t)slot * vocab + tok;
+  if (kind == 0) atomicOr(cell, IN_PROMPT);
+  else atomicAdd(cell, 1);
+}
+
+__global__ void __launch_bounds__(256) penalties_dense_kernel(float* __restrict__ logits, int64_t ld,
+                                                              const int32_t* __restrict__ history,
+                                                              const PenaltyRow* __restrict__ rows, int vocab) {
+  const PenaltyRow pr = rows[blockIdx.y];
+  if (pr.slot < 0) return;
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= vocab) return;
+  const int32_t st = history[(int64_t)pr.slot * vocab + i];
+  if (st == 0) return;
+  float v = logits[(int64_t)blockIdx.y * ld + i];
+  if (pr.repetition != 1.f) v = v > 0.f ? v / pr.repetition : v * pr.repetition;
+  const int c = st & (IN_PROMPT - 1);
+  if (c > 0) v -= pr.frequency * (float)c + pr.presence;
+  logits[(int64_t)blockIdx.y * ld + i] = v;
+}
+
 }  // namespace
 
 extern "C" int dinfer_argmax(const float* logits, int64_t ld, int32_t* out, int64_t rows, int64_t vocab,
@@ -854,5 +895,28 @@ extern "C" int dinfer_sample_rows(const float* logits, int64_t ld, float* work, 
   }
   sample_final_kernel<<<(unsigned)rows, BLOCK, 0, stream>>>(logits, ld, work, sr, sc, out, (int)vocab, (int)segs,
                                                             force_generic);
+  return launch_status();
+}
+
+
+// history [slots, vocab] int32 (zero = a request without tokens yet); entries [n][3] int32 = (slot, token,
+// kind 0: the token occurs in the prompt, kind 1: one more occurrence among the outputs).
+extern "C" int dinfer_history_add(int32_t* history, int64_t slots, int64_t vocab, const int32_t* entries, int64_t n,
+                                  hipStream_t stream) {
+  if (n <= 0) return OK;
+  if (!history || !entries || slots <= 0 || vocab <= 0 || n > 0x7fffffff || slots > 0x7fffffff) return ERR_BAD_SHAPE;
+  history_add_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(history, vocab, entries, (int)n, (int)slots);
+  return launch_status();
+}
+
+// In place on logits [rows, ld]: rows packed as {int32 slot; float repetition, frequency, presence} (slot < 0:
+// untouched) take their penalties from history[slot] (the rule of dinfer_penalties).
+extern "C" int dinfer_penalties_dense(float* logits, int64_t ld, const int32_t* history, int64_t slots,
+                                      const void* rows_packed, int64_t rows, int64_t vocab, hipStream_t stream) {
+  if (rows <= 0) return OK;
+  if (!history || !rows_packed || vocab <= 0 || ld < vocab || rows > 65535 || vocab > 0x7fffffff || slots <= 0)
+    return ERR_BAD_SHAPE;
+  const dim3 grid((unsigned)((vocab + 255) / 256), (unsigned)rows);
+  penalties_dense_kernel<<<grid, 256, 0, stream>>>(logits, ld, history, (const PenaltyRow*)rows_packed, (int)vocab);
   return launch_status();
 }

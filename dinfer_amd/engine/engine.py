@@ -65,6 +65,7 @@ class Engine:
 
     def abort(self, request_id) -> None:
         self.scheduler.abort(request_id)
+        self.sampler.forget(request_id)
 
     def has_unfinished(self) -> bool:
         return self.scheduler.has_unfinished()
@@ -76,10 +77,13 @@ class Engine:
         if not len(so):
             return outs
         logits = self.runner.step_planned(self.scheduler, so)
-        rows = [(r.sampling, len(r.output_ids), r.prompt_ids, r.output_ids, r.seed) for r in so.sampling_requests()]
+        rows = [(r.sampling, len(r.output_ids), r.prompt_ids, r.output_ids, r.seed, r.id) for r in so.sampling_requests()]
         tokens = self.sampler.sample(logits, rows)
         for r, tok, reason in self.scheduler.update(so, tokens):
             outs.append(StepOutput(r.id, tok, reason is not None, reason))
+        for o in outs:
+            if o.finished:
+                self.sampler.forget(o.request_id)
         return outs
 
     def generate(self, prompts: list, sampling: SamplingParams | list | None = None) -> list[list[int]]:

@@ -49,6 +49,8 @@ SIGNATURES = {
     "dinfer_sample": ("sampling", [_P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _P]),
     "dinfer_sample_rows": ("sampling", [_P, _L, _P, _P, _L, _P, _P, _L, _L, _I, _I, _P]),
     "dinfer_sample_scratch_bytes": ("sampling", [_L, _L, _P]),
+    "dinfer_history_add": ("sampling", [_P, _L, _L, _P, _L, _P]),
+    "dinfer_penalties_dense": ("sampling", [_P, _L, _P, _L, _P, _L, _L, _P]),
     "dinfer_penalties": ("sampling", [_P, _L, _P, _P, _P, _P, _P, _P, _L, _L, _P]),
 }
 

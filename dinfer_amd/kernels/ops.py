@@ -358,6 +358,31 @@ def sample_rows(logits: torch.Tensor, work: torch.Tensor, scratch: torch.Tensor,
     return out
 
 
+# One row of penalties_dense: which history slot a row of logits takes its penalties from (< 0: none).
+PENALTY_ROW = np.dtype([("slot", "<i4"), ("repetition", "<f4"), ("frequency", "<f4"), ("presence", "<f4")])
+
+
+def history_add(history: torch.Tensor, entries: torch.Tensor) -> None:
+    """history [slots, vocab] int32; entries [n, 3] int32 = (slot, token, kind): kind 0 marks a token of the
+    prompt, kind 1 counts one more occurrence among the outputs."""
+    _need_gpu(history, entries)
+    assert history.dtype == torch.int32 and history.is_contiguous() and history.dim() == 2
+    assert entries.dtype == torch.int32 and entries.is_contiguous() and entries.dim() == 2 and entries.shape[1] == 3
+    lib.call("dinfer_history_add", history.data_ptr(), history.shape[0], history.shape[1], entries.data_ptr(),
+             entries.shape[0], _stream())
+
+
+def penalties_dense(logits: torch.Tensor, rows: int, history: torch.Tensor, packed: torch.Tensor) -> None:
+    """In place on logits: row r takes repetition / frequency / presence penalties from history[slot_r]
+    (packed: uint8 device tensor of `rows` PENALTY_ROW records; slot < 0 leaves the row alone)."""
+    _need_gpu(logits, history, packed)
+    assert logits.dtype == torch.float32 and history.dtype == torch.int32 and history.is_contiguous()
+    assert history.shape[1] == logits.shape[1]
+    assert packed.dtype == torch.uint8 and packed.is_contiguous() and packed.numel() >= rows * PENALTY_ROW.itemsize
+    lib.call("dinfer_penalties_dense", logits.data_ptr(), _rows(logits), history.data_ptr(), history.shape[0],
+             packed.data_ptr(), rows, logits.shape[1], _stream())
+
+
 def penalties(logits: torch.Tensor, rows: int, ids: torch.Tensor, counts: torch.Tensor, offsets: torch.Tensor,
               repetition: torch.Tensor, frequency: torch.Tensor, presence: torch.Tensor) -> None:
     """In place on logits: per row, entries offsets[b]..offsets[b+1] list the distinct tokens of the

@@ -9,8 +9,6 @@ depend on the row's place in the batch or on the other rows
 """
 from __future__ import annotations
 
-from collections import Counter
-
 import numpy as np
 import torch
 
@@ -28,6 +26,9 @@ class Sampler:
         self.scratch: torch.Tensor | None = None
         self.rows_host: torch.Tensor | None = None
         self.rows_dev: torch.Tensor | None = None
+        self.history: torch.Tensor | None = None   # [max_rows, vocab] int32, made on first use of a penalty
+        self._slots: dict = {}                      # request -> [history slot, outputs already counted]
+        self._free: list = []
 
     def _buffers(self) -> None:
         if self.work is not None:
@@ -41,7 +42,9 @@ class Sampler:
         self._rows_np = self.rows_host.numpy().view(ops.SAMPLE_ROW)
 
     def sample(self, logits: torch.Tensor, rows: list) -> list[int]:
-        """rows: per logits row (SamplingParams, num_output_tokens, prompt_ids, output_ids, seed)."""
+        """rows: per logits row (SamplingParams, num_output_tokens, prompt_ids, output_ids, seed[, request]).
+        request: any hashable name of the request, under which its history is kept from step to step
+        (forget() when it is over); without it a row with penalties sends its whole history every time."""
         R = len(rows)
         assert logits.shape[0] == R and R <= self.max_rows
         if R == 0:
@@ -53,27 +56,56 @@ class Sampler:
             self._penalties(logits, rows)
         self._buffers()
         rec = self._rows_np
-        for i, (p, n_out, _prompt, _output, seed) in enumerate(rows):
+        for i, (p, n_out, _prompt, _output, seed, *_key) in enumerate(rows):
             rec[i] = (p.temperature, p.top_k, p.top_p, p.min_p, seed & 0xFFFFFFFFFFFFFFFF, n_out)
         n = R * ops.SAMPLE_ROW.itemsize
+        # pinned memory the device may still be reading from the step before: this step's tokens were read
+        # back (tolist) before it returned, so that copy is done
         self.rows_dev[:n].copy_(self.rows_host[:n], non_blocking=True)
         any_filter = any(p.top_k > 0 or p.top_p < 1.0 for p, *_ in rows)
         ops.sample_rows(logits, self.work, self.scratch, self.rows_dev, self.out, R, any_filter=any_filter)
         return self.out[:R].tolist()   # waits for the stream, and with it for the copy out of rows_host
 
+    def forget(self, key) -> None:
+        """The request is over: its history slot is free again."""
+        st = self._slots.pop(key, None)
+        if st is not None:
+            self._free.append(st[0])
+
     def _penalties(self, logits, rows) -> None:
-        ids, cnts, offs = [], [], [0]
-        for p, _n, prompt, output, _s in rows:
-            if p.has_penalties:
-                c_out = Counter(output)
-                seen = set(prompt) | set(output)
-                for t in seen:
-                    ids.append(t)
-                    cnts.append(c_out.get(t, 0))
-            offs.append(len(ids))
-        dev = self.device
-        i32 = lambda xs: torch.tensor(np.asarray(xs, dtype=np.int32), dtype=torch.int32, device=dev)
-        f32 = lambda xs: torch.tensor(xs, dtype=torch.float32, device=dev)
-        ops.penalties(logits, len(rows), i32(ids if ids else [0]), i32(cnts if cnts else [0]), i32(offs),
-                      f32([p.repetition_penalty for p, *_ in rows]), f32([p.frequency_penalty for p, *_ in rows]),
-                      f32([p.presence_penalty for p, *_ in rows]))
+        """Repetition, frequency and presence penalties, in place. The tokens a request has seen live on the
+        device ([max_rows, vocab] int32, a slot per request with penalties); only what is new goes there:
+        the distinct prompt tokens once, then the outputs since the last step."""
+        if self.history is None:
+            self.history = torch.empty((self.max_rows, self.vocab), dtype=torch.int32, device=self.device)
+            self._free = list(range(self.max_rows - 1, -1, -1))
+        R = len(rows)
+        pen = np.zeros(R, dtype=ops.PENALTY_ROW)
+        pen["slot"] = -1
+        entries: list = []
+        passing: list = []
+        try:
+            for i, (p, _n, prompt, output, _seed, *key) in enumerate(rows):
+                if not p.has_penalties:
+                    continue
+                key = key[0] if key else None
+                st = self._slots.get(key) if key is not None else None
+                if st is None:
+                    if not self._free:
+                        raise RuntimeError(f"more than {self.max_rows} live requests with penalties")
+                    st = [self._free.pop(), 0]
+                    self.history[st[0]].zero_()
+                    entries += [(st[0], t, 0) for t in set(prompt)]
+                    if key is None:
+                        passing.append(st[0])          # a row without a name: the slot lasts for this call
+                    else:
+                        self._slots[key] = st
+                slot, counted = st
+                entries += [(slot, t, 1) for t in output[counted:]]
+                st[1] = len(output)
+                pen[i] = (slot, p.repetition_penalty, p.frequency_penalty, p.presence_penalty)
+            if entries:
+                ops.history_add(self.history, torch.from_numpy(np.asarray(entries, dtype=np.int32)).to(self.device))
+            ops.penalties_dense(logits, R, self.history, torch.from_numpy(pen.view(np.uint8)).to(self.device))
+        finally:
+            self._free += passing

@@ -131,10 +131,16 @@ def test_engine_loop_with_a_stand_in_runner():
         def sample(self, logits, rows):
             return logits.argmax(-1).tolist()
 
+        def forget(self, key):
+            self.forgotten.append(key)
+
+        forgotten: list = []
+
     eng = Engine(runner=FakeRunner())
     eng.sampler = FakeSampler()
     outs = eng.generate([list(range(10)), list(range(30)), [1, 2]], SamplingParams(max_tokens=3, temperature=0.0))
     assert outs == [[10, 11, 12], [30, 31, 32], [2, 3, 4]]
+    assert sorted(eng.sampler.forgotten) == [0, 1, 2]                          # told of every request that ended
     assert eng.runner.steps[0] == [(0, 10, 0), (1, 6, 0)]                   # budget 16: the second prompt is cut
     assert eng.runner.steps[1] == [(0, 1, 10), (1, 16, 6)]                  # the decode row is exempt: the prompt gets all 16
     assert eng.runner.cache.num_free() == 32 and not eng.has_unfinished()

@@ -492,6 +492,53 @@ def test_penalties_match_plain_rule():
         torch.testing.assert_close(got[r].cpu().double(), want, rtol=1e-6, atol=1e-6)
 
 
+def test_penalties_from_a_history_on_the_device():
+    """The sampler keeps what each request has seen on the device and sends only what is new: requests come, take
+    steps in changing company, end, and their slots are used again; every step's penalised logits are the plain
+    rule's over the request's whole prompt and outputs."""
+    from dinfer_amd.sampling.params import SamplingParams
+    from dinfer_amd.sampling.sampler import Sampler
+    V = 331
+    rng = random.Random(2)
+    s = Sampler(DEV, 3, V)
+    sp = {"a": SamplingParams(temperature=0.0, repetition_penalty=1.4),
+          "b": SamplingParams(temperature=0.0, frequency_penalty=0.6, presence_penalty=0.3),
+          "c": SamplingParams(temperature=0.0),                                    # no penalties: no slot
+          "d": SamplingParams(temperature=0.0, repetition_penalty=0.8, frequency_penalty=0.2, presence_penalty=1.0),
+          "e": SamplingParams(temperature=0.0, presence_penalty=2.0)}
+    prompts = {k: [rng.randrange(V) for _ in range(rng.randint(1, 60))] for k in sp}
+    outputs = {k: [] for k in sp}
+    plan = [["a"], ["a", "b"], ["b", "c", "a"], ["d", "a", "b"], ["d"], ["e", "d", "c"], ["e", "d", "b"]]
+    ends = {3: ["a"], 4: ["b"], 6: ["e"]}      # after step 3 a is over (then d and e need its slot) ...
+    for step, live in enumerate(plan):
+        if step == 6:                         # ... and b comes back under its old name as a new request
+            prompts["b"], outputs["b"] = [rng.randrange(V) for _ in range(9)], []
+        logits = torch.randn(len(live), V, device=DEV) * 3
+        want = []
+        for i, k in enumerate(live):
+            p = sp[k]
+            z = plain.apply_penalties(logits[i].cpu().double(), prompts[k], outputs[k], p.repetition_penalty,
+                                      p.frequency_penalty, p.presence_penalty)
+            want.append(int(z.argmax()))
+        toks = s.sample(logits, [(sp[k], len(outputs[k]), prompts[k], outputs[k], 0, k) for k in live])
+        assert toks == want, (step, live, toks, want)
+        for k, t in zip(live, toks):
+            outputs[k].append(t)
+            outputs[k].append(prompts[k][0])   # and one the sampler did not choose (a forced token): counted all the same
+        for k in ends.get(step, []):
+            s.forget(k)
+    assert len(s._slots) == 2 and len(s._free) == 1
+    # rows without a name send their whole history and keep no slot
+    logits = torch.randn(2, V, device=DEV) * 3
+    rows = [(sp["d"], 3, [5, 6, 7], [7, 7, 8], 0), (sp["e"], 0, [1], [], 0)]
+    want = [int(plain.apply_penalties(logits[i].cpu().double(), r[2], r[3], r[0].repetition_penalty, r[0].frequency_penalty,
+                                      r[0].presence_penalty).argmax()) for i, r in enumerate(rows)]
+    with pytest.raises(RuntimeError, match="live requests with penalties"):
+        s.sample(logits, rows)               # one slot is free, two are needed
+    s.forget("d")
+    assert s.sample(logits, rows) == want and len(s._free) == 2
+
+
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 33, 64])
 def test_gemm_small_m(M, out_dtype):
