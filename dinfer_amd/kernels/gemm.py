@@ -3,13 +3,15 @@
 float32 operands: the vector-ALU kernel with a fixed summation order (the true
 32-bit path). bfloat16 operands: the hand-written MFMA kernel that streams the
 weight once for few rows (decode, LM head), and the vendor library for many
-rows, where the reference uses a library too (crates/kernels/src/gemm.rs:605-647).
+rows, where the reference uses a library too (crates/kernels/src/gemm.rs:605-647):
+hipBLASLt called directly with the algorithm measured per shape (blaslt.py), or
+through torch.mm where that library cannot be loaded.
 """
 from __future__ import annotations
 
 import torch
 
-from . import ops
+from . import blaslt, ops
 
 
 # Up to this many rows the weight-streaming kernel beats the library on MI355X (measured at the four layer
@@ -22,8 +24,15 @@ def fuses_gated_act(a: torch.Tensor, w: torch.Tensor, m: int, act: str) -> bool:
     return a.dtype == torch.bfloat16 and act == "silu" and 0 < m <= SMALL_M and w.shape[1] % 8 == 0
 
 
-def matmul_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int) -> torch.Tensor:
-    """out[:m] = a[:m] @ w.T; out has a's dtype, or float32 (logits)."""
+# Rows of a library product are rounded up to a multiple of this where the caller allows it: a prompt portion
+# beside a changing number of decoding requests then meets a handful of shapes, each with its algorithm chosen
+# once, instead of a new shape every step.
+ROW_BUCKET = 32
+
+
+def matmul_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, may_pad: bool = False) -> torch.Tensor:
+    """out[:m] = a[:m] @ w.T; out has a's dtype, or float32 (logits). may_pad: a and out are scratch
+    buffers whose rows beyond m hold nothing of value; the product may read and write a few of them."""
     if m <= 0:
         return out
     if a.dtype == torch.float32:
@@ -36,5 +45,8 @@ def matmul_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int) -> to
         tmp = torch.mm(a[:m], w.t())
         ops.widen(tmp, out, m * w.shape[0]) if out.is_contiguous() else out[:m].copy_(tmp)
         return out
+    if blaslt.available() and a.stride(1) == 1 and w.stride(1) == 1 and out.stride(1) == 1:
+        rows = min(a.shape[0], out.shape[0], -(-m // ROW_BUCKET) * ROW_BUCKET) if may_pad else m
+        return blaslt.matmul(a, w, out, rows)
     torch.mm(a[:m], w.t(), out=out[:m])
     return out

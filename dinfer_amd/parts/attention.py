@@ -72,7 +72,7 @@ class Attention(Mixer):
     def forward(self, x, batch, cache: CacheView):
         T = batch.num_tokens
         g = cache.group
-        self.qkv.forward(x, self.qkv_buf, T)
+        self.qkv.forward(x, self.qkv_buf, T, scratch=True)
         qn = self.q_norm
         ops.qkv_post(
             self.qkv_buf, T, heads=self.heads, kv_heads=self.kv_heads, head_dim=self.head_dim,
@@ -87,4 +87,4 @@ class Attention(Mixer):
             self.qkv_buf, self.attn_buf, cache.k, cache.v, batch, g, self.attn_ws, scale=self.scale,
             window=self.window or 0, heads=self.heads, kv_heads=self.kv_heads, head_dim=self.head_dim,
             page_size=self.page_size)
-        return self.o.forward(self.attn_buf, self.out_buf, T)
+        return self.o.forward(self.attn_buf, self.out_buf, T, scratch=True)

@@ -16,5 +16,6 @@ class Linear:
             raise ValueError(f"linear weight is {tuple(w.shape)}, expected {(self.out_features, self.in_features)}")
         self.weight = w.contiguous()
 
-    def forward(self, x: torch.Tensor, out: torch.Tensor, m: int) -> torch.Tensor:
-        return gemm.matmul_nt(x, self.weight, out, m)
+    def forward(self, x: torch.Tensor, out: torch.Tensor, m: int, scratch: bool = False) -> torch.Tensor:
+        """scratch: x and out are activation buffers with spare rows beyond m that nothing reads."""
+        return gemm.matmul_nt(x, self.weight, out, m, may_pad=scratch)

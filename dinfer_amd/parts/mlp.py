@@ -42,6 +42,6 @@ class GatedMLP(FeedForward):
             # decode-sized steps: both projections and the activation in one weight-streaming kernel
             ops.gemm_small_m_gated(x, self.gate_up.weight, self.act_buf, T)
         else:
-            self.gate_up.forward(x, self.gu_buf, T)
+            self.gate_up.forward(x, self.gu_buf, T, scratch=True)
             ops.gated_act(self.gu_buf, self.act_buf, T, self.act)
-        return self.down.forward(self.act_buf, self.out_buf, T)
+        return self.down.forward(self.act_buf, self.out_buf, T, scratch=True)

@@ -554,6 +554,25 @@ def test_gemm_small_m(M, out_dtype):
             torch.testing.assert_close(out.double(), want, **t, msg=lambda m_: f"M={M} N={N} K={K} rt={rt} waves={waves}: {m_}")
 
 
+def test_library_gemm_with_measured_algorithm():
+    """Products of many rows: the vendor library called directly, its candidates timed once per shape. Rows may be
+    rounded up to a bucket inside scratch buffers: the rows asked for are right, rows past the bucket untouched."""
+    from dinfer_amd.kernels import blaslt, gemm
+    assert blaslt.available()
+    for M, N, K in ((130, 200, 264), (520, 1000, 1096), (33, 96, 512), (257, 4096, 512)):
+        a = torch.randn(M + 70, K, device=DEV).to(torch.bfloat16)
+        w = (torch.randn(N, K, device=DEV) * 0.05).to(torch.bfloat16)
+        want = a[:M].double() @ w.double().T
+        for pad in (False, True):
+            out = torch.full((M + 70, N), 7.0, device=DEV, dtype=torch.bfloat16)
+            for _ in range(2):                                   # the first call measures, the second replays the choice
+                gemm.matmul_nt(a, w, out, M, may_pad=pad)
+            torch.testing.assert_close(out[:M].double(), want, rtol=2e-2, atol=2e-2, msg=lambda m_: f"{M}x{N}x{K} pad={pad}: {m_}")
+            last = -(-M // gemm.ROW_BUCKET) * gemm.ROW_BUCKET if pad else M
+            assert bool((out[last:] == 7.0).all()), f"{M}x{N}x{K} pad={pad}: rows past {last} were written"
+    assert any(p.tuned for p in blaslt._plans.values())
+
+
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 32])
 def test_gemm_small_m_gated(M):
     """Both projections of a gated feed-forward and silu(gate) * up in one kernel, against float64."""
