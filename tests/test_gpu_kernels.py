@@ -472,6 +472,35 @@ def test_sample_paths_agree_on_random_options():
     assert len(differ) <= 2, [(r, a[r], b[r], temps[r], {k: v[r] for k, v in kw.items()}) for r in differ]
 
 
+def test_sample_paths_agree_at_the_edges_of_the_options():
+    """Very cold and very hot rows, a nucleus of almost nothing, min_p of 1, top-k of 1 on a tie, rows of equal
+    logits and rows that are -inf but for one entry: the spread launches give the one-workgroup kernel's token."""
+    V = 20011
+    g = torch.Generator().manual_seed(21)
+    base = torch.randn(V, generator=g) * 4
+    tie = base.clone()
+    tie[[17, 4000, 19999]] = base.max() + 1.0                  # three equal maxima
+    lonely = torch.full((V,), float("-inf"))
+    lonely[12345] = 0.3
+    flat = torch.zeros(V)
+    cases = [(base, 1e-4, {}), (base, 50.0, {}), (base, 1.0, dict(top_p=1e-6)), (base, 1.0, dict(min_p=1.0)),
+             (tie, 1.0, dict(top_k=1)), (tie, 0.7, dict(top_p=1e-6)), (tie, 0.7, dict(min_p=1.0)), (flat, 1.0, dict(top_k=5)),
+             (flat, 1.0, dict(top_p=0.5)), (lonely, 1.0, {}), (lonely, 0.5, dict(top_k=3, top_p=0.9, min_p=0.1)),
+             (base, 1e-4, dict(top_k=40, top_p=0.9)), (base, 50.0, dict(top_k=V - 1, top_p=0.99999))]
+    logits = torch.stack([c[0] for c in cases]).to(DEV)
+    temps = [c[1] for c in cases]
+    kw = {k: [c[2].get(k, d) for c in cases] for k, d in (("top_k", -1), ("top_p", 1.0), ("min_p", 0.0))}
+    for seed in (1, 2, 3):
+        seeds, offsets = [seed * 100 + i for i in range(len(cases))], [seed] * len(cases)
+        a = draw(logits, temps, seeds, offsets, "one_workgroup", **kw)
+        b = draw(logits, temps, seeds, offsets, "spread", **kw)
+        differ = [(i, a[i], b[i]) for i in range(len(cases)) if a[i] != b[i]]
+        # the hot rows and the flat ones have intervals of 1 / V: a target within rounding of an edge may fall either way
+        assert all(i in (1, 7, 8, 12) for i, _, _ in differ) and len(differ) <= 2, differ
+        assert b[4] in (17, 4000, 19999) and b[5] in (17, 4000, 19999) and b[6] in (17, 4000, 19999)
+        assert b[9] == 12345 and b[10] == 12345 and b[0] == int(base.argmax()) and b[3] == int(base.argmax())
+
+
 def test_penalties_match_plain_rule():
     V = 512
     logits = torch.randn(4, V, device=DEV) * 3
