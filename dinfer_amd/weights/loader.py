@@ -70,14 +70,14 @@ class WeightLoader:
         """compute=True: a matrix-product operand, always brought to the engine's dtype."""
         if name not in self.src:
             raise WeightError([name], [], [])
-        t = self.src.read(name)
+        t = self.src.read_to(name, self.device)   # conversions happen where the tensor lives
         if t.dtype in (torch.int64, torch.int32, torch.int16, torch.int8, torch.uint8, torch.bool):
-            return t.to(torch.int32).to(self.device)
+            return t.to(torch.int32)
         if t.dtype == torch.float64:
             t = t.to(torch.float32)
         if compute or t.dtype != torch.float32:
             t = t.to(self.dtype)
-        return t.to(self.device).contiguous()
+        return t.contiguous()
 
     def close(self) -> None:
         self.src.close()

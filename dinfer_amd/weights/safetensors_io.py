@@ -49,7 +49,9 @@ class _File:
         size = path.stat().st_size
         if size < 8:
             raise WeightFileError(f"{path}: too short for a safetensors header")
-        self.mm = mmap.mmap(self.fh.fileno(), 0, access=mmap.ACCESS_READ)
+        # a private mapping: pages come from the page cache without a copy, and the buffer counts as writable, which
+        # lets torch wrap it without complaint (nothing ever writes to it)
+        self.mm = mmap.mmap(self.fh.fileno(), 0, access=mmap.ACCESS_COPY)
         (n,) = struct.unpack("<Q", self.mm[:8])
         if 8 + n > size:
             raise WeightFileError(f"{path}: header length {n} exceeds the file size {size}")
@@ -98,18 +100,36 @@ class SafetensorsDir:
     def info(self, name: str) -> TensorInfo:
         return self.index[name]
 
+    def raw(self, name: str) -> torch.Tensor:
+        """The tensor's bytes as a uint8 view of the mapped file: no copy. The view must be dropped before
+        close(); callers copy it (to the device, or clone) right away."""
+        ti = self.index[name]
+        if ti.end == ti.start:
+            return torch.empty(0, dtype=torch.uint8)
+        return torch.frombuffer(ti.file.mm, dtype=torch.uint8, count=ti.end - ti.start, offset=ti.start)
+
     def read(self, name: str) -> torch.Tensor:
-        """The tensor as stored (a CPU copy, in its stored dtype)."""
+        """The tensor as stored (a CPU copy of its own, in its stored dtype)."""
         ti = self.index[name]
         dt, _ = DTYPES[ti.dtype_name]
-        buf = ti.file.mm[ti.start:ti.end]  # bytes copy; keeps the mapping free of exported pointers
-        if len(buf) == 0:
-            return torch.empty(ti.shape, dtype=dt)
-        return torch.frombuffer(bytearray(buf), dtype=dt).reshape(ti.shape)
+        return self.raw(name).clone().view(dt).reshape(ti.shape)
+
+    def read_to(self, name: str, device) -> torch.Tensor:
+        """The tensor as stored, on `device`: one copy, from the mapped file straight to where it will live
+        (the bytes are reinterpreted there, where the allocation is aligned whatever the file's offsets)."""
+        ti = self.index[name]
+        dt, _ = DTYPES[ti.dtype_name]
+        raw = self.raw(name)
+        dev = torch.device(device)
+        moved = raw.clone() if dev.type == "cpu" else raw.to(dev)
+        return moved.view(dt).reshape(ti.shape)
 
     def close(self) -> None:
         for f in self.files:
-            f.mm.close()
+            try:
+                f.mm.close()
+            except BufferError:   # a view of the mapping is still alive somewhere: the mapping goes when it does
+                pass
             f.fh.close()
 
 
