@@ -500,7 +500,7 @@ __global__ void __launch_bounds__(SEG_THREADS) sample_cut_kernel(const SampleRow
   uint32_t cbefore = 0, ctotal = 0;
   unsigned long long mbefore = 0, mtotal = 0;
   for (int t = 0; t < SEG_THREADS; ++t) {
-    if (t == threadIdx.x) {
+    if (t == (int)threadIdx.x) {
       cbefore = ctotal;
       mbefore = mtotal;
     }
@@ -529,7 +529,7 @@ __global__ void __launch_bounds__(SEG_THREADS) sample_cut_kernel(const SampleRow
 #pragma unroll
   for (int e = 0; e < PER; ++e) {
     cc += c[e];
-    if (threadIdx.x * PER + e == cut) {
+    if ((int)threadIdx.x * PER + e == cut) {
       sc.cut[r] = cut;
       sc.generic[r] = cc > (uint32_t)CAP ? 1u : 0u;
     }

@@ -8,7 +8,6 @@ a loader of its own (models/qwen3/src/executor.rs:977-1031, model.rs:684-832).
 """
 from __future__ import annotations
 
-import json
 from pathlib import Path
 
 import torch

@@ -5,7 +5,6 @@ A failing call returns minus the kind of its error; the text comes from dh_last_
 """
 from __future__ import annotations
 
-import ctypes
 from ctypes import POINTER, Structure, c_char_p, c_int32, c_int64, c_void_p
 
 from .kernels.lib import load_library

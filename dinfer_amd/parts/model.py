@@ -6,10 +6,10 @@ from __future__ import annotations
 import torch
 
 from ..kernels import gemm, ops
-from .base import BuildContext, CacheView
+from .base import BuildContext
 from .linear import Linear
 from .registry import BLOCKS, NORMS
-from .spec import KVSpec, ModelSpec, RunEntry, StateSpec, TensorSpec
+from .spec import ModelSpec, RunEntry, TensorSpec
 
 
 def _build_blocks(spec: ModelSpec):

@@ -13,7 +13,6 @@ import numpy as np
 import torch
 
 from ..kernels import ops
-from .params import SamplingParams
 
 
 class Sampler:

@@ -19,7 +19,7 @@ from __future__ import annotations
 import torch
 
 from ..parts.spec import TensorSpec
-from .safetensors_io import SafetensorsDir, WeightFileError
+from .safetensors_io import SafetensorsDir
 
 
 class WeightError(ValueError):

@@ -10,7 +10,6 @@ judge the engine's 32-bit path; it does not imitate bfloat16 roundings.
 from __future__ import annotations
 
 import json
-import math
 from pathlib import Path
 
 import torch

@@ -3,7 +3,6 @@ BASELINE names for the tiny configurations, sampling rules through the whole eng
 import random
 
 import pytest
-import torch
 
 import plain_qwen3 as plain
 from tiny_configs import CONFIGS, PAGE

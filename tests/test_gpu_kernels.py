@@ -1,7 +1,6 @@
 """Each HIP kernel alone against a plain float64 torch reference of the same operation, at
 sizes other than the engine tests use (widths and vocabularies that are no power of two,
 head sizes 32..256, group sizes 1..8, page sizes 8..64, shuffled page order)."""
-import math
 import random
 
 import pytest

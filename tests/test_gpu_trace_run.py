@@ -1,6 +1,5 @@
 """bin/trace_run as a user runs it: a subprocess fed JSON lines, logits read from files."""
 import json
-import os
 import random
 import subprocess
 import sys
@@ -11,7 +10,6 @@ import pytest
 import torch
 
 import plain_qwen3 as plain
-from tiny_configs import CONFIGS
 
 pytestmark = pytest.mark.gpu
 ROOT = Path(__file__).resolve().parent.parent

@@ -1,7 +1,6 @@
 """The plain implementation is the judge of the engine, so it is pinned here by what fixes it
 besides the reference's text: special cases that reduce to a library routine, invariants, and
 known answers. Each check is chosen so that a plausible mistake fails it (noted per test). No GPU."""
-import math
 
 import pytest
 import torch
