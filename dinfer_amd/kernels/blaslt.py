@@ -170,7 +170,14 @@ def matmul(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int) -> torch
     key = (dev, m, n, k, a.stride(0), w.stride(0), out.stride(0), out.dtype)
     plan = _plans.get(key)
     if plan is None:
-        plan = _plans[key] = _Plan(handle, m, n, k, a.stride(0), w.stride(0), out.stride(0), out.dtype)
+        try:
+            plan = _Plan(handle, m, n, k, a.stride(0), w.stride(0), out.stride(0), out.dtype)
+        except RuntimeError:
+            plan = False   # a shape the direct interface does not take: torch's own call of the library serves it
+        _plans[key] = plan
+    if plan is False:
+        torch.mm(a[:m], w.t(), out=out[:m])
+        return out
     workspace = _workspaces[dev]
     if (not plan.tuned and m >= TUNE_FROM_ROWS and len(plan.candidates) > 1
             and os.environ.get("DINFER_GEMM_TUNE", "1") != "0" and not torch.cuda.is_current_stream_capturing()):
