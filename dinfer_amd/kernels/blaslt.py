@@ -176,7 +176,10 @@ def matmul(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int) -> torch
             plan = False   # a shape the direct interface does not take: torch's own call of the library serves it
         _plans[key] = plan
     if plan is False:
-        torch.mm(a[:m], w.t(), out=out[:m])
+        if out.dtype == a.dtype:
+            torch.mm(a[:m], w.t(), out=out[:m])
+        else:
+            out[:m].copy_(torch.mm(a[:m], w.t()))
         return out
     workspace = _workspaces[dev]
     if (not plan.tuned and m >= TUNE_FROM_ROWS and len(plan.candidates) > 1

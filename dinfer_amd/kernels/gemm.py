@@ -41,12 +41,13 @@ def matmul_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, may_p
         raise RuntimeError("matrix products run on the GPU only")
     if m <= SMALL_M and w.shape[1] % 8 == 0:
         return ops.gemm_small_m(a, w, out, m)
+    if blaslt.available() and a.stride(1) == 1 and w.stride(1) == 1 and out.stride(1) == 1:
+        # float32 out (logits at many positions): straight from the accumulators, as the few-row kernel gives them
+        rows = min(a.shape[0], out.shape[0], -(-m // ROW_BUCKET) * ROW_BUCKET) if may_pad else m
+        return blaslt.matmul(a, w, out, rows)
     if out.dtype == torch.float32:
         tmp = torch.mm(a[:m], w.t())
         ops.widen(tmp, out, m * w.shape[0]) if out.is_contiguous() else out[:m].copy_(tmp)
         return out
-    if blaslt.available() and a.stride(1) == 1 and w.stride(1) == 1 and out.stride(1) == 1:
-        rows = min(a.shape[0], out.shape[0], -(-m // ROW_BUCKET) * ROW_BUCKET) if may_pad else m
-        return blaslt.matmul(a, w, out, rows)
     torch.mm(a[:m], w.t(), out=out[:m])
     return out

@@ -599,6 +599,12 @@ def test_library_gemm_with_measured_algorithm():
             last = -(-M // gemm.ROW_BUCKET) * gemm.ROW_BUCKET if pad else M
             assert bool((out[last:] == 7.0).all()), f"{M}x{N}x{K} pad={pad}: rows past {last} were written"
     assert any(p and p.tuned for p in blaslt._plans.values())
+    # float32 out (logits at many positions): not rounded to bfloat16 on the way
+    a = torch.randn(100, 264, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(1000, 264, device=DEV) * 0.05).to(torch.bfloat16)
+    out = torch.empty(100, 1000, device=DEV)
+    gemm.matmul_nt(a, w, out, 100)
+    torch.testing.assert_close(out.double(), a.double() @ w.double().T, rtol=1e-4, atol=1e-4)
 
 
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 32])
