@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """In-process throughput of the engine on one MI355X: Qwen3-8B-shaped random weights.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L] [--shape 8b|14b|32b]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L] [--shape 8b|14b|32b|0.6b]
                     [--prompt P] [--context C]
 
 Prints ONE JSON line. `value` is decoded tokens per second at the default batch (8), each
@@ -37,6 +37,9 @@ SHAPES = {
     "8b": {},
     "14b": dict(hidden_size=5120, intermediate_size=17408, num_hidden_layers=40, num_attention_heads=40),
     "32b": dict(hidden_size=5120, intermediate_size=25600, num_hidden_layers=64, num_attention_heads=64),
+    # the size the reference publishes its own numbers for (models/qwen3/src/config.rs:84-101)
+    "0.6b": dict(hidden_size=1024, intermediate_size=3072, num_hidden_layers=28, num_attention_heads=16,
+                 tie_word_embeddings=True),
 }
 DEFAULT_PROMPT, DEFAULT_CONTEXT = 2048, 4096
 HBM_PEAK = 8.0e12
