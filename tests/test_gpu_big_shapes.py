@@ -68,3 +68,43 @@ def test_layer_sizes_of_the_large_models(big_models, name, dtype):
                 assert err < 0.08, f"{name} {e.req_id}@{e.start}: {err:.3f} row-sigmas"
             i += len(e.tokens)
             fed[e.req_id] += len(e.tokens)
+
+
+def test_decode_graph_with_library_products_replays_equal_eager(big_models):
+    """40 requests decoding: more rows than the weight-streaming kernel takes, so the vendor library's products
+    (with the algorithm measured per shape) are inside the captured graph. Every replay is checked against the
+    same step run eagerly, with eager steps (another request's prompt portions) between the replays."""
+    from dinfer_amd.config import EngineOptions
+    from dinfer_amd.engine.batch import Entry
+    from dinfer_amd.engine.runner import ModelRunner
+    rng = random.Random(4)
+    B = 40
+    prompts = [[rng.randrange(2048) for _ in range(12 + i % 5)] for i in range(B)]
+    tail = [[rng.randrange(2048) for _ in range(6)] for _ in range(B)]
+    extra = [rng.randrange(2048) for _ in range(90)]
+    outs = {}
+    for graph in (False, True):
+        opt = EngineOptions(dtype="bfloat16", max_model_len=512, max_num_seqs=48, max_num_batched_tokens=1024,
+                            block_size=16, num_blocks=256, max_logits_rows=64, decode_exempt_from_budget=False,
+                            hip_graph=graph)
+        r = ModelRunner.from_dir(big_models["8B"], opt)
+        got = []
+        entries = []
+        for i, p in enumerate(prompts):
+            assert r.reserve(i, 0, len(p))
+            entries.append(Entry(i, p, 0, [len(p) - 1]))
+        got.append(r.step(entries).float().cpu())
+        fed_extra = 0
+        for s in range(6):
+            entries = []
+            for i, p in enumerate(prompts):
+                assert r.reserve(i, len(p) + s, 1)
+                entries.append(Entry(i, [tail[i][s]], len(p) + s, [0]))
+            got.append(r.step(entries).float().cpu())                        # the graph's bucket of 48 rows
+            assert r.reserve("x", fed_extra, 15)
+            got.append(r.step([Entry("x", extra[fed_extra:fed_extra + 15], fed_extra, [14])]).float().cpu())  # eager
+            fed_extra += 15
+        assert bool(r._graphs) == graph
+        outs[graph] = got
+    for step, (a, b) in enumerate(zip(outs[False], outs[True])):
+        torch.testing.assert_close(b, a, rtol=2e-2, atol=2e-2, msg=lambda m: f"step {step}: {m}")
