@@ -1,6 +1,10 @@
-// Token selection on float logits, one workgroup of 1024 threads per row:
-// argmax, and the chain penalties -> temperature -> min_p -> top-k / top-p ->
-// inverse-CDF draw with a counter-based random number, fused in one kernel.
+// Token selection on float logits: argmax, and the chain penalties -> temperature ->
+// min_p -> top-k / top-p -> inverse-CDF draw with a counter-based random number.
+// The chain exists in two forms that follow the same rule: one kernel with one
+// workgroup of 1024 threads per row (first half of this file), and five launches
+// that spread a row over many workgroups (second half; what the sampler uses, a
+// tenth of the time at a vocabulary of 152k). Penalties come from a list of the
+// row's tokens, or from a per-request history kept on the device.
 //
 //   greedy (temperature <= 1e-5): largest logit, ties to the lowest index.
 //   otherwise: z = logit / temperature; min_p drops z with

@@ -1,8 +1,9 @@
 """Turns logits rows into tokens on the device.
 
 One row per request that reached the end of its known tokens. All rows greedy:
-one argmax kernel. Otherwise: penalties (if any row has them) and the fused
-temperature -> min_p -> top-k/top-p -> draw kernel. A row's random number comes
+one argmax kernel. Otherwise: penalties (if any row has them; from a history of
+each request's tokens kept on the device) and the chain temperature -> min_p ->
+top-k/top-p -> draw, a row spread over many workgroups. A row's random number comes
 from (seed, number of tokens the request has produced so far), so it does not
 depend on the row's place in the batch or on the other rows
 (crates/core/src/sampler.rs:1-4,84,197-212; models/qwen3/src/executor.rs:534-605).
