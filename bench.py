@@ -2,7 +2,7 @@
 """In-process throughput of the engine on one MI355X: Qwen3-8B-shaped random weights.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L] [--shape 8b|14b|32b|0.6b]
-                    [--prompt P] [--context C]
+                    [--prompt P] [--context C] [--workload decode|serving [--sampled]]
 
 Prints ONE JSON line. `value` is decoded tokens per second at the default batch (8), each
 request with a 2,048-token prompt in a 4,096-token context; a "step" is one decode step
@@ -55,6 +55,50 @@ def model_numbers(c, dtype_bytes):
                 kv_bytes_per_token=L * 2 * Hkv * D * dtype_bytes)
 
 
+def serving(a, torch, Engine, SamplingParams, Qwen3Config) -> int:
+    """32 requests arrive at once: prompts uniform in [512, 3072] tokens, a step budget of 512 prompt tokens beside
+    the decoding requests, 256 outputs each. Timed from the first step (a cold engine: the first uses of a shape
+    pay for its measurement) to the last token."""
+    sizes = {**SIZES, **SHAPES[a.shape]}
+    if a.layers:
+        sizes["num_hidden_layers"] = a.layers
+    cfg = Qwen3Config.from_dict(sizes)
+    n_req, out_len, budget, ctx = 32, 256, 512, 4096
+    eng = Engine(config=cfg, seed=0, dtype=a.dtype, max_model_len=ctx, max_num_seqs=n_req, max_num_batched_tokens=budget,
+                 block_size=16, num_blocks=n_req * ctx // 16 + 64, hip_graph=not a.no_hip_graph)
+    rng = random.Random(0)
+    prompts = [[rng.randrange(cfg.vocab_size) for _ in range(rng.randint(512, 3072))] for _ in range(n_req)]
+    sp = (SamplingParams(max_tokens=out_len, temperature=0.7, top_k=50, top_p=0.9, presence_penalty=0.5, seed=3, ignore_eos=True)
+          if a.sampled else SamplingParams(max_tokens=out_len, temperature=0.0, ignore_eos=True))
+    for p in prompts:
+        eng.add_request(p, sp)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    steps = mixed = outs = 0
+    t_mixed = 0.0
+    while eng.has_unfinished():
+        ts = time.perf_counter()
+        got = eng.step()
+        steps += 1
+        outs += sum(1 for o in got if o.token is not None)
+        if eng.runner.batch.num_tokens != eng.runner.batch.num_reqs:
+            mixed += 1
+            t_mixed += time.perf_counter() - ts
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ptoks = sum(len(p) for p in prompts)
+    print(json.dumps({
+        "metric": f"tokens/s, prompt and output (Qwen3-{a.shape.upper()} shape, 32 requests, prompts 512-3072 in portions of 512, 256 outputs each)",
+        "value": round((ptoks + outs) / dt, 1), "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True,
+        "vs_baseline": None, "dtype": "bf16" if a.dtype == "bfloat16" else "fp32", "data": "synthetic",
+        "seconds": round(dt, 3), "prompt_tokens": ptoks, "output_tokens": outs, "output_tokens_per_s": round(outs / dt, 1),
+        "steps": steps, "steps_with_prompt_portions": mixed, "seconds_in_those": round(t_mixed, 3),
+        "sampling": "temperature 0.7, top-k 50, top-p 0.9, presence penalty 0.5" if a.sampled else "greedy",
+        "config": {"model": f"Qwen3-{a.shape.upper()} shape, random weights", "layers": sizes["num_hidden_layers"],
+                   "requests": n_req, "token_budget": budget, "context": ctx, "parallelism": "single GPU"}}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -69,6 +113,11 @@ def main() -> int:
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="layer sizes (default: Qwen3-8B)")
     ap.add_argument("--prompt", type=int, default=DEFAULT_PROMPT, help="prompt tokens per request (and of the timed prefill)")
     ap.add_argument("--context", type=int, default=DEFAULT_CONTEXT, help="max_model_len the engine is built for")
+    ap.add_argument("--workload", default="decode", choices=["decode", "serving"],
+                    help="serving: 32 requests with prompts of 512 to 3,072 tokens fed in portions of 512 beside the "
+                         "requests that decode, 256 outputs each (BASELINE.json names it for the 14B shape); its own JSON line")
+    ap.add_argument("--sampled", action="store_true",
+                    help="serving: temperature 0.7, top-k 50, top-p 0.9 and a presence penalty instead of greedy")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py measures one GPU only (this engine does not use a second one); got --gpus {a.gpus}")
@@ -77,6 +126,8 @@ def main() -> int:
     import torch
     from dinfer_amd import Engine, SamplingParams
     from dinfer_amd.config.qwen3 import Qwen3Config
+    if a.workload == "serving":
+        return serving(a, torch, Engine, SamplingParams, Qwen3Config)
 
     sizes = {**SIZES, **SHAPES[a.shape]}
     PROMPT, CONTEXT = a.prompt, a.context
