@@ -229,3 +229,57 @@ def test_prefix_cache_is_on_where_every_layer_keeps_its_keys(model_dirs):
     assert not engine(model_dirs["A"], "A", enable_prefix_caching=False).runner.cache.prefix_caching
     with pytest.raises(ValueError, match="keep every key"):
         engine(model_dirs["C"], "C", enable_prefix_caching=True)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_workloads_equal_the_plain_continuations(seed, tmp_path):
+    """Requests that arrive over time, share prompt stems (the prefix cache is on where the model allows), are cut
+    by small budgets, meet a pool so small that some are preempted, and are aborted now and then; graphs on or off.
+    In 32-bit, every request that finishes has generated exactly the plain implementation's greedy continuation,
+    and every page is back at the end."""
+    from dinfer_amd import Engine, SamplingParams
+    from dinfer_amd.config.qwen3 import Qwen3Config
+    from dinfer_amd.weights import write_random_model
+    rng = random.Random(500 + seed)
+    name = "ABC"[seed % 3]
+    cfgd, page = CONFIGS[name][0], PAGE[name]
+    write_random_model(Qwen3Config.from_dict(cfgd), tmp_path, seed=seed, dtype="float32")
+    cfg, w = plain.load(tmp_path)
+    nblocks = rng.choice([12, 20, 40])
+    maxlen = min(cfgd["max_position_embeddings"], nblocks * page)
+    eng = Engine(str(tmp_path), dtype="float32", max_model_len=maxlen, max_num_seqs=rng.choice([2, 4]),
+                 max_num_batched_tokens=rng.choice([8, 16, 64]), block_size=page, num_blocks=nblocks,
+                 hip_graph=seed % 2 == 0)
+    V = cfgd["vocab_size"]
+    stems = [[rng.randrange(V) for _ in range(rng.randint(1, 3 * page))] for _ in range(2)]
+    arrivals = []
+    for _ in range(rng.randint(4, 8)):
+        p = (rng.choice(stems) if rng.random() < 0.6 else []) + [rng.randrange(V) for _ in range(rng.randint(1, 2 * page))]
+        n = rng.randint(1, 8)
+        arrivals.append((rng.randint(0, 12), p[:maxlen - n], n))
+    arrivals.sort(key=lambda x: x[0])
+    asked, got, aborted, step = {}, {}, set(), 0
+    while arrivals or eng.has_unfinished():
+        while arrivals and arrivals[0][0] <= step:
+            _, p, n = arrivals.pop(0)
+            rid = eng.add_request(p, SamplingParams(max_tokens=n, temperature=0.0, ignore_eos=True))
+            asked[rid], got[rid] = (p, n), []
+        if rng.random() < 0.04 and got:
+            victim = rng.choice(list(got))
+            if len(got[victim]) < asked[victim][1]:
+                eng.abort(victim)
+                aborted.add(victim)
+        for o in eng.step():
+            if o.token is not None:
+                got[o.request_id].append(o.token)
+        step += 1
+        assert step < 2000, "the engine makes no progress"
+    eng.runner.cache.check()
+    assert all(eng.runner.cache.num_free(g) == nblocks for g in range(len(eng.runner.group_specs)))
+    for rid, (p, n) in asked.items():
+        if rid in aborted:
+            continue
+        ids = list(p)
+        for _ in range(n):
+            ids.append(int(plain.forward(cfg, w, ids)[-1].argmax()))
+        assert got[rid] == ids[len(p):], f"request {rid} (prompt of {len(p)}): {got[rid]} != {ids[len(p):]}"
