@@ -481,3 +481,153 @@ def test_toy_routing_position_encoding_and_shared_cache(tmp_path):
         unregister_architecture("ToyRoutedLM")
         FEED_FORWARDS.unregister("toy_routed")
         POSITION_ENCODINGS.unregister("toy_slowed_rotary")
+
+
+# ---- a norm of another kind and another arrangement of the block -----------------------------------------------
+def register_parallel_toy():
+    from dinfer_amd.config import ModelConfig, key, register_architecture
+    from dinfer_amd.parts import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Block, LayerSpec, ModelSpec, Norm, RunEntry,
+                                  TensorSpec, part)
+
+    class CenteredNorm(Norm):
+        """y = (x - mean) / sqrt(var + eps) * weight + bias (with `residual`: residual += x first, rows gathered by `rows`)."""
+
+        def __init__(self, width, eps):
+            self.width, self.eps = width, eps
+
+        def tensors(self):
+            return {"weight": TensorSpec((self.width,), init="gain"), "bias": TensorSpec((self.width,))}
+
+        def load(self, get):
+            self.weight, self.bias = get("weight").float(), get("bias").float()
+
+        def forward(self, x, out, n_rows, *, residual=None, rows=None):
+            idx = rows[:n_rows].long() if rows is not None else torch.arange(n_rows, device=x.device)
+            v = x[idx].float()
+            if residual is not None:
+                v = v + residual[idx].float()
+                residual[idx] = v.to(residual.dtype)
+            c = v - v.mean(-1, keepdim=True)
+            out[:n_rows] = (c / torch.sqrt(c.pow(2).mean(-1, keepdim=True) + self.eps) * self.weight + self.bias).to(out.dtype)
+            return out
+
+    class ParallelBlock(Block):
+        """h += mixer(norm(h)) + ff(norm(h)): one norm, both branches read it."""
+
+        def __init__(self, hidden, layer):
+            self.hidden = hidden
+            self.mixer = MIXERS.get(layer.mixer.kind)(hidden=hidden, **layer.mixer.params)
+            self.ff = FEED_FORWARDS.get(layer.feed_forward.kind)(hidden=hidden, **layer.feed_forward.params)
+            self.norm = NORMS.get(layer.norm.kind)(hidden, **layer.norm.params)
+            self._parts = (("attn.", self.mixer), ("ff.", self.ff), ("ln.", self.norm))
+
+        def tensors(self):
+            return {p + n: s for p, part_ in self._parts for n, s in part_.tensors().items()}
+
+        def load(self, get):
+            for p, part_ in self._parts:
+                part_.load(lambda name, _p=p, **kw: get(_p + name, **kw))
+
+        def bind(self, ctx):
+            for _, part_ in self._parts:
+                part_.bind(ctx)
+            self.normed = ctx.workspace.buffer("normed", self.hidden)
+            self.both = ctx.workspace.buffer("both_branches", self.hidden)
+
+        def forward(self, hidden, pending, batch, cache):
+            T = batch.num_tokens
+            self.norm.forward(hidden if pending is None else pending, self.normed, T,
+                              residual=None if pending is None else hidden)
+            a = self.mixer.forward(self.normed, batch, cache)
+            f = self.ff.forward(self.normed, batch)
+            self.both[:T] = a[:T] + f[:T]
+            return self.both
+
+    @dataclass(frozen=True)
+    class ParallelConfig(ModelConfig):
+        vocab_size: int = key(int)
+        hidden_size: int = key(int)
+        layers: int = key(int)
+        ARCHITECTURE = "ToyParallelLM"
+
+    def build_spec(c):
+        norm = part("toy_centered", eps=1e-5)
+        attn = part("attention", heads=4, kv_heads=2, head_dim=16, position=part("rotary", theta=1e4, max_positions=128))
+        layers = [LayerSpec(part("toy_parallel"), attn, part("gated_mlp", intermediate=56), norm, f"blocks.{i}.")
+                  for i in range(c.layers)]
+        return ModelSpec("ToyParallelLM", c.vocab_size, c.hidden_size, 128, layers, [RunEntry(i) for i in range(c.layers)],
+                         norm, "ln_f.", "wte.weight", "head.weight", tie_embeddings=True)
+
+    NORMS.register("toy_centered", CenteredNorm)
+    BLOCKS.register("toy_parallel", ParallelBlock)
+    register_architecture("ToyParallelLM", ParallelConfig, build_spec)
+    return ParallelConfig
+
+
+def parallel_toy_plain(w, ids, layers):
+    W = {k: v.double() for k, v in w.items()}
+    T = len(ids)
+    h = W["wte.weight"][ids]
+
+    def ln(x, p):
+        c = x - x.mean(-1, keepdim=True)
+        return c / torch.sqrt(c.pow(2).mean(-1, keepdim=True) + 1e-5) * W[p + "weight"] + W[p + "bias"]
+
+    for i in range(layers):
+        p = f"blocks.{i}."
+        x = ln(h, p + "ln.")
+        q = (x @ W[p + "attn.q_proj.weight"].T).view(T, 4, 16)
+        k = (x @ W[p + "attn.k_proj.weight"].T).view(T, 2, 16)
+        v = (x @ W[p + "attn.v_proj.weight"].T).view(T, 2, 16)
+        ang = plain.rope_angles(list(range(T)), 16, 1e4)
+        o = plain.causal_attention(plain.rope_neox(q, ang), plain.rope_neox(k, ang), v, 16 ** -0.5)
+        a = o.reshape(T, 64) @ W[p + "attn.o_proj.weight"].T
+        f = plain.swiglu_mlp(x, W[p + "ff.gate_proj.weight"], W[p + "ff.up_proj.weight"], W[p + "ff.down_proj.weight"])
+        h = h + a + f
+    return ln(h, "ln_f.") @ W["wte.weight"].T
+
+
+def test_toy_norm_and_block_arrangement(tmp_path):
+    """A norm that centres and has a bias, and a block whose two branches read one norm and are added together:
+    both defined here, registered, built from a configuration and stepped (whole, in portions, token by token,
+    the last step asking for the logits of a few rows only, which the final norm then gathers)."""
+    from safetensors.torch import load_file
+    from dinfer_amd.config import EngineOptions, unregister_architecture
+    from dinfer_amd.engine.batch import Entry
+    from dinfer_amd.engine.runner import ModelRunner
+    from dinfer_amd.parts import BLOCKS, NORMS
+    from dinfer_amd.weights import write_random_model
+    Config = register_parallel_toy()
+    try:
+        cfg = Config.from_dict(dict(vocab_size=89, hidden_size=48, layers=3, architectures=["ToyParallelLM"]))
+        write_random_model(cfg, tmp_path, seed=2, dtype="float32")
+        w = load_file(str(tmp_path / "model.safetensors"))
+        assert "blocks.2.ln.bias" in w and "ln_f.bias" in w and "head.weight" not in w
+        opt = EngineOptions(dtype="float32", max_model_len=128, max_num_seqs=2, max_num_batched_tokens=64, block_size=8,
+                            num_blocks=16, max_logits_rows=64)
+        r = ModelRunner.from_dir(tmp_path, opt)
+        rng = random.Random(6)
+        a = [rng.randrange(89) for _ in range(41)]
+        b = [rng.randrange(89) for _ in range(23)]
+        want = {"a": parallel_toy_plain(w, a, 3), "b": parallel_toy_plain(w, b, 3)}
+        seqs = {"a": a, "b": b}
+        fed = {"a": 0, "b": 0}
+        plan = [[("a", 30, None)], [("a", 1, None), ("b", 9, None)], [("a", 1, None), ("b", 1, None)],
+                [("a", 9, [0, 8]), ("b", 13, [12])]]
+        for st in plan:
+            entries = []
+            for k, n, wants in st:
+                assert r.reserve(k, fed[k], n)
+                entries.append(Entry(k, seqs[k][fed[k]:fed[k] + n], fed[k], list(range(n)) if wants is None else wants))
+            logits = r.step(entries).double().cpu()
+            i = 0
+            for e in entries:
+                for j in e.want:
+                    torch.testing.assert_close(logits[i], want[e.req_id][e.start + j], rtol=2e-4, atol=2e-5)
+                    i += 1
+                fed[e.req_id] += len(e.tokens)
+        assert fed == {"a": 41, "b": 23}
+    finally:
+        unregister_architecture("ToyParallelLM")
+        NORMS.unregister("toy_centered")
+        BLOCKS.unregister("toy_parallel")
