@@ -108,3 +108,40 @@ def test_decode_graph_with_library_products_replays_equal_eager(big_models):
         outs[graph] = got
     for step, (a, b) in enumerate(zip(outs[False], outs[True])):
         torch.testing.assert_close(b, a, rtol=2e-2, atol=2e-2, msg=lambda m: f"step {step}: {m}")
+
+
+def test_bfloat16_against_the_32bit_path_at_the_8b_layer_sizes(tmp_path):
+    """Four layers of the 8B sizes with a 32k vocabulary: the bfloat16 path (MFMA attention, weight-streaming and
+    library products) against the true 32-bit path of the same engine on the same weights. Rows whose best two
+    logits lie apart in 32-bit must keep their winner (the reference's rule, models/qwen3/tests/real_parity.rs:58-62,
+    129-145), prompt positions and decoded ones alike, and no logit strays by more than a fraction of its row's spread."""
+    from dinfer_amd.config import EngineOptions
+    from dinfer_amd.config.qwen3 import Qwen3Config
+    from dinfer_amd.engine.batch import Entry
+    from dinfer_amd.engine.runner import ModelRunner
+    from dinfer_amd.weights import write_random_model
+    cfg = dict(architectures=["Qwen3ForCausalLM"], vocab_size=32768, head_dim=128, num_hidden_layers=4, rms_norm_eps=1e-6,
+               rope_theta=1e6, max_position_embeddings=1024, tie_word_embeddings=False, **SHAPES["8B"])
+    write_random_model(Qwen3Config.from_dict(cfg), tmp_path, seed=9)
+    rng = random.Random(2)
+    toks = [rng.randrange(32768) for _ in range(330)]
+    got = {}
+    for dtype in ("float32", "bfloat16"):
+        opt = EngineOptions(dtype=dtype, max_model_len=1024, max_num_seqs=2, max_num_batched_tokens=512, block_size=16,
+                            num_blocks=64, max_logits_rows=512)
+        r = ModelRunner.from_dir(tmp_path, opt)
+        assert r.reserve("a", 0, 300)
+        rows = [r.step([Entry("a", toks[:300], 0, list(range(300)))]).float().cpu()]
+        for i in range(300, 330):
+            assert r.reserve("a", i, 1)
+            rows.append(r.step([Entry("a", [toks[i]], i, [0])]).float().cpu())
+        got[dtype] = torch.cat(rows)
+        del r
+        torch.cuda.empty_cache()
+    ref, low = got["float32"], got["bfloat16"]
+    spread = ref.std(-1, keepdim=True)
+    assert float(((low - ref).abs() / spread).max()) < 0.1
+    top2 = ref.topk(2, -1).values
+    clear = (top2[:, 0] - top2[:, 1]) > 0.15 * spread[:, 0]
+    assert int(clear.sum()) > 100
+    assert bool((low.argmax(-1)[clear] == ref.argmax(-1)[clear]).all())
