@@ -123,5 +123,5 @@ class DecoderModel:
         else:
             # the last add happens on the wanted rows only, inside the norm kernel
             self.final_norm.forward(pending, self.final_normed, R, residual=self.hidden, rows=batch.logits_rows)
-        gemm.matmul_nt(self.final_normed, self.head.weight, self.logits, R)
+        gemm.matmul_nt(self.final_normed, self.head.weight, self.logits, R, may_pad=True)  # both are buffers of max_rows rows
         return self.logits[:R]

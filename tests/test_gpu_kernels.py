@@ -598,7 +598,8 @@ def test_library_gemm_with_measured_algorithm():
             torch.testing.assert_close(out[:M].double(), want, rtol=2e-2, atol=2e-2, msg=lambda m_: f"{M}x{N}x{K} pad={pad}: {m_}")
             last = -(-M // gemm.ROW_BUCKET) * gemm.ROW_BUCKET if pad else M
             assert bool((out[last:] == 7.0).all()), f"{M}x{N}x{K} pad={pad}: rows past {last} were written"
-    assert any(p and p.tuned for p in blaslt._plans.values())
+    assert any(p and p.tuned for p in blaslt._plans.values())        # the larger shapes above were measured
+    assert any(p and not p.tuned for p in blaslt._plans.values())    # the tiny ones took the library's first suggestion
     # float32 out (logits at many positions): not rounded to bfloat16 on the way
     a = torch.randn(100, 264, device=DEV).to(torch.bfloat16)
     w = (torch.randn(1000, 264, device=DEV) * 0.05).to(torch.bfloat16)
