@@ -269,7 +269,7 @@ extern "C" int dinfer_gemm_small_m(int out_f32, const void* A, int64_t lda, cons
   if (nw == 0) {
     nw = (rt == 1 || N < 8192) ? 8 : 4;
     const int64_t steps = (K + 63) / 64;
-    while (nw > 1 && steps < 2 * nw) nw /= 2;  // every wave at least two k steps
+    while (nw > 1 && steps < 4 * nw) nw /= 2;  // every wave at least four k steps (K = 1024: 4 waves, measured)
   }
   while (nw > 1 && lds_bytes(nw, rt, mt) > 64 * 1024) nw /= 2;
   if (nw < 1 || nw > 16) return ERR_BAD_SHAPE;

@@ -21,7 +21,7 @@ WORKSPACE_BYTES = 128 << 20   # for the library's split-K and stream-K kernels
 CANDIDATES = 32               # how many of the library's suggestions are timed (the best has been seen as far down as 21st)
 FLUSH_BYTES = 512 << 20       # written before each timed run: twice the memory-side cache
 TUNE_FROM_ROWS = 33           # every size that comes here (up to 32 rows the weight-streaming kernel runs)
-TUNE_FROM_WORK = 1 << 28      # rows x columns x depth below which no choice of kernel repays its measurement
+TUNE_FROM_WORK = 1 << 24      # rows x columns x depth below which no choice of kernel repays its measurement
 
 _HIP_R_32F, _HIP_R_16BF = 0, 14
 _OP_N, _OP_T = 111, 112
