@@ -31,6 +31,7 @@ SOURCES = {
     "attention": "attention.hip",
     "gemm_ref": "gemm_ref.hip",
     "gemm": "gemm.hip",
+    "gemm_mid": "gemm_mid.hip",
     "sampling": "sampling.hip",
     "host": "host/api.cpp",
 }

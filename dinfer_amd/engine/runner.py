@@ -51,9 +51,11 @@ class ModelRunner:
         self._build_caches()
         self.batch = StepBatch(device, self.max_tokens, options.max_num_seqs, self.max_rows,
                                [self.max_blocks_per_seq] * len(self.group_specs))
-        # batch-size buckets of the decode graphs: powers of two and the largest batch
+        # batch-size buckets of the decode graphs: powers of two, from 32 on the step between two of them as well
+        # (the matrix products work in tiles of 16 rows: 48 rows cost them three quarters of 64), and the largest batch
         top = min(options.max_num_seqs, self.max_rows, self.max_tokens)
-        self._buckets = sorted({min(1 << i, top) for i in range(top.bit_length() + 1)})
+        sizes = {1 << i for i in range(top.bit_length() + 1)} | {3 << i for i in range(4, top.bit_length())}
+        self._buckets = sorted({min(x, top) for x in sizes})
         self._graphs: dict[int, torch.cuda.CUDAGraph] = {}
         self._graph_pool = None
 

@@ -128,15 +128,20 @@ def _run(handle, plan, algo, a, w, out, workspace) -> None:
                              WORKSPACE_BYTES, stream), "matmul")
 
 
+def flush_buffer(dev) -> torch.Tensor:
+    """FLUSH_BYTES of device memory; `zero_()` on it before a timed run pushes everything else out of the caches."""
+    flush = _flush.get(dev)
+    if flush is None:
+        flush = _flush[dev] = torch.empty(FLUSH_BYTES, dtype=torch.uint8, device=dev)
+    return flush
+
+
 def _tune(handle, plan, a, w, out, workspace) -> None:
     """Times every candidate on the call's own operands and keeps the fastest. In a model the weight of a
     product comes from HBM (the layers before have pushed it out of every cache), so each timed run follows a
     write of FLUSH_BYTES that empties the memory-side cache; timed on a weight that stays cached, kernels win
     that lose in place."""
-    dev = a.device
-    flush = _flush.get(dev)
-    if flush is None:
-        flush = _flush[dev] = torch.empty(FLUSH_BYTES, dtype=torch.uint8, device=dev)
+    flush = flush_buffer(a.device)
     best, best_t = plan.candidates[0], float("inf")
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     for algo in plan.candidates:

@@ -301,6 +301,30 @@ def gemm_small_m_gated(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: i
     return out
 
 
+def gemm_mid_m_workspace(m: int, n: int, k: int, *, gated: bool = False, ks: int = 0, rt: int = 0) -> int:
+    """Bytes of float workspace gemm_mid_m needs for these sizes (0: the product is stored directly)."""
+    need = ctypes.c_int64(0)
+    lib.call("dinfer_gemm_mid_m_workspace", m, n, k, 1 if gated else 0, ks, rt, ctypes.addressof(need))
+    return need.value
+
+
+def gemm_mid_m(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, workspace: torch.Tensor | None = None, *,
+               gated: bool = False, ks: int = 0, rt: int = 0) -> torch.Tensor:
+    """out[:m] = a[:m] @ w.T for m <= 64 (made for 33 to 64), bf16 operands; gated: w = [wg; wu] stacked
+    [2N, K] and out = silu(a @ wg.T) * (a @ wu.T). A narrow weight is cut into slices of k whose float
+    partial sums go through `workspace` and are added in slice order by a second kernel."""
+    _need_gpu(a, w, out, workspace)
+    k = w.shape[1]
+    n = w.shape[0] // 2 if gated else w.shape[0]
+    assert a.dtype == w.dtype == torch.bfloat16 and a.shape[1] == k and out.shape[1] == n
+    assert a.shape[0] >= m and out.shape[0] >= m and out.dtype in (torch.bfloat16, torch.float32)
+    assert workspace is None or workspace.is_contiguous()
+    lib.call("dinfer_gemm_mid_m", 1 if out.dtype == torch.float32 else 0, a.data_ptr(), _rows(a), w.data_ptr(), _rows(w),
+             out.data_ptr(), _rows(out), m, n, k, 1 if gated else 0, ks, rt, _ptr(workspace),
+             workspace.numel() * workspace.element_size() if workspace is not None else 0, _stream())
+    return out
+
+
 def argmax(logits: torch.Tensor, out: torch.Tensor, rows: int) -> torch.Tensor:
     _need_gpu(logits, out)
     assert logits.dtype == torch.float32 and out.dtype == torch.int32 and out.numel() >= rows

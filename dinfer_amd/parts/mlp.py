@@ -4,7 +4,7 @@ from __future__ import annotations
 
 import torch
 
-from ..kernels import gemm, ops
+from ..kernels import gemm
 from .base import FeedForward
 from .linear import Linear
 from .registry import FEED_FORWARDS
@@ -38,10 +38,6 @@ class GatedMLP(FeedForward):
 
     def forward(self, x, batch):
         T = batch.num_tokens
-        if gemm.fuses_gated_act(x, self.gate_up.weight, T, self.act):
-            # decode-sized steps: both projections and the activation in one weight-streaming kernel
-            ops.gemm_small_m_gated(x, self.gate_up.weight, self.act_buf, T)
-        else:
-            self.gate_up.forward(x, self.gu_buf, T, scratch=True)
-            ops.gated_act(self.gu_buf, self.act_buf, T, self.act)
+        # decode-sized steps: both projections and the activation in one weight-streaming kernel
+        gemm.gated_nt(x, self.gate_up.weight, self.act_buf, self.gu_buf, T, self.act)
         return self.down.forward(self.act_buf, self.out_buf, T, scratch=True)

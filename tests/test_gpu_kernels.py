@@ -624,6 +624,65 @@ def test_gemm_small_m_gated(M):
             assert bool((err <= 1e-2 * want.abs() + 1e-3 * want.std()).all()), f"M={M} N={N} K={K}: {float(err.max())}"
 
 
+@pytest.mark.parametrize("M", [1, 17, 32, 33, 48, 64])
+def test_gemm_mid_m(M):
+    """The product that keeps a slice of the activations in LDS, plain and gated, against float64: sizes that are no
+    multiples of its tiles, slices that end inside a 64-wide step, one slice and many, every form it has."""
+    from dinfer_amd.kernels.lib import KernelError
+    ran = 0
+    for N, K in ((96, 512), (332, 80), (4096, 4096), (1000, 1096), (52, 8), (260, 2600)):
+        a = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+        w = (torch.randn(2 * N, K, device=DEV) * 0.05).to(torch.bfloat16)
+        z = a.double() @ w.double().T
+        for gated in (False, True):
+            want = plain.silu(z[:, :N]) * z[:, N:] if gated else z[:, :N]
+            for ks, rt in ((0, 0), (1024, 1), (1024, 2), (64, 4), (2048, 1), (1536, 2), (256, 1)):
+                try:
+                    need = ops().gemm_mid_m_workspace(M, N, K, gated=gated, ks=ks, rt=rt)
+                except KernelError:
+                    assert M > 32 and ks > 1024          # only a slice that LDS does not hold is refused
+                    continue
+                ws = torch.full((need // 4 + 8,), float("nan"), device=DEV)
+                for out_dtype in (torch.bfloat16,) if gated else (torch.bfloat16, torch.float32):
+                    out = torch.full((M + 2, N), 7.0, device=DEV, dtype=out_dtype)
+                    ops().gemm_mid_m(a, w if gated else w[:N], out, M, ws, gated=gated, ks=ks, rt=rt)
+                    err = (out[:M].double() - want).abs()
+                    tol = 1e-2 * want.abs() + 1e-3 * want.std() if out_dtype == torch.bfloat16 else 1e-4 * want.abs() + 1e-4
+                    assert bool((err <= tol).all()), f"M={M} N={N} K={K} gated={gated} ks={ks} rt={rt}: {float(err.max())}"
+                    assert bool((out[M:] == 7.0).all())
+                    ran += 1
+                with pytest.raises(KernelError):             # a workspace that is too small is refused, not overrun
+                    ops().gemm_mid_m(a, w if gated else w[:N], out, M, ws[:max(need // 4 - 16, 0)], gated=gated, ks=ks, rt=rt)
+    assert ran >= 60
+
+
+def test_products_of_17_to_64_rows_take_the_measured_kernel():
+    """Between the few-row kernel and the library the kernel is chosen per shape by timing; whatever wins, the
+    product is right, twice in a row (the first call measures), plain and gated, bfloat16 and float32 out."""
+    from dinfer_amd.kernels import gemm
+    for M in (17, 32, 33, 50, 64):
+        for N, K in ((96, 512), (1000, 1096), (333, 264), (2048, 4096)):
+            a = torch.randn(M + 70, K, device=DEV).to(torch.bfloat16)
+            w = (torch.randn(2 * N, K, device=DEV) * 0.05).to(torch.bfloat16)
+            z = a[:M].double() @ w.double().T
+            for out_dtype in (torch.bfloat16, torch.float32):
+                out = torch.full((M + 70, 2 * N), 7.0, device=DEV, dtype=out_dtype)
+                for _ in range(2):
+                    gemm.matmul_nt(a, w, out, M, may_pad=True)
+                t = dict(rtol=2e-2, atol=2e-2) if out_dtype == torch.bfloat16 else dict(rtol=1e-4, atol=1e-4)
+                torch.testing.assert_close(out[:M].double(), z, **t, msg=lambda m_: f"{M}x{2 * N}x{K}: {m_}")
+                assert bool((out[96:] == 7.0).all())
+            want = plain.silu(z[:, :N]) * z[:, N:]
+            act = torch.full((M + 70, N), 7.0, device=DEV, dtype=torch.bfloat16)
+            scratch = torch.empty(M + 70, 2 * N, device=DEV, dtype=torch.bfloat16)
+            for _ in range(2):
+                gemm.gated_nt(a, w, act, scratch, M, "silu")
+            err = (act[:M].double() - want).abs()
+            assert bool((err <= 2e-2 * want.abs() + 2e-3 * want.std()).all()), f"gated {M}x{N}x{K}: {float(err.max())}"
+            assert bool((act[M:] == 7.0).all())
+    assert len(gemm._choice) >= 8 and len(set(gemm._choice.values())) >= 1
+
+
 @pytest.mark.parametrize("start", [0, 8, 3])
 def test_qkv_post_many_tokens_writes_v_transposed(start):
     """From 64 tokens on, V is written by the gathering kernel: slots that start on a multiple of 8
