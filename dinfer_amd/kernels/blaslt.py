@@ -13,13 +13,14 @@ from __future__ import annotations
 
 import ctypes
 import os
+import sys
 from ctypes import POINTER, byref, c_float, c_int, c_int32, c_int64, c_size_t, c_uint64, c_void_p
 
 import torch
 
 WORKSPACE_BYTES = 128 << 20   # for the library's split-K and stream-K kernels
 CANDIDATES = 32               # how many of the library's suggestions are timed (the best has been seen as far down as 21st)
-FLUSH_BYTES = 512 << 20       # written before each timed run: twice the memory-side cache
+FLUSH_BYTES = 512 << 20       # read before each timed run: twice the memory-side cache
 TUNE_FROM_ROWS = 33           # every size that comes here (up to 32 rows the weight-streaming kernel runs)
 TUNE_FROM_WORK = 1 << 24      # rows x columns x depth below which no choice of kernel repays its measurement
 
@@ -128,28 +129,29 @@ def _run(handle, plan, algo, a, w, out, workspace) -> None:
                              WORKSPACE_BYTES, stream), "matmul")
 
 
-def flush_buffer(dev) -> torch.Tensor:
-    """FLUSH_BYTES of device memory; `zero_()` on it before a timed run pushes everything else out of the caches."""
+def flush_caches(dev) -> None:
+    """Reads FLUSH_BYTES of other memory, so that what runs next finds its operands in HBM, as a weight is found
+    in a model whose other layers have passed through the caches since. Read, not written: lines written here
+    would still be on their way out while the timed kernel runs, and compete with it."""
     flush = _flush.get(dev)
     if flush is None:
-        flush = _flush[dev] = torch.empty(FLUSH_BYTES, dtype=torch.uint8, device=dev)
-    return flush
+        flush = _flush[dev] = torch.zeros(FLUSH_BYTES // 4, dtype=torch.int32, device=dev)
+    flush.sum()
 
 
 def _tune(handle, plan, a, w, out, workspace) -> None:
     """Times every candidate on the call's own operands and keeps the fastest. In a model the weight of a
     product comes from HBM (the layers before have pushed it out of every cache), so each timed run follows a
-    write of FLUSH_BYTES that empties the memory-side cache; timed on a weight that stays cached, kernels win
+    read of FLUSH_BYTES of other memory that empties the memory-side cache; timed on a weight that stays cached, kernels win
     that lose in place."""
-    flush = flush_buffer(a.device)
-    best, best_t = plan.candidates[0], float("inf")
+    best, best_t, best_i, times = plan.candidates[0], float("inf"), 0, []
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    for algo in plan.candidates:
+    for i, algo in enumerate(plan.candidates):
         try:
             _run(handle, plan, algo, a, w, out, workspace)   # first use of a kernel loads it
             t = float("inf")
             for _ in range(3):   # the least of three: a single timing wanders by a few per cent, as much as the candidates differ
-                flush.zero_()
+                flush_caches(a.device)
                 start.record()
                 _run(handle, plan, algo, a, w, out, workspace)
                 end.record()
@@ -157,9 +159,13 @@ def _tune(handle, plan, a, w, out, workspace) -> None:
                 t = min(t, start.elapsed_time(end))
         except RuntimeError:
             continue
+        times.append(round(t * 1e3, 1))
         if t < best_t:
-            best, best_t = algo, t
+            best, best_t, best_i = algo, t, i
     plan.algo, plan.tuned = best, True
+    if os.environ.get("DINFER_GEMM_TUNE_LOG"):
+        print(f"[dinfer_amd] library product {tuple(out.shape)[1]} x {tuple(a.shape)[1]}, {out.dtype}: algorithm {best_i} of {times} (us)",
+              file=sys.stderr, flush=True)
 
 
 def matmul(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int) -> torch.Tensor:
