@@ -135,7 +135,7 @@ def flush_caches(dev) -> None:
     would still be on their way out while the timed kernel runs, and compete with it."""
     flush = _flush.get(dev)
     if flush is None:
-        flush = _flush[dev] = torch.zeros(FLUSH_BYTES // 4, dtype=torch.int32, device=dev)
+        flush = _flush[dev] = torch.zeros(FLUSH_BYTES // 4, dtype=torch.float32, device=dev)   # summed as it is: no widened copy
     flush.sum()
 
 
