@@ -39,14 +39,19 @@ TALL_BYTES = 32 << 20
 ROW_BUCKET = 32
 
 _workspace: dict = {}   # device -> float32 buffer for partial sums
+_outgrown: list = []    # earlier, smaller buffers: graphs captured with them still write there
 
 
 def _mid_workspace(dev, need: int) -> torch.Tensor | None:
-    """The buffer for partial sums, grown to `need` bytes; None where it would have to grow under capture."""
+    """The buffer for partial sums, grown to `need` bytes; None where it would have to grow under capture.
+    A buffer that is outgrown is kept, never freed: a captured graph holds its address."""
     ws = _workspace.get(dev)
     if ws is None or ws.numel() * 4 < need:
         if torch.cuda.is_current_stream_capturing():
             return None
+        if ws is not None:
+            _outgrown.append(ws)
+            need = max(need, 2 * ws.numel() * 4)
         ws = _workspace[dev] = torch.empty((need + 3) // 4, dtype=torch.float32, device=dev)
     return ws
 

@@ -683,6 +683,36 @@ def test_products_of_17_to_64_rows_by_the_rule_of_sizes():
     assert seen == {True, False}          # both sides of the rule were met
 
 
+def test_a_graph_keeps_its_partial_sums_when_the_buffer_grows():
+    """A decode graph captured while the buffer for partial sums was small must still be right after a larger
+    product has made the buffer grow: the old buffer stays where it is and belongs to nobody else."""
+    from dinfer_amd.kernels import gemm
+    M, N, K = 20, 2048, 8192
+    assert gemm._tall(M, N, K)
+    a = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(N, K, device=DEV) * 0.05).to(torch.bfloat16)
+    out = torch.zeros(M, N, device=DEV, dtype=torch.bfloat16)
+    gemm._workspace.pop(a.device, None)                  # as in a new process: the first product sizes the buffer
+    gemm.matmul_nt(a, w, out, M)
+    want = out.clone()
+    small = gemm._workspace[a.device]
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        gemm.matmul_nt(a, w, out, M)
+    a2 = torch.randn(64, 4 * K, device=DEV).to(torch.bfloat16)
+    w2 = (torch.randn(N, 4 * K, device=DEV) * 0.05).to(torch.bfloat16)
+    gemm.matmul_nt(a2, w2, torch.empty(64, N, device=DEV, dtype=torch.bfloat16), 64)   # needs more: the buffer grows
+    assert gemm._workspace[a.device] is not small and gemm._workspace[a.device].numel() > small.numel()
+    del small
+    others = [torch.full((1 << 20,), 3.0, device=DEV) for _ in range(16)]                # would land in freed memory
+    for _ in range(2):
+        out.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want)
+    assert all(bool((t == 3.0).all()) for t in others)
+
+
 @pytest.mark.parametrize("start", [0, 8, 3])
 def test_qkv_post_many_tokens_writes_v_transposed(start):
     """From 64 tokens on, V is written by the gathering kernel: slots that start on a multiple of 8
