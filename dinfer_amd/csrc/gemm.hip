@@ -263,9 +263,13 @@ extern "C" int dinfer_gemm_small_m(int out_f32, const void* A, int64_t lda, cons
   const int mt = (int)(M + 15) / 16;
   int rt = row_tiles_per_block, nw = waves;
   // measured on MI355X (K = 4096 and 12288, N from 4096 to 151936): one row tile and 8 waves a workgroup,
-  // two row tiles and 4 waves from N = 8192 on when there are more than a few tokens (four row tiles for a
-  // vocabulary-sized N at 17 to 32 tokens)
-  if (rt == 0) rt = mt >= 2 ? ((mt == 2 && N >= 65536) ? 4 : 2) : ((N >= 8192 && M > 4) ? 2 : 1);
+  // two row tiles and 4 waves from N = 8192 on when there are more than a few tokens; with two token tiles
+  // and more, two row tiles from N = 6144 on and for every weight large enough to be read past the caches
+  // (32 tokens: N = K = 4096 9.1 us with one row tile, 11.2 with two; N = K = 5120 24.0 with one, 18.3 with
+  // two); four row tiles for a vocabulary-sized N at 17 to 32 tokens
+  if (rt == 0)
+    rt = mt >= 2 ? ((mt == 2 && N >= 65536) ? 4 : ((N >= 6144 || streams_weight(N, K)) ? 2 : 1))
+                 : ((N >= 8192 && M > 4) ? 2 : 1);
   if (nw == 0) {
     nw = (rt == 1 || N < 8192) ? 8 : 4;
     const int64_t steps = (K + 63) / 64;
