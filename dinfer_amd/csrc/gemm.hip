@@ -23,6 +23,14 @@
 //
 // K must be a multiple of 8 (16-byte loads); any M <= 64, any N.
 //
+// Two more forms take the norm kernels out of a decode layer (a kernel costs 3 to 5 us however small):
+//   SINK    the product is added to the residual stream in place (one rounding), and what the next RMSNorm
+//           needs leaves with it: the new stream times that norm's gain (XG), and per token and tile of 16
+//           columns the sum of squares of the new stream (rounded as stored), in float;
+//   SCALED  the consumer of those: A is XG, and every token's result is multiplied by
+//           rsqrt(sum of its partial sums of squares / width + eps) before it is stored (or gated).
+// Together: y = (x g) W^T / rms(x) instead of ((x / rms(x)) g) W^T, the same value rounded at other places.
+//
 // Reference behaviour: crates/kernels/cuda/gemm_small_m.cu:42-114,148-285
 // (weight read once, split-K, M <= 32).
 #include "common.cuh"
@@ -67,13 +75,36 @@ __device__ __forceinline__ void store4<bf16>(bf16* p, f32x4 v) {
 }
 
 
+enum : int { PLAIN = 0, SCALED = 1, SINK = 2 };
+
+// LDS of a workgroup: a strip per wave while streaming, then the partial sums of every wave
+__host__ __device__ inline size_t lds_core_bytes(int waves, int rt, int mt) {
+  const size_t strips = (size_t)waves * 16 * 144, sums = (size_t)waves * rt * mt * 64 * sizeof(f32x4);
+  return strips > sums ? strips : sums;
+}
+
+// What the SCALED and SINK forms need beside the product's own operands.
+struct NormLink {
+  const float* stats;  // SCALED: [M][ld_stats] partial sums of squares, `cols` of them a token
+  float* stats_out;    // SINK: where this product's partial sums go, one a token and tile of 16 columns
+  int64_t ld_stats;
+  int cols;
+  float eps, inv_width;
+  bf16* xg;            // SINK: the new stream times the next norm's gain
+  int64_t ld_xg;
+  const void* gain;    // SINK: that gain, bf16 or float (gain_f32), plus gain_offset
+  int gain_f32;
+  float gain_offset;
+};
+
 // GATED (RT == 2): W is [2N, K], rows [0, N) the gate and [N, 2N) the up projection; the workgroup's
 // two row tiles are gate rows n0.. and up rows N + n0.., and the epilogue stores
 // silu(gate) * up into C [M, N]: the activation costs no pass of its own.
-template <int MT, int RT, class O, bool GATED, bool STREAM>
+template <int MT, int RT, class O, bool GATED, bool STREAM, int MODE = PLAIN>
 __global__ void __launch_bounds__(1024) gemm_small_m_kernel(const bf16* __restrict__ A, int64_t lda,
                                                             const bf16* __restrict__ W, int64_t ldw,
-                                                            O* __restrict__ C, int64_t ldc, int M, int N, int K) {
+                                                            O* __restrict__ C, int64_t ldc, int M, int N, int K,
+                                                            NormLink link = NormLink{}) {
   static_assert(!GATED || RT == 2, "the gated form pairs one gate tile with one up tile");
   // 64-wide k steps in flight per wave: as many as the register file takes at 16 waves a workgroup
   constexpr int UNROLL = MT <= 2 ? (4 / RT > 0 ? 4 / RT : 1) : (2 / RT > 0 ? 2 / RT : 1);
@@ -163,6 +194,17 @@ __global__ void __launch_bounds__(1024) gemm_small_m_kernel(const bf16* __restri
       }
     }
   }
+  // SCALED: every token's 1 / rms from the producer's partial sums, added in a fixed order; kept behind the
+  // strips and the sums (the launch sizes LDS for it)
+  float* rs = (float*)(smem + lds_core_bytes(nw, RT, MT));
+  if constexpr (MODE == SCALED) {
+    for (int m = wave; m < M; m += nw) {
+      float a = 0.f;
+      for (int j = lane; j < link.cols; j += 64) a += link.stats[(int64_t)m * link.ld_stats + j];
+      a = wave_sum(a);
+      if (lane == 0) rs[m] = rsqrtf(a * link.inv_width + link.eps);
+    }
+  }
   __syncthreads();  // the strips are done with: the same memory now takes the sums
 
   // partial sums of the waves meet in LDS
@@ -179,6 +221,12 @@ __global__ void __launch_bounds__(1024) gemm_small_m_kernel(const bf16* __restri
       const f32x4 v = ((const f32x4*)red)[(int64_t)w * RT * MT * 64 + x];
       s[0] += v[0]; s[1] += v[1]; s[2] += v[2]; s[3] += v[3];
     }
+    const int tile = x >> 6, ln = x & 63;
+    const int r = tile / MT, t = tile % MT;
+    const int m = t * 16 + (ln & 15);
+    const int n = n0 + r * 16 + 4 * (ln >> 4);
+    float scale = 1.f;
+    if constexpr (MODE == SCALED) scale = m < M ? rs[m] : 0.f;
     if (GATED) {  // slot x of the up tile lies MT * 64 slots further on
       f32x4 u = ((const f32x4*)red)[MT * 64 + x];
       for (int w = 1; w < nw; ++w) {
@@ -186,13 +234,35 @@ __global__ void __launch_bounds__(1024) gemm_small_m_kernel(const bf16* __restri
         u[0] += v[0]; u[1] += v[1]; u[2] += v[2]; u[3] += v[3];
       }
 #pragma unroll
-      for (int e = 0; e < 4; ++e) s[e] = (s[e] / (1.f + expf(-s[e]))) * u[e];
+      for (int e = 0; e < 4; ++e) {
+        const float g = s[e] * scale;
+        s[e] = (g / (1.f + expf(-g))) * (u[e] * scale);
+      }
+    } else if constexpr (MODE == SCALED) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) s[e] *= scale;
     }
-    const int tile = x >> 6, ln = x & 63;
-    const int r = tile / MT, t = tile % MT;
-    const int m = t * 16 + (ln & 15);
-    const int n = n0 + r * 16 + 4 * (ln >> 4);
-    if (m < M) {
+    if constexpr (MODE == SINK) {
+      // C is the residual stream: read, added to, rounded once, written back; the same lanes feed the next norm
+      float ss = 0.f;
+      if (m < M) {
+        bf16* hp = (bf16*)C + (int64_t)m * ldc + n;
+        bf16* xp = link.xg + (int64_t)m * link.ld_xg + n;
+        for (int e = 0; e < 4 && n + e < N; ++e) {
+          const bf16 h = (bf16)((float)hp[e] + s[e]);
+          const float hf = (float)h;
+          hp[e] = h;
+          ss += hf * hf;
+          const float g = (link.gain_f32 ? ((const float*)link.gain)[n + e] : (float)((const bf16*)link.gain)[n + e]) +
+                          link.gain_offset;
+          xp[e] = (bf16)(hf * g);
+        }
+      }
+      // the tile's 16 columns of a token lie in the four lanes ln, ln + 16, + 32, + 48
+      ss += __shfl_xor(ss, 16, 64);
+      ss += __shfl_xor(ss, 32, 64);
+      if ((ln >> 4) == 0 && m < M) link.stats_out[(int64_t)m * link.ld_stats + (n0 >> 4) + r] = ss;
+    } else if (m < M) {
       O* cp = C + (int64_t)m * ldc + n;
       if (n + 3 < N) {
         store4<O>(cp, s);
@@ -205,11 +275,8 @@ __global__ void __launch_bounds__(1024) gemm_small_m_kernel(const bf16* __restri
 
 inline bool streams_weight(int64_t rows, int64_t K) { return rows * K * (int64_t)sizeof(bf16) >= (int64_t)40 << 20; }
 
-// LDS of a workgroup: a strip per wave while streaming, then the partial sums of every wave
-inline size_t lds_bytes(int waves, int rt, int mt) {
-  const size_t strips = (size_t)waves * 16 * 144, sums = (size_t)waves * rt * mt * 64 * sizeof(f32x4);
-  return strips > sums ? strips : sums;
-}
+inline size_t lds_bytes(int waves, int rt, int mt) { return lds_core_bytes(waves, rt, mt); }
+constexpr size_t RS_BYTES = 64 * sizeof(float);  // SCALED: a token's 1 / rms, behind the rest
 
 template <int MT, int RT, class O>
 int launch(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, O* C, int64_t ldc, int M, int N, int K, int waves,
@@ -246,6 +313,59 @@ int dispatch(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, O* C, int64
   if (mt == 4) { if (rt == 1) GO(4, 1); if (rt == 2) GO(4, 2); }
 #undef GO
   return ERR_UNSUPPORTED;
+}
+
+// The SCALED and SINK forms: up to 32 rows, bf16 out, one or two row tiles.
+template <int MT, int RT, int MODE>
+int launch_linked(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, bf16* C, int64_t ldc, int M, int N, int K,
+                  int waves, const NormLink& link, hipStream_t stream) {
+  const int row_tiles = (N + 16 * RT - 1) / (16 * RT);
+  const size_t lds = lds_bytes(waves, RT, MT) + RS_BYTES;
+  if (streams_weight(N, K))
+    gemm_small_m_kernel<MT, RT, bf16, false, true, MODE><<<(unsigned)row_tiles, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, link);
+  else
+    gemm_small_m_kernel<MT, RT, bf16, false, false, MODE><<<(unsigned)row_tiles, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, link);
+  return launch_status();
+}
+
+template <int MODE>
+int dispatch_linked(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, bf16* C, int64_t ldc, int M, int N, int K,
+                    int rt, int waves, const NormLink& link, hipStream_t stream) {
+  const int mt = (M + 15) / 16;
+#define GO(MT_, RT_) return launch_linked<MT_, RT_, MODE>(A, lda, W, ldw, C, ldc, M, N, K, waves, link, stream)
+  if (mt == 1) { if (rt == 1) GO(1, 1); if (rt == 2) GO(1, 2); }
+  if (mt == 2) { if (rt == 1) GO(2, 1); if (rt == 2) GO(2, 2); }
+#undef GO
+  return ERR_UNSUPPORTED;
+}
+
+template <int MT>
+int launch_gated_scaled(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, bf16* C, int64_t ldc, int M, int N, int K,
+                        int waves, const NormLink& link, hipStream_t stream) {
+  const int col_tiles = (N + 15) / 16;
+  const size_t lds = lds_bytes(waves, 2, MT) + RS_BYTES;
+  if (streams_weight(2 * (int64_t)N, K))
+    gemm_small_m_kernel<MT, 2, bf16, true, true, SCALED><<<(unsigned)col_tiles, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, link);
+  else
+    gemm_small_m_kernel<MT, 2, bf16, true, false, SCALED><<<(unsigned)col_tiles, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, link);
+  return launch_status();
+}
+
+// Row tiles and waves of a launch, as dinfer_gemm_small_m chooses them (at most two row tiles here).
+inline void shape_for(int64_t M, int64_t N, int64_t K, int* rt_out, int* nw_out) {
+  const int mt = (int)(M + 15) / 16;
+  int rt = mt >= 2 ? ((N >= 6144 || streams_weight(N, K)) ? 2 : 1) : ((N >= 8192 && M > 4) ? 2 : 1);
+  int nw = (rt == 1 || N < 8192) ? 8 : 4;
+  const int64_t steps = (K + 63) / 64;
+  while (nw > 1 && steps < 4 * nw) nw /= 2;
+  while (nw > 1 && lds_bytes(nw, rt, mt) + RS_BYTES > 64 * 1024) nw /= 2;
+  *rt_out = rt, *nw_out = nw;
+}
+
+inline bool linked_operands_ok(const void* A, int64_t lda, const void* W, int64_t ldw, int64_t ldc, int64_t M, int64_t N,
+                               int64_t K) {
+  return M > 0 && M <= 32 && N > 0 && K > 0 && K % 8 == 0 && lda >= K && ldw >= K && ldc >= N && lda % 8 == 0 &&
+         ldw % 8 == 0 && N <= 0x3fffffff && K <= 0x7fffffff && !((uintptr_t)A % 16) && !((uintptr_t)W % 16);
 }
 
 }  // namespace
@@ -308,4 +428,56 @@ extern "C" int dinfer_gemm_small_m_gated(const void* A, int64_t lda, const void*
   if (mt == 1)
     return launch_gated<1>((const bf16*)A, lda, (const bf16*)W, ldw, (bf16*)C, ldc, (int)M, (int)N, (int)K, nw, stream);
   return launch_gated<2>((const bf16*)A, lda, (const bf16*)W, ldw, (bf16*)C, ldc, (int)M, (int)N, (int)K, nw, stream);
+}
+
+
+// C[:M] = (A . W^T) scaled per row by rsqrt(sum(stats[m][0..cols)) / width + eps): A is the residual stream times the
+// gain of an RMSNorm (dinfer_gemm_small_m_sink wrote both it and stats), so C is W applied to the normed stream.
+// gated: W = [gate; up] stacked [2N, K] and C[M,N] = silu(scaled gate) * scaled up. M <= 32, bf16 in and out.
+extern "C" int dinfer_gemm_small_m_scaled(const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc,
+                                          int64_t M, int64_t N, int64_t K, int gated, const float* stats, int64_t ld_stats,
+                                          int64_t cols, float eps, int64_t width, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return OK;
+  if (M > 32) return ERR_UNSUPPORTED;
+  if (!linked_operands_ok(A, lda, W, ldw, ldc, M, N, K) || !stats || cols <= 0 || cols > ld_stats || width <= 0 ||
+      cols > 0x7fffffff)
+    return ERR_BAD_SHAPE;
+  NormLink link{};
+  link.stats = stats, link.ld_stats = ld_stats, link.cols = (int)cols, link.eps = eps, link.inv_width = 1.f / (float)width;
+  const int mt = (int)(M + 15) / 16;
+  if (gated) {
+    const int64_t tiles = (N + 15) / 16;
+    int nw = 4;
+    while (nw < 16 && tiles * nw < 768) nw *= 2;
+    const int64_t steps = (K + 63) / 64;
+    while (nw > 1 && steps < 2 * nw) nw /= 2;
+    while (nw > 1 && lds_bytes(nw, 2, mt) + RS_BYTES > 64 * 1024) nw /= 2;
+    if (mt == 1)
+      return launch_gated_scaled<1>((const bf16*)A, lda, (const bf16*)W, ldw, (bf16*)C, ldc, (int)M, (int)N, (int)K, nw, link, stream);
+    return launch_gated_scaled<2>((const bf16*)A, lda, (const bf16*)W, ldw, (bf16*)C, ldc, (int)M, (int)N, (int)K, nw, link, stream);
+  }
+  int rt, nw;
+  shape_for(M, N, K, &rt, &nw);
+  return dispatch_linked<SCALED>((const bf16*)A, lda, (const bf16*)W, ldw, (bf16*)C, ldc, (int)M, (int)N, (int)K, rt, nw, link,
+                                 stream);
+}
+
+// H[:M] += A . W^T in place (H bf16, the residual stream; summed in float, rounded once), and for the RMSNorm that
+// reads H next: XG[:M] = H * (gain + gain_offset), and stats[m][j] = sum of squares of H[m] over columns 16 j .. 16 j + 15
+// (ceil(N / 16) of them a token). M <= 32.
+extern "C" int dinfer_gemm_small_m_sink(const void* A, int64_t lda, const void* W, int64_t ldw, void* H, int64_t ldh, void* XG,
+                                        int64_t ld_xg, const void* gain, int gain_f32, float gain_offset, float* stats,
+                                        int64_t ld_stats, int64_t M, int64_t N, int64_t K, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return OK;
+  if (M > 32) return ERR_UNSUPPORTED;
+  if (!linked_operands_ok(A, lda, W, ldw, ldh, M, N, K) || !H || !XG || !gain || !stats || ld_xg < N ||
+      ld_stats < (N + 15) / 16)
+    return ERR_BAD_SHAPE;
+  NormLink link{};
+  link.stats_out = stats, link.ld_stats = ld_stats, link.xg = (bf16*)XG, link.ld_xg = ld_xg, link.gain = gain;
+  link.gain_f32 = gain_f32, link.gain_offset = gain_offset;
+  int rt, nw;
+  shape_for(M, N, K, &rt, &nw);
+  return dispatch_linked<SINK>((const bf16*)A, lda, (const bf16*)W, ldw, (bf16*)H, ldh, (int)M, (int)N, (int)K, rt, nw, link,
+                               stream);
 }

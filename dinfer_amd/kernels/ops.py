@@ -301,6 +301,37 @@ def gemm_small_m_gated(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: i
     return out
 
 
+def gemm_small_m_sink(a: torch.Tensor, w: torch.Tensor, stream_: torch.Tensor, xg: torch.Tensor, gain: torch.Tensor,
+                      stats: torch.Tensor, m: int, *, gain_offset: float = 0.0) -> None:
+    """stream_[:m] += a[:m] @ w.T in place (the residual stream: summed in float, rounded once), and what the RMSNorm
+    that reads it next needs: xg[:m] = stream_ * (gain + gain_offset), stats[r, j] = sum of squares of stream_[r] over
+    columns 16 j .. 16 j + 15. m <= 32, bf16."""
+    _need_gpu(a, w, stream_, xg, gain, stats)
+    n, k = w.shape
+    assert a.dtype == w.dtype == stream_.dtype == xg.dtype == torch.bfloat16 and stats.dtype == torch.float32
+    assert a.shape[1] == k and stream_.shape[1] == n and xg.shape[1] == n and gain.numel() == n and gain.is_contiguous()
+    assert min(a.shape[0], stream_.shape[0], xg.shape[0], stats.shape[0]) >= m and stats.shape[1] >= -(-n // 16)
+    lib.call("dinfer_gemm_small_m_sink", a.data_ptr(), _rows(a), w.data_ptr(), _rows(w), stream_.data_ptr(), _rows(stream_),
+             xg.data_ptr(), _rows(xg), gain.data_ptr(), _is_param_f32(gain, torch.bfloat16), float(gain_offset),
+             stats.data_ptr(), _rows(stats), m, n, k, _stream())
+
+
+def gemm_small_m_scaled(xg: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, stats: torch.Tensor, cols: int,
+                        eps: float, width: int, *, gated: bool = False) -> torch.Tensor:
+    """out[:m] = (xg[:m] @ w.T) * rsqrt(sum(stats[r, :cols]) / width + eps) per row r: with xg and stats from
+    gemm_small_m_sink, the product of the RMS-normed stream with w. gated: w = [wg; wu] stacked and
+    out = silu(scaled gate) * scaled up. m <= 32, bf16."""
+    _need_gpu(xg, w, out, stats)
+    k = w.shape[1]
+    n = w.shape[0] // 2 if gated else w.shape[0]
+    assert xg.dtype == w.dtype == out.dtype == torch.bfloat16 and stats.dtype == torch.float32
+    assert xg.shape[1] == k and out.shape[1] == n and min(xg.shape[0], out.shape[0], stats.shape[0]) >= m
+    assert 0 < cols <= stats.shape[1]
+    lib.call("dinfer_gemm_small_m_scaled", xg.data_ptr(), _rows(xg), w.data_ptr(), _rows(w), out.data_ptr(), _rows(out),
+             m, n, k, 1 if gated else 0, stats.data_ptr(), _rows(stats), cols, float(eps), width, _stream())
+    return out
+
+
 def gemm_mid_m_workspace(m: int, n: int, k: int, *, gated: bool = False, ks: int = 0, rt: int = 0) -> int:
     """Bytes of float workspace gemm_mid_m needs for these sizes (0: the product is stored directly)."""
     need = ctypes.c_int64(0)

@@ -624,6 +624,55 @@ def test_gemm_small_m_gated(M):
             assert bool((err <= 1e-2 * want.abs() + 1e-3 * want.std()).all()), f"M={M} N={N} K={K}: {float(err.max())}"
 
 
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 32])
+def test_gemm_small_m_carries_the_norm(M):
+    """A product that adds into the residual stream and leaves what the next RMSNorm needs (the stream times the gain,
+    sums of squares per 16 columns), and the product that takes those: together they equal add, norm and product, to
+    rounding, at widths that are no multiples of the tiles, with the gain in either dtype and an offset."""
+    eps = 1e-5
+    for N, K, N2 in ((96, 512, 136), (328, 80, 1000), (4096, 4096, 6144), (1000, 1096, 50)):
+        for gain_dtype, offset in ((torch.float32, 0.0), (torch.bfloat16, 1.0)):
+            a = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+            w = (torch.randn(N, K, device=DEV) * 0.05).to(torch.bfloat16)
+            h0 = torch.randn(M + 1, N, device=DEV).to(torch.bfloat16)
+            gain = (torch.randn(N, device=DEV) * 0.1 + (1.0 - offset)).to(gain_dtype)
+            h = h0.clone()
+            xg = torch.full((M + 1, N), 7.0, device=DEV, dtype=torch.bfloat16)
+            cols = -(-N // 16)
+            stats = torch.full((M + 1, cols + 3), 7.0, device=DEV)
+            ops().gemm_small_m_sink(a, w, h, xg, gain, stats, M, gain_offset=offset)
+            want_h = (h0[:M].double() + a.double() @ w.double().T)
+            err = (h[:M].double() - want_h).abs()
+            assert bool((err <= 2 ** -8 * want_h.abs() + 1e-6).all()), f"stream M={M} N={N} K={K}: {float(err.max())}"   # one rounding
+            assert torch.equal(h[M:], h0[M:]) and bool((xg[M:] == 7.0).all()) and bool((stats[M:] == 7.0).all())
+            assert bool((stats[:M, cols:] == 7.0).all())
+            hs = h[:M].double()                                       # from here on the stream as it was stored
+            pad = torch.zeros(M, cols * 16 - N, device=DEV, dtype=torch.float64)
+            want_stats = torch.cat([hs, pad], dim=1).reshape(M, cols, 16).pow(2).sum(-1)
+            torch.testing.assert_close(stats[:M, :cols].double(), want_stats, rtol=1e-5, atol=1e-6)
+            want_xg = hs * (gain.double() + offset)
+            assert bool(((xg[:M].double() - want_xg).abs() <= 2 ** -8 * want_xg.abs() + 1e-6).all())
+            if N % 8:
+                continue                                              # the consumer reads 16 bytes at a time
+            normed = hs / (hs.pow(2).mean(-1, keepdim=True) + eps).sqrt() * (gain.double() + offset)
+            rstd = (stats[:M, :cols].double().sum(-1, keepdim=True) / N + eps).rsqrt()
+            for gated in (False, True):
+                w2 = (torch.randn((2 if gated else 1) * N2, N, device=DEV) * 0.05).to(torch.bfloat16)
+                out = torch.full((M + 1, N2), 7.0, device=DEV, dtype=torch.bfloat16)
+                ops().gemm_small_m_scaled(xg, w2, out, M, stats, cols, eps, N, gated=gated)
+                assert bool((out[M:] == 7.0).all())
+                # the kernel itself, on the operands as they are stored: only the result is rounded
+                z = (xg[:M].double() @ w2.double().T) * rstd
+                want = plain.silu(z[:, :N2]) * z[:, N2:] if gated else z
+                err = (out[:M].double() - want).abs()
+                assert bool((err <= 1e-2 * want.abs() + 1e-3 * want.std()).all()), f"M={M} N={N} N2={N2} gated={gated}: {float(err.max())}"
+                if not gated:
+                    # and the pair against norm, then product: the operand is rounded once more, as a norm's output is
+                    want = normed @ w2.double().T
+                    err = (out[:M].double() - want).abs()
+                    assert bool((err <= 2e-2 * want.abs() + 2e-2 * want.abs().mean()).all()), f"M={M} N={N} N2={N2}: {float(err.max())}"
+
+
 @pytest.mark.parametrize("M", [1, 17, 32, 33, 48, 64])
 def test_gemm_mid_m(M):
     """The product that keeps a slice of the activations in LDS, plain and gated, against float64: sizes that are no
