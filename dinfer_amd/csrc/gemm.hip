@@ -146,6 +146,26 @@ __global__ void __launch_bounds__(1024) gemm_small_m_kernel(const bf16* __restri
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[r][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  // SINK: what the epilogue adds to and multiplies by is fetched now, where the latency hides behind the first
+  // weights (for the first slot a thread sums; a workgroup with fewer threads than slots fetches the rest when it
+  // gets there)
+  float res0[4] = {0.f, 0.f, 0.f, 0.f}, gain0[4] = {0.f, 0.f, 0.f, 0.f};
+  if constexpr (MODE == SINK) {
+    const int x = threadIdx.x;
+    if (x < RT * MT * 64) {
+      const int tile = x >> 6, ln = x & 63;
+      const int m = (tile % MT) * 16 + (ln & 15), n = n0 + (tile / MT) * 16 + 4 * (ln >> 4);
+      if (m < M) {
+        const bf16* hp = (const bf16*)C + (int64_t)m * ldc + n;
+        for (int e = 0; e < 4 && n + e < N; ++e) {
+          res0[e] = (float)hp[e];
+          gain0[e] = (link.gain_f32 ? ((const float*)link.gain)[n + e] : (float)((const bf16*)link.gain)[n + e]) +
+                     link.gain_offset;
+        }
+      }
+    }
+  }
+
   // k steps of 64; wave w takes a contiguous run of them, so its loads walk each row in long pieces
   const int steps = (K + 63) / 64;
   const int per_wave = (steps + nw - 1) / nw;
@@ -248,14 +268,26 @@ __global__ void __launch_bounds__(1024) gemm_small_m_kernel(const bf16* __restri
       if (m < M) {
         bf16* hp = (bf16*)C + (int64_t)m * ldc + n;
         bf16* xp = link.xg + (int64_t)m * link.ld_xg + n;
-        for (int e = 0; e < 4 && n + e < N; ++e) {
-          const bf16 h = (bf16)((float)hp[e] + s[e]);
-          const float hf = (float)h;
-          hp[e] = h;
+        const bool first = x == (int)threadIdx.x;
+        bf16x4 hv, xv;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float res = res0[e], g = gain0[e];
+          if (!first && n + e < N) {
+            res = (float)hp[e];
+            g = (link.gain_f32 ? ((const float*)link.gain)[n + e] : (float)((const bf16*)link.gain)[n + e]) + link.gain_offset;
+          }
+          const bf16 h = (bf16)(res + s[e]);
+          const float hf = n + e < N ? (float)h : 0.f;
+          hv[e] = h;
           ss += hf * hf;
-          const float g = (link.gain_f32 ? ((const float*)link.gain)[n + e] : (float)((const bf16*)link.gain)[n + e]) +
-                          link.gain_offset;
-          xp[e] = (bf16)(hf * g);
+          xv[e] = (bf16)(hf * g);
+        }
+        if (n + 3 < N && ((ldc | link.ld_xg) & 3) == 0 && (((uintptr_t)C | (uintptr_t)link.xg) & 7) == 0) {
+          *(bf16x4*)hp = hv;  // four columns as one 8-byte store
+          *(bf16x4*)xp = xv;
+        } else {
+          for (int e = 0; e < 4 && n + e < N; ++e) hp[e] = hv[e], xp[e] = xv[e];
         }
       }
       // the tile's 16 columns of a token lie in the four lanes ln, ln + 16, + 32, + 48

@@ -105,3 +105,29 @@ def gated_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, scratch: torch
     matmul_nt(a, w, scratch, m, may_pad=True)
     ops.gated_act(scratch, out, m, act)
     return out
+
+
+CARRY_M = 32   # the products that carry a norm take up to this many rows (the block arrangement asks for fewer)
+
+
+def sink_nt(a: torch.Tensor, w: torch.Tensor, stream: torch.Tensor, xg: torch.Tensor, gain: torch.Tensor, offset: float,
+            stats: torch.Tensor, m: int) -> bool:
+    """stream[:m] += a[:m] @ w.T in place, leaving xg = stream * (gain + offset) and per-row partial sums of squares in
+    stats for the RMSNorm that reads the stream next. False (nothing done) where no kernel does this for the sizes."""
+    n, k = w.shape
+    if not (a.is_cuda and a.dtype == torch.bfloat16 and 0 < m <= CARRY_M and k % 8 == 0 and not _tall(m, n, k)):
+        return False
+    ops.gemm_small_m_sink(a, w, stream, xg, gain, stats, m, gain_offset=offset)
+    return True
+
+
+def scaled_nt(xg: torch.Tensor, stats: torch.Tensor, cols: int, eps: float, width: int, w: torch.Tensor, out: torch.Tensor,
+              m: int, gated: bool = False) -> bool:
+    """out[:m] = (xg[:m] @ w.T) * rsqrt(sum(stats[r, :cols]) / width + eps), the product of the normed stream; gated: w is
+    [gate; up] and out = silu(gate part) * up part. False (nothing done) where no kernel does this for the sizes."""
+    n, k = (w.shape[0] // 2 if gated else w.shape[0]), w.shape[1]
+    if not (xg.is_cuda and xg.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and 0 < m <= CARRY_M and k % 8 == 0
+            and (gated or not _tall(m, n, k))):
+        return False
+    ops.gemm_small_m_scaled(xg, w, out, m, stats, cols, eps, width, gated=gated)
+    return True

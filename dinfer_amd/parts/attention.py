@@ -19,6 +19,8 @@ from .spec import KVSpec, PartSpec, TensorSpec
 
 @MIXERS.register("attention")
 class Attention(Mixer):
+    carries_norms = True   # the q/k/v product takes a Carried, the output product an Into
+
     def __init__(self, hidden: int, heads: int, kv_heads: int, head_dim: int, position: PartSpec,
                  qk_norm: PartSpec | None = None, window: int | None = None, scale: float | None = None):
         if heads % kv_heads:
@@ -69,7 +71,7 @@ class Attention(Mixer):
         self.out_buf = ws.buffer("mixer_out", self.hidden)
         self.attn_ws = attn_kernels.Workspace(ctx, self.heads, self.kv_heads, self.head_dim)
 
-    def forward(self, x, batch, cache: CacheView):
+    def forward(self, x, batch, cache: CacheView, into=None):
         T = batch.num_tokens
         g = cache.group
         self.qkv.forward(x, self.qkv_buf, T, scratch=True)
@@ -87,4 +89,8 @@ class Attention(Mixer):
             self.qkv_buf, self.attn_buf, cache.k, cache.v, batch, g, self.attn_ws, scale=self.scale,
             window=self.window or 0, heads=self.heads, kv_heads=self.kv_heads, head_dim=self.head_dim,
             page_size=self.page_size)
+        if into is not None:
+            done = self.o.forward_into(self.attn_buf, into, T)
+            if done is not None:
+                return done
         return self.o.forward(self.attn_buf, self.out_buf, T, scratch=True)

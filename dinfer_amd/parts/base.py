@@ -71,6 +71,37 @@ class Norm(Part):
         """out[r] = norm(x[src r]); with residual: residual = x + residual first, normed after."""
         raise NotImplementedError
 
+    def carried(self):
+        """(gain, offset, eps) if the norm is y = x / sqrt(mean(x^2) + eps) * (gain + offset), which the products
+        around it can carry (see Carried); None for any other norm."""
+        return None
+
+
+class Carried:
+    """A norm that is still to be applied to the residual stream, carried by the products around it: the product
+    that completed the stream has left `xg` (the stream times the norm's gain) and `stats` (per row, `cols` partial
+    sums of the squares of the stream); a product that takes xg as its operand and multiplies its result rows by
+    rsqrt(sum(stats) / width + eps) has applied the norm. A consumer that cannot do that calls `materialise()`,
+    which runs the norm's own kernel on the (complete) stream."""
+    __slots__ = ("xg", "stats", "cols", "eps", "width", "norm", "stream", "buf", "rows")
+
+    def __init__(self, xg, stats, cols, eps, width, norm, stream, buf, rows):
+        self.xg, self.stats, self.cols, self.eps, self.width = xg, stats, cols, eps, width
+        self.norm, self.stream, self.buf, self.rows = norm, stream, buf, rows
+
+    def materialise(self) -> torch.Tensor:
+        return self.norm.forward(self.stream, self.buf, self.rows)
+
+
+class Into:
+    """Where a part's last product may put its result instead of into a buffer of its own: added to `stream`
+    in place, leaving a Carried for `norm`, the norm that reads the stream next (xg, stats, buf: the buffers for it).
+    A part that cannot (sizes, dtype, a last operation that is no product) ignores it and returns its buffer."""
+    __slots__ = ("stream", "norm", "xg", "stats", "buf")
+
+    def __init__(self, stream, norm, xg, stats, buf):
+        self.stream, self.norm, self.xg, self.stats, self.buf = stream, norm, xg, stats, buf
+
 
 class PositionEncoding(Part):
     """Gives the rotation table the mixer's kernel applies to q and k."""
@@ -95,6 +126,10 @@ class CacheView:
 
 
 class Mixer(Part):
+    # True: forward also takes a Carried as x and the keyword `into` (an Into or None), and may return a Carried
+    # when it has added its result to the stream itself. Parts that leave it False are given plain tensors.
+    carries_norms = False
+
     def cache_spec(self) -> KVSpec | StateSpec | None:
         return None
 
@@ -104,6 +139,8 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    carries_norms = False   # as for Mixer
+
     def forward(self, x: torch.Tensor, batch) -> torch.Tensor:
         raise NotImplementedError
 
@@ -114,7 +151,16 @@ class Block(Part):
     forward(hidden, pending, batch, cache) -> pending': `hidden` is the residual
     stream, updated in place; `pending` is a branch output not yet added to it
     (None at the first layer). Deferring the add lets the next norm kernel do it.
+
+    A block whose `input_norm()` is not None may be handed a Carried for that norm as `pending` (the
+    stream is complete then); a block with `carries_norms` is told the next block's input norm as
+    `next_norm` so that it can return one. Other blocks see neither.
     """
+    carries_norms = False
+
+    def input_norm(self):
+        """The norm this block applies to the stream first, if the block before may carry it; else None."""
+        return None
 
     def forward(self, hidden, pending, batch, cache: CacheView):
         raise NotImplementedError

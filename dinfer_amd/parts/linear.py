@@ -4,6 +4,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import gemm
+from .base import Carried, Into
 
 
 class Linear:
@@ -16,6 +17,23 @@ class Linear:
             raise ValueError(f"linear weight is {tuple(w.shape)}, expected {(self.out_features, self.in_features)}")
         self.weight = w.contiguous()
 
-    def forward(self, x: torch.Tensor, out: torch.Tensor, m: int, scratch: bool = False) -> torch.Tensor:
-        """scratch: x and out are activation buffers with spare rows beyond m that nothing reads."""
+    def forward(self, x, out: torch.Tensor, m: int, scratch: bool = False) -> torch.Tensor:
+        """scratch: x and out are activation buffers with spare rows beyond m that nothing reads. x may be a
+        Carried: the norm it stands for is applied inside the product where a kernel does that."""
+        if isinstance(x, Carried):
+            if gemm.scaled_nt(x.xg, x.stats, x.cols, x.eps, x.width, self.weight, out, m):
+                return out
+            x = x.materialise()
         return gemm.matmul_nt(x, self.weight, out, m, may_pad=scratch)
+
+    def forward_into(self, x: torch.Tensor, into: Into, m: int) -> Carried | None:
+        """into.stream[:m] += x[:m] @ W^T, returning the Carried for into.norm; None (nothing done) where that norm
+        cannot be carried or no kernel does this for the sizes."""
+        params = into.norm.carried() if into is not None and into.norm is not None else None
+        if params is None or isinstance(x, Carried):
+            return None
+        gain, offset, eps = params
+        if gain is None or not gemm.sink_nt(x, self.weight, into.stream, into.xg, gain, offset, into.stats, m):
+            return None
+        width = self.out_features
+        return Carried(into.xg, into.stats, -(-width // 16), eps, width, into.norm, into.stream, into.buf, m)

@@ -5,7 +5,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import gemm
-from .base import FeedForward
+from .base import Carried, FeedForward
 from .linear import Linear
 from .registry import FEED_FORWARDS
 from .spec import TensorSpec
@@ -13,6 +13,8 @@ from .spec import TensorSpec
 
 @FEED_FORWARDS.register("gated_mlp")
 class GatedMLP(FeedForward):
+    carries_norms = True   # the gate/up product takes a Carried, the down product an Into
+
     def __init__(self, hidden: int, intermediate: int, act: str = "silu"):
         self.hidden, self.intermediate, self.act = hidden, intermediate, act
         self.gate_up = Linear(hidden, 2 * intermediate)
@@ -36,8 +38,17 @@ class GatedMLP(FeedForward):
         self.act_buf = ws.buffer("act", self.intermediate)
         self.out_buf = ws.buffer("ffn_out", self.hidden)
 
-    def forward(self, x, batch):
+    def forward(self, x, batch, into=None):
         T = batch.num_tokens
-        # decode-sized steps: both projections and the activation in one weight-streaming kernel
-        gemm.gated_nt(x, self.gate_up.weight, self.act_buf, self.gu_buf, T, self.act)
+        w = self.gate_up.weight
+        if isinstance(x, Carried):
+            if not (self.act == "silu" and gemm.scaled_nt(x.xg, x.stats, x.cols, x.eps, x.width, w, self.act_buf, T, gated=True)):
+                x = x.materialise()
+        if not isinstance(x, Carried):
+            # decode-sized steps: both projections and the activation in one weight-streaming kernel
+            gemm.gated_nt(x, w, self.act_buf, self.gu_buf, T, self.act)
+        if into is not None:
+            done = self.down.forward_into(self.act_buf, into, T)
+            if done is not None:
+                return done
         return self.down.forward(self.act_buf, self.out_buf, T, scratch=True)

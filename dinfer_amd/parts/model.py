@@ -6,7 +6,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import gemm, ops
-from .base import BuildContext
+from .base import BuildContext, Carried
 from .linear import Linear
 from .registry import BLOCKS, NORMS
 from .spec import ModelSpec, RunEntry, TensorSpec
@@ -115,10 +115,16 @@ class DecoderModel:
         ops.embedding(batch.input_ids[:T], self.embed, self.hidden)
         pending = None
         for i, e in enumerate(self.run):
-            pending = self.blocks[e.layer].forward(self.hidden, pending, batch, caches[i])
+            # the input norm of the block that runs next, if that block lets the one before carry it
+            block = self.blocks[e.layer]
+            if block.carries_norms and i + 1 < len(self.run):
+                nxt = self.blocks[self.run[i + 1].layer].input_norm()
+                pending = block.forward(self.hidden, pending, batch, caches[i], next_norm=nxt)
+            else:
+                pending = block.forward(self.hidden, pending, batch, caches[i])
         if R == 0:
             return self.logits[:0]
-        if pending is None:
+        if pending is None or isinstance(pending, Carried):
             self.final_norm.forward(self.hidden, self.final_normed, R, rows=batch.logits_rows)
         else:
             # the last add happens on the wanted rows only, inside the norm kernel

@@ -20,6 +20,9 @@ class RMSNorm(Norm):
     def load(self, get):
         self.weight = get("weight")
 
+    def carried(self):
+        return (self.weight, self.weight_offset, self.eps)
+
     def forward(self, x, out, n_rows, *, residual=None, rows=None):
         return ops.rmsnorm(x, self.weight, out, self.eps, n_rows, residual=residual, rows=rows,
                            weight_offset=self.weight_offset)

@@ -643,7 +643,8 @@ def test_gemm_small_m_carries_the_norm(M):
             ops().gemm_small_m_sink(a, w, h, xg, gain, stats, M, gain_offset=offset)
             want_h = (h0[:M].double() + a.double() @ w.double().T)
             err = (h[:M].double() - want_h).abs()
-            assert bool((err <= 2 ** -8 * want_h.abs() + 1e-6).all()), f"stream M={M} N={N} K={K}: {float(err.max())}"   # one rounding
+            # one rounding of a float sum of K products
+            assert bool((err <= 2 ** -8 * want_h.abs() + 1e-5 * want_h.abs().mean()).all()), f"stream M={M} N={N} K={K}: {float(err.max())}"
             assert torch.equal(h[M:], h0[M:]) and bool((xg[M:] == 7.0).all()) and bool((stats[M:] == 7.0).all())
             assert bool((stats[:M, cols:] == 7.0).all())
             hs = h[:M].double()                                       # from here on the stream as it was stored
