@@ -36,6 +36,8 @@
 // paged: 64-key tiles, base-2 online softmax, P rounded to bf16 before P.V),
 // gqa_decode_v3_core.cuh:72-242 and gqa.cu:1423-1461 (split-K decode, merge of
 // (m, l, o) partials).
+#include <cmath>
+
 #include "common.cuh"
 
 using namespace dinfer;
@@ -449,15 +451,21 @@ __device__ __forceinline__ void split_range(int seq, int window, int splits, int
 }
 
 // One wave per (split, kv head, request). part: [B, H, splits, D + 4] float = (m in base-2 units, l, -, -, o[D]).
-template <int DT, bool P2, bool STREAM>
-__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 8))) attn_decode_kernel(
+// JOIN (up to JOIN_SPLITS parts: many requests): the parts of a (kv head, request) are the waves of one workgroup,
+// meet in LDS and are combined there as attn_decode_merge_kernel combines them, so that kernel does not run.
+constexpr int JOIN_SPLITS = 4;
+
+template <int DT, bool P2, bool STREAM, bool JOIN = false>
+// (JOIN runs where requests are many and parts few: a CU holds 4 to 8 of its waves, registers are no limit there)
+__global__ void __launch_bounds__(JOIN ? 64 * JOIN_SPLITS : 64) __attribute__((amdgpu_waves_per_eu(JOIN ? 2 : 4, 8)))
+attn_decode_kernel(
     const bf16* __restrict__ q, int64_t ld_q, float* __restrict__ part, const bf16* __restrict__ kc,
     const bf16* __restrict__ vc, const int32_t* __restrict__ block_table, int64_t max_blocks,
     const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_lens, int splits, float scale_log2e,
-    int window, int H, int Hkv, int ps) {
+    int window, int H, int Hkv, int ps, bf16* __restrict__ out = nullptr, int64_t ld_out = 0) {
   constexpr int D = DT * 16;
   constexpr int KS = (DT + 1) / 2;
-  const int sp = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
+  const int sp = JOIN ? (int)(threadIdx.x >> 6) : (int)blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
   const int G = H / Hkv;
   int row = b;  // without cu_seqlens every request has exactly one row
   if (cu_seqlens) {
@@ -466,7 +474,9 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 8)))
   }
   int k_lo, k_hi, kps;
   split_range(seq_lens[b], window, splits, sp, &k_lo, &k_hi, &kps);
-  if (k_lo >= k_hi) return;  // an empty part writes nothing; the merge kernel skips it by the same rule
+  // an empty part writes nothing; the merge kernel skips it by the same rule. (JOIN: it walks no block and
+  // leaves m = -inf, which weighs nothing; its wave must reach the barrier below.)
+  if (!JOIN && k_lo >= k_hi) return;
   const int lane = threadIdx.x & 63, i16 = lane & 15, g4 = lane >> 4;
   const int32_t* bt = block_table + (int64_t)b * max_blocks;
 
@@ -485,7 +495,36 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 8)))
   tl.init(kc, vc, bt, (int)max_blocks, hk, Hkv, ps, k_lo, k_hi, scale_log2e);
   tl.template walk<false>(qf, col_lo, col_hi, [&](int kb) { return kb < k_lo || kb + 32 > k_hi; });
   const float lt = tl.sum_l(0);
-  if (i16 < G) {
+  if constexpr (JOIN) {
+    __shared__ __attribute__((aligned(16))) float joined[JOIN_SPLITS][16][D + 4];
+    if (i16 < G) {
+      float* pp = &joined[sp][i16][0];
+      if (g4 == 0) {
+        pp[0] = tl.m[0] * scale_log2e;  // -inf for an empty part
+        pp[1] = lt;
+      }
+#pragma unroll
+      for (int d = 0; d < DT; ++d) *(f32x4*)(pp + 4 + d * 16 + 4 * g4) = tl.o[0][d];
+    }
+    __syncthreads();
+    // out[head, d] = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s, parts in ascending order
+    for (int idx = threadIdx.x; idx < G * D; idx += blockDim.x) {
+      const int i = idx / D, d = idx - i * D;
+      float M = -INFINITY;
+      for (int s = 0; s < splits; ++s) M = fmaxf(M, joined[s][i][0]);
+      float L = 0.f, acc = 0.f;
+      for (int s = 0; s < splits; ++s) {
+        const float m = joined[s][i][0];
+        const float a = m == -INFINITY ? 0.f : exp2f(m - M);
+        if (a > 0.f) {
+          L += a * joined[s][i][1];
+          acc += a * joined[s][i][4 + d];
+        }
+      }
+      const float inv = L > 0.f ? 1.f / L : 0.f;
+      out[(int64_t)row * ld_out + (int64_t)(hk * G + i) * D + d] = (bf16)(acc * inv);
+    }
+  } else if (i16 < G) {
     float* pp = part + (((int64_t)b * H + hk * G + i16) * splits + sp) * (D + 4);
     if (g4 == 0) {
       pp[0] = tl.m[0] * scale_log2e;  // the tile keeps raw maxima; partials carry base-2 units
@@ -573,6 +612,18 @@ int launch_flash(const bf16* q, int64_t ld_q, bf16* out, int64_t ld_out, const b
   return launch_status();
 }
 
+// CUs of the current device (asked once per device).
+inline int compute_units() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (!cached[dev]) {
+    int n = 0;
+    cached[dev] = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0 ? n : 256;
+  }
+  return cached[dev];
+}
+
 template <int DT>
 int launch_decode(const bf16* q, int64_t ld_q, bf16* out, int64_t ld_out, float* part, const bf16* kc, const bf16* vc,
                   const int32_t* bt, int64_t max_blocks, const int32_t* cu, const int32_t* sl, int num_reqs,
@@ -580,10 +631,23 @@ int launch_decode(const bf16* q, int64_t ld_q, bf16* out, int64_t ld_out, float*
   // many requests: the keys of a step exceed the caches and each is used once, so they are read past
   // them (measured at 64 requests of 2k-4k keys: 10% faster; at 8 or fewer, slightly slower)
   const bool p2 = (ps & (ps - 1)) == 0, stream_kv = num_reqs >= 32;
+  if constexpr (DT <= 8) {  // (the parts of head size 256 do not fit the LDS of a workgroup)
+    // Workgroups of `splits` waves are placed whole: where their number leaves the last round over the CUs thin
+    // (320 workgroups on 256 CUs: some CUs get two, most one) single waves spread better and the merge kernel is the
+    // lesser cost. Measured at 8 kv heads: 32, 56 and 64 requests gain 0.12 to 0.17 ms a step, 40 and 48 lose.
+    const double per_cu = (double)Hkv * num_reqs / compute_units();
+    if (splits <= JOIN_SPLITS && (per_cu <= 1. || ceil(per_cu) <= 1.15 * per_cu)) {
+      auto kernel = p2 ? (stream_kv ? attn_decode_kernel<DT, true, true, true> : attn_decode_kernel<DT, true, false, true>)
+                       : (stream_kv ? attn_decode_kernel<DT, false, true, true> : attn_decode_kernel<DT, false, false, true>);
+      kernel<<<dim3(1, (unsigned)Hkv, (unsigned)num_reqs), 64 * splits, 0, stream>>>(
+          q, ld_q, part, kc, vc, bt, max_blocks, cu, sl, splits, scale * LOG2E, window, H, Hkv, ps, out, ld_out);
+      return launch_status();
+    }
+  }
   auto kernel = p2 ? (stream_kv ? attn_decode_kernel<DT, true, true> : attn_decode_kernel<DT, true, false>)
                    : (stream_kv ? attn_decode_kernel<DT, false, true> : attn_decode_kernel<DT, false, false>);
   kernel<<<dim3((unsigned)splits, (unsigned)Hkv, (unsigned)num_reqs), 64, 0, stream>>>(
-      q, ld_q, part, kc, vc, bt, max_blocks, cu, sl, splits, scale * LOG2E, window, H, Hkv, ps);
+      q, ld_q, part, kc, vc, bt, max_blocks, cu, sl, splits, scale * LOG2E, window, H, Hkv, ps, (bf16*)nullptr, (int64_t)0);
   const int D = DT * 16;
   attn_decode_merge_kernel<<<dim3((unsigned)H, (unsigned)num_reqs), 64, 0, stream>>>(part, out, ld_out, cu, sl, splits,
                                                                                      window, H, D);

@@ -238,7 +238,9 @@ def test_attention_flash(H, Hkv, D, page, window):
 def test_attention_decode_split_k(H, Hkv, D, page, window):
     # 300 / 70 / 1: several splits, a short one, a single key; then 1..64 at batch 32
     for hist, splits in (([299, 69, 0, 1000], 7), ([random.Random(7).randrange(64) for _ in range(32)], 2),
-                         ([5000, 31, 32], 64), ([100, 200], 1)):
+                         ([5000, 31, 32], 64), ([100, 200], 1),
+                         # up to four parts meet inside the workgroup (no merge kernel): with empty parts, a single key
+                         ([0, 45, 1000, 130], 4), ([70, 2, 500, 33, 64], 3)):
         new = [1] * len(hist)
         q, kc, vc, m, outs = paged_case(torch.bfloat16, H, Hkv, D, page, hist, new, seed=5)
         out = torch.zeros(len(hist), H * D, device=DEV, dtype=torch.bfloat16)
@@ -263,12 +265,12 @@ def test_attention_flash_long_portions(H, Hkv, D, page, window):
     torch.testing.assert_close(out.double().cpu().view(-1, H, D), want, rtol=2e-2, atol=2e-2)
 
 
-def test_attention_mixed_routes_single_rows_to_split_k():
+@pytest.mark.parametrize("splits", [5, 3])   # parts merged by a kernel of their own, and inside the workgroup
+def test_attention_mixed_routes_single_rows_to_split_k(splits):
     H, Hkv, D, page = 16, 4, 128, 16
     hist, new = [500, 0, 64, 900, 33, 10], [1, 40, 1, 1, 20, 1]
     q, kc, vc, m, outs = paged_case(torch.bfloat16, H, Hkv, D, page, hist, new, seed=9)
     out = torch.zeros(sum(new), H * D, device=DEV, dtype=torch.bfloat16)
-    splits = 5
     part = torch.zeros(len(hist) * H * splits * (D + 4), device=DEV)
     geo = dict(scale=D ** -0.5, window=0, heads=H, kv_heads=Hkv, head_dim=D, page_size=page)
     ops().attn_decode(q, out, part, kc, vc, m["bt"], m["cu"], m["sl"], len(hist), splits, **geo)
