@@ -142,8 +142,8 @@ def test_block_part(dtype):
         b = whole_batch([n], page=page)
         kc = torch.zeros(ops.k_cache_shape(64, Hkv, page, D), device=DEV, dtype=dtype)
         vc = torch.zeros(64, Hkv, D, page, device=DEV, dtype=dtype)
-        h0 = torch.randn(64, Hd, device=DEV).to(dtype)
-        prev = torch.randn(64, Hd, device=DEV).to(dtype)       # the previous layer's branch, not yet added
+        h0 = torch.randn(64, Hd, generator=g).to(DEV).to(dtype)
+        prev = torch.randn(64, Hd, generator=g).to(DEV).to(dtype)       # the previous layer's branch, not yet added
         hidden = h0.clone()
         pending = blk.forward(hidden, prev, b, CacheView(0, kc, vc, owner=True))
         got = (hidden[:n].double() + pending[:n].double()).cpu()
@@ -186,19 +186,22 @@ def test_block_carries_its_norms_into_the_next_block():
     b = whole_batch([n], page=page)
     caches = [CacheView(0, torch.zeros(ops.k_cache_shape(64, Hkv, page, D), device=DEV, dtype=dtype),
                         torch.zeros(64, Hkv, D, page, device=DEV, dtype=dtype), owner=True) for _ in blocks]
-    h0 = torch.randn(64, Hd, device=DEV).to(dtype)
+    h0 = torch.randn(64, Hd, generator=g).to(DEV).to(dtype)
     hidden = h0.clone()
     carried = blocks[0].forward(hidden, None, b, caches[0], next_norm=blocks[1].input_norm())
     assert isinstance(carried, Carried) and carried.norm is blocks[1].norm_in
     want1 = plain.decoder_layer(h0[:n].double().cpu(), list(range(n)), wd, 0, cfg)
-    err = (hidden[:n].double().cpu() - want1).abs()          # the stream is complete: nothing is pending
-    assert float(err.pow(2).mean().sqrt() / want1.std()) < 0.008
+    # the stream is complete: nothing is pending. (Root mean square of the error over the output's spread, over 40
+    # seeds: 0.006 at the median and 0.009 at worst after one layer, 0.008 and 0.013 after two, with the norms carried
+    # and with norm kernels alike; the largest error after two layers 0.03 and 0.07.)
+    err = (hidden[:n].double().cpu() - want1).abs()
+    assert float(err.pow(2).mean().sqrt() / want1.std()) < 0.011
     pending = blocks[1].forward(hidden, carried, b, caches[1])
     assert isinstance(pending, torch.Tensor)                 # nobody to carry the next norm: the branch comes back
     got = (hidden[:n].double() + pending[:n].double()).cpu()
     want2 = plain.decoder_layer(want1, list(range(n)), wd, 1, cfg)
     err = (got - want2).abs()
-    assert float(err.pow(2).mean().sqrt() / want2.std()) < 0.012 and float(err.max() / want2.std()) < 0.06
+    assert float(err.pow(2).mean().sqrt() / want2.std()) < 0.016 and float(err.max() / want2.std()) < 0.08
     # a consumer that cannot take a Carried gets the norm's own kernel on the stream as it stands
     normed = carried.materialise()[:n].double().cpu()
     hs = hidden[:n].double().cpu()
