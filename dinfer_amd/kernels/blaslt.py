@@ -122,9 +122,10 @@ class _Plan:
         self.tuned = False
 
 
-def _run(handle, plan, algo, a, w, out, workspace) -> None:
+def _run(handle, plan, algo, a, w, out, workspace, beta=_zero) -> None:
+    """out = a . w^T + beta * out (the library reads and writes the same matrix)."""
     stream = torch.cuda.current_stream(a.device).cuda_stream
-    _ok(_lib.hipblasLtMatmul(handle, plan.desc, byref(_one), w.data_ptr(), plan.lw, a.data_ptr(), plan.la, byref(_zero),
+    _ok(_lib.hipblasLtMatmul(handle, plan.desc, byref(_one), w.data_ptr(), plan.lw, a.data_ptr(), plan.la, byref(beta),
                              out.data_ptr(), plan.lc, out.data_ptr(), plan.lc, byref(algo), workspace.data_ptr(),
                              WORKSPACE_BYTES, stream), "matmul")
 
@@ -139,21 +140,23 @@ def flush_caches(dev) -> None:
     flush.sum()
 
 
-def _tune(handle, plan, a, w, out, workspace) -> None:
+def _tune(handle, plan, a, w, out, workspace, beta=_zero) -> None:
     """Times every candidate on the call's own operands and keeps the fastest. In a model the weight of a
     product comes from HBM (the layers before have pushed it out of every cache), so each timed run follows a
     read of FLUSH_BYTES of other memory that empties the memory-side cache; timed on a weight that stays cached, kernels win
-    that lose in place."""
+    that lose in place. A product that adds to its output is timed on a copy of it."""
+    if beta is not _zero:
+        out = out.clone()
     best, best_t, best_i, times = plan.candidates[0], float("inf"), 0, []
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     for i, algo in enumerate(plan.candidates):
         try:
-            _run(handle, plan, algo, a, w, out, workspace)   # first use of a kernel loads it
+            _run(handle, plan, algo, a, w, out, workspace, beta)   # first use of a kernel loads it
             t = float("inf")
             for _ in range(3):   # the least of three: a single timing wanders by a few per cent, as much as the candidates differ
                 flush_caches(a.device)
                 start.record()
-                _run(handle, plan, algo, a, w, out, workspace)
+                _run(handle, plan, algo, a, w, out, workspace, beta)
                 end.record()
                 end.synchronize()
                 t = min(t, start.elapsed_time(end))
@@ -168,8 +171,10 @@ def _tune(handle, plan, a, w, out, workspace) -> None:
               file=sys.stderr, flush=True)
 
 
-def matmul(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int) -> torch.Tensor:
-    """out[:m] = a[:m] @ w.T; a, w bfloat16 with contiguous rows, out bfloat16 or float32."""
+def matmul(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, accumulate: bool = False) -> torch.Tensor:
+    """out[:m] = a[:m] @ w.T; a, w bfloat16 with contiguous rows, out bfloat16 or float32. accumulate: out[:m] +=
+    instead, the sum of the float accumulators and out rounded once."""
+    beta = _one if accumulate else _zero
     dev = a.device
     handle = _handles.get(dev)
     if handle is None:
@@ -179,7 +184,7 @@ def matmul(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int) -> torch
             _workspaces[dev] = torch.empty(WORKSPACE_BYTES, dtype=torch.uint8, device=dev)
         _handles[dev] = handle
     n, k = w.shape
-    key = (dev, m, n, k, a.stride(0), w.stride(0), out.stride(0), out.dtype)
+    key = (dev, m, n, k, a.stride(0), w.stride(0), out.stride(0), out.dtype, accumulate)
     plan = _plans.get(key)
     if plan is None:
         try:
@@ -188,7 +193,9 @@ def matmul(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int) -> torch
             plan = False   # a shape the direct interface does not take: torch's own call of the library serves it
         _plans[key] = plan
     if plan is False:
-        if out.dtype == a.dtype:
+        if accumulate:
+            out[:m].addmm_(a[:m].to(out.dtype), w.t().to(out.dtype))
+        elif out.dtype == a.dtype:
             torch.mm(a[:m], w.t(), out=out[:m])
         else:
             out[:m].copy_(torch.mm(a[:m], w.t()))
@@ -196,6 +203,6 @@ def matmul(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int) -> torch
     workspace = _workspaces[dev]
     if (not plan.tuned and m >= TUNE_FROM_ROWS and m * n * k >= TUNE_FROM_WORK and len(plan.candidates) > 1
             and os.environ.get("DINFER_GEMM_TUNE", "1") != "0" and not torch.cuda.is_current_stream_capturing()):
-        _tune(handle, plan, a, w, out, workspace)
-    _run(handle, plan, plan.algo, a, w, out, workspace)
+        _tune(handle, plan, a, w, out, workspace, beta)
+    _run(handle, plan, plan.algo, a, w, out, workspace, beta)
     return out

@@ -121,6 +121,19 @@ def sink_nt(a: torch.Tensor, w: torch.Tensor, stream: torch.Tensor, xg: torch.Te
     return True
 
 
+def add_nt(a: torch.Tensor, w: torch.Tensor, stream: torch.Tensor, m: int) -> bool:
+    """stream[:m] += a[:m] @ w.T in place through the library (its `beta = 1`): the sum of the float accumulators and the
+    stream, rounded once. For the steps of many rows, where sink_nt has no kernel; a and stream are activation buffers
+    (rows beyond m hold nothing of value). False (nothing done) where the library does not run the product."""
+    n, k = w.shape
+    if not (a.is_cuda and a.dtype == torch.bfloat16 and stream.dtype == torch.bfloat16 and m > SMALL_M
+            and not _tall(m, n, k) and blaslt.available() and a.stride(1) == 1 and w.stride(1) == 1 and stream.stride(1) == 1):
+        return False
+    rows = min(a.shape[0], stream.shape[0], -(-m // ROW_BUCKET) * ROW_BUCKET)
+    blaslt.matmul(a, w, stream, rows, accumulate=True)
+    return True
+
+
 def scaled_nt(xg: torch.Tensor, stats: torch.Tensor, cols: int, eps: float, width: int, w: torch.Tensor, out: torch.Tensor,
               m: int, gated: bool = False) -> bool:
     """out[:m] = (xg[:m] @ w.T) * rsqrt(sum(stats[r, :cols]) / width + eps), the product of the normed stream; gated: w is

@@ -82,12 +82,17 @@ class Carried:
     that completed the stream has left `xg` (the stream times the norm's gain) and `stats` (per row, `cols` partial
     sums of the squares of the stream); a product that takes xg as its operand and multiplies its result rows by
     rsqrt(sum(stats) / width + eps) has applied the norm. A consumer that cannot do that calls `materialise()`,
-    which runs the norm's own kernel on the (complete) stream."""
+    which runs the norm's own kernel on the (complete) stream. Without xg (`scaled` False) the product has only
+    added into the stream (steps of many rows), and `materialise()` is the one way on."""
     __slots__ = ("xg", "stats", "cols", "eps", "width", "norm", "stream", "buf", "rows")
 
     def __init__(self, xg, stats, cols, eps, width, norm, stream, buf, rows):
         self.xg, self.stats, self.cols, self.eps, self.width = xg, stats, cols, eps, width
         self.norm, self.stream, self.buf, self.rows = norm, stream, buf, rows
+
+    @property
+    def scaled(self) -> bool:
+        return self.xg is not None
 
     def materialise(self) -> torch.Tensor:
         return self.norm.forward(self.stream, self.buf, self.rows)

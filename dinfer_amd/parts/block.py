@@ -6,6 +6,8 @@ next block's input norm kernel, and the mixer's add into this block's second
 norm kernel, so each add costs no pass of its own (model.rs:700-701,722-731,772-781).
 In steps of a few tokens the norms have no kernel at all: the product before a norm adds
 into the stream and leaves what the norm needs, the product after it applies it (Carried).
+In steps of many tokens the product before a norm adds into the stream as well (the library's
+beta = 1), and the norm's kernel reads the stream alone.
 """
 from __future__ import annotations
 
@@ -62,7 +64,7 @@ class PreNormBlock(Block):
         return self.norm_in if self.mixer.carries_norms else None
 
     def _into(self, hidden, norm, part, T):
-        if norm is None or not part.carries_norms or T > CARRY_ROWS or norm.carried() is None:
+        if norm is None or not part.carries_norms:
             return {}
         return {"into": Into(hidden, norm, self.xg, self.stats, self.normed)}
 

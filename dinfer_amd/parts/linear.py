@@ -21,19 +21,23 @@ class Linear:
         """scratch: x and out are activation buffers with spare rows beyond m that nothing reads. x may be a
         Carried: the norm it stands for is applied inside the product where a kernel does that."""
         if isinstance(x, Carried):
-            if gemm.scaled_nt(x.xg, x.stats, x.cols, x.eps, x.width, self.weight, out, m):
+            if x.scaled and gemm.scaled_nt(x.xg, x.stats, x.cols, x.eps, x.width, self.weight, out, m):
                 return out
             x = x.materialise()
         return gemm.matmul_nt(x, self.weight, out, m, may_pad=scratch)
 
     def forward_into(self, x: torch.Tensor, into: Into, m: int) -> Carried | None:
-        """into.stream[:m] += x[:m] @ W^T, returning the Carried for into.norm; None (nothing done) where that norm
-        cannot be carried or no kernel does this for the sizes."""
-        params = into.norm.carried() if into is not None and into.norm is not None else None
-        if params is None or isinstance(x, Carried):
-            return None
-        gain, offset, eps = params
-        if gain is None or not gemm.sink_nt(x, self.weight, into.stream, into.xg, gain, offset, into.stats, m):
+        """into.stream[:m] += x[:m] @ W^T, returning the Carried for into.norm; None (nothing done) where no kernel
+        does this for the sizes. In steps of few rows the norm rides along (where it can be carried); in steps of many
+        the product only adds, and the norm's kernel reads one matrix instead of two and writes one instead of two."""
+        if into is None or into.norm is None or isinstance(x, Carried):
             return None
         width = self.out_features
-        return Carried(into.xg, into.stats, -(-width // 16), eps, width, into.norm, into.stream, into.buf, m)
+        params = into.norm.carried()
+        if params is not None and params[0] is not None and m <= into.xg.shape[0]:
+            gain, offset, eps = params
+            if gemm.sink_nt(x, self.weight, into.stream, into.xg, gain, offset, into.stats, m):
+                return Carried(into.xg, into.stats, -(-width // 16), eps, width, into.norm, into.stream, into.buf, m)
+        if gemm.add_nt(x, self.weight, into.stream, m):
+            return Carried(None, None, 0, 0.0, width, into.norm, into.stream, into.buf, m)
+        return None

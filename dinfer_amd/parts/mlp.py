@@ -42,7 +42,7 @@ class GatedMLP(FeedForward):
         T = batch.num_tokens
         w = self.gate_up.weight
         if isinstance(x, Carried):
-            if not (self.act == "silu" and gemm.scaled_nt(x.xg, x.stats, x.cols, x.eps, x.width, w, self.act_buf, T, gated=True)):
+            if not (x.scaled and self.act == "silu" and gemm.scaled_nt(x.xg, x.stats, x.cols, x.eps, x.width, w, self.act_buf, T, gated=True)):
                 x = x.materialise()
         if not isinstance(x, Carried):
             # decode-sized steps: both projections and the activation in one weight-streaming kernel

@@ -610,6 +610,33 @@ def test_library_gemm_with_measured_algorithm():
     torch.testing.assert_close(out.double(), a.double() @ w.double().T, rtol=1e-4, atol=1e-4)
 
 
+def test_library_gemm_adds_into_its_output():
+    """stream += a . w^T through the library: the first call of a shape times the candidates on a copy (the stream
+    itself gets the product once), later calls add once each; rows past the bucket are untouched; the few-row and
+    tall shapes are refused (other kernels serve them)."""
+    from dinfer_amd.kernels import blaslt, gemm
+    assert blaslt.available()
+    for M, N, K in ((520, 1000, 1096), (130, 200, 264), (40, 33, 8), (257, 4096, 512)):
+        a = torch.randn(M + 70, K, device=DEV).to(torch.bfloat16)
+        w = (torch.randn(N, K, device=DEV) * 0.05).to(torch.bfloat16)
+        start = torch.randn(M + 70, N, device=DEV).to(torch.bfloat16)
+        prod = a[:M].double() @ w.double().T
+        stream = start.clone()
+        last = -(-M // gemm.ROW_BUCKET) * gemm.ROW_BUCKET
+        for call in (1, 2):
+            before = stream[:M].double()
+            assert gemm.add_nt(a, w, stream, M)
+            want = before + prod
+            # one rounding of (float sum of products + stream) per call
+            err = (stream[:M].double() - want).abs()
+            assert bool((err <= 2.0 ** -8 * want.abs() + 1e-3 * prod.abs().mean()).all()), f"{M}x{N}x{K} call {call}: {err.max()}"
+            assert torch.equal(stream[last:], start[last:]), f"{M}x{N}x{K}: rows past {last} were written"
+    assert any(p and p.tuned for key, p in blaslt._plans.items() if key[-1])   # an adding product was measured too
+    a = torch.randn(32, 64, device=DEV).to(torch.bfloat16)
+    assert not gemm.add_nt(a, torch.zeros(48, 64, device=DEV, dtype=torch.bfloat16), torch.zeros(32, 48, device=DEV, dtype=torch.bfloat16), 32)
+    assert not gemm.add_nt(a.float(), torch.zeros(48, 64, device=DEV), torch.zeros(32, 48, device=DEV), 32)
+
+
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 32])
 def test_gemm_small_m_gated(M):
     """Both projections of a gated feed-forward and silu(gate) * up in one kernel, against float64."""
