@@ -538,6 +538,10 @@ attn_decode_kernel(
 constexpr int MAX_SPLITS = 256;
 
 // out[b, h, :] = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s over the non-empty parts. One wave per (head, request).
+// The kernel is a chain of memory round trips and little else, so everything whose address is known at the start
+// is asked for at the start: the length, every part's (m, l), and the outputs of the first MERGE_AHEAD parts; which
+// parts are empty (they hold anything) is settled afterwards. Head sizes up to 256, up to MAX_SPLITS parts.
+constexpr int MERGE_AHEAD = 8;
 __global__ void __launch_bounds__(64) attn_decode_merge_kernel(const float* __restrict__ part, bf16* __restrict__ out,
                                                                int64_t ld_out, const int32_t* __restrict__ cu_seqlens,
                                                                const int32_t* __restrict__ seq_lens, int splits,
@@ -549,32 +553,57 @@ __global__ void __launch_bounds__(64) attn_decode_merge_kernel(const float* __re
     row = cu_seqlens[b];
     if (cu_seqlens[b + 1] - row != 1) return;
   }
-  const int seq = seq_lens[b];
   const float* pp = part + ((int64_t)b * H + h) * splits * (D + 4);
+  f32x2 ml[MAX_SPLITS / 64];
+#pragma unroll
+  for (int j = 0; j < MAX_SPLITS / 64; ++j) {
+    const int s = lane + 64 * j < splits ? lane + 64 * j : splits - 1;  // clamped, not skipped: no branch around a load
+    ml[j] = *(const f32x2*)(pp + (int64_t)s * (D + 4));
+  }
+  float ahead[MERGE_AHEAD][4];
+#pragma unroll
+  for (int s = 0; s < MERGE_AHEAD; ++s)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int sc = s < splits ? s : splits - 1, d = lane + 64 * j < D ? lane + 64 * j : D - 1;
+      ahead[s][j] = pp[(int64_t)sc * (D + 4) + 4 + d];
+    }
+  const int seq = seq_lens[b];
   float mloc = -INFINITY;
-  for (int s = lane; s < splits; s += 64) {
+#pragma unroll
+  for (int j = 0; j < MAX_SPLITS / 64; ++j) {
+    const int s = lane + 64 * j;
     int k_lo, k_hi, kps;
     split_range(seq, window, splits, s, &k_lo, &k_hi, &kps);
-    const float m = k_lo < k_hi ? pp[(int64_t)s * (D + 4)] : -INFINITY;
-    wgt[s] = m;
+    const float m = s < splits && k_lo < k_hi ? ml[j][0] : -INFINITY;
+    ml[j][0] = m;
     mloc = fmaxf(mloc, m);
   }
   const float M = wave_max(mloc);
   float lloc = 0.f;
-  for (int s = lane; s < splits; s += 64) {
-    const float m = wgt[s];
+#pragma unroll
+  for (int j = 0; j < MAX_SPLITS / 64; ++j) {
+    const int s = lane + 64 * j;
+    const float m = ml[j][0];
     const float a = m == -INFINITY ? 0.f : exp2f(m - M);
-    wgt[s] = a;
-    const float lv = pp[(int64_t)s * (D + 4) + 1];  // read unconditionally (an empty part holds anything)
-    lloc += a > 0.f ? a * lv : 0.f;
+    if (s < splits) wgt[s] = a;
+    lloc += a > 0.f ? a * ml[j][1] : 0.f;
   }
   const float L = wave_sum(lloc);
   __syncthreads();
   const float inv = L > 0.f ? 1.f / L : 0.f;
-  for (int d = lane; d < D; d += 64) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int d = lane + 64 * j;
+    if (d >= D) break;
     float acc = 0.f;
+#pragma unroll
+    for (int s = 0; s < MERGE_AHEAD; ++s) {
+      const float a = s < splits ? wgt[s] : 0.f;
+      acc += a > 0.f ? a * ahead[s][j] : 0.f;
+    }
 #pragma unroll 8
-    for (int s = 0; s < splits; ++s) {
+    for (int s = MERGE_AHEAD; s < splits; ++s) {
       const float a = wgt[s];
       const float v = pp[(int64_t)s * (D + 4) + 4 + d];  // loads do not wait for the weights
       acc += a > 0.f ? a * v : 0.f;
