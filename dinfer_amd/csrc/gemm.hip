@@ -383,13 +383,33 @@ int launch_gated_scaled(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, 
   return launch_status();
 }
 
+// Row tiles a workgroup (16 weight rows each) for up to 16 tokens. Measured inside whole decode steps on MI355X (256
+// CUs): with one row tile there is one workgroup per 16 columns, and from 257 to 511 of them the CUs are loaded
+// unevenly (320 workgroups: a quarter of the CUs get two); half as many workgroups of twice the work finish no later
+// and each wave keeps more loads in flight. N = 5,120: 14B-sized steps 6.93 -> 6.60 ms at 8 tokens, 6.35 -> 5.91 at one;
+// N = 6,144 (K = 4,096): 3.93 -> 3.88 ms. At N = 4,096 (256 workgroups, one a CU) two row tiles lose (4.00 ms). From
+// N = 8,192 on, two row tiles when there are more than a few tokens (measured on the kernel alone).
+inline int few_rows_row_tiles(int64_t M, int64_t N) {
+  if (N > 4096 && N < 8192) return 2;
+  return N >= 8192 && M > 4 ? 2 : 1;
+}
+
+// Waves of a workgroup (they share K): 8, or 4 with two row tiles of a wide weight; 16 for a small square weight with
+// one workgroup a CU, where 8 waves a CU keep too few loads in flight (N = K = 4,096: 3.93 -> 3.90 ms a step; with
+// K = 12,288 or N = 5,120 sixteen lose). Every wave gets at least four k steps (K = 1,024: 4 waves, measured).
+inline int few_rows_waves(int mt, int rt, int64_t N, int64_t K) {
+  int nw = (rt == 1 || N < 8192) ? 8 : 4;
+  if (mt == 1 && rt == 1 && N <= 4096 && K <= 4096) nw = 16;
+  const int64_t steps = (K + 63) / 64;
+  while (nw > 1 && steps < 4 * nw) nw /= 2;
+  return nw;
+}
+
 // Row tiles and waves of a launch, as dinfer_gemm_small_m chooses them (at most two row tiles here).
 inline void shape_for(int64_t M, int64_t N, int64_t K, int* rt_out, int* nw_out) {
   const int mt = (int)(M + 15) / 16;
-  int rt = mt >= 2 ? ((N >= 6144 || streams_weight(N, K)) ? 2 : 1) : ((N >= 8192 && M > 4) ? 2 : 1);
-  int nw = (rt == 1 || N < 8192) ? 8 : 4;
-  const int64_t steps = (K + 63) / 64;
-  while (nw > 1 && steps < 4 * nw) nw /= 2;
+  int rt = mt >= 2 ? ((N >= 6144 || streams_weight(N, K)) ? 2 : 1) : few_rows_row_tiles(M, N);
+  int nw = few_rows_waves(mt, rt, N, K);
   while (nw > 1 && lds_bytes(nw, rt, mt) + RS_BYTES > 64 * 1024) nw /= 2;
   *rt_out = rt, *nw_out = nw;
 }
@@ -420,13 +440,8 @@ extern "C" int dinfer_gemm_small_m(int out_f32, const void* A, int64_t lda, cons
   // (32 tokens: N = K = 4096 9.1 us with one row tile, 11.2 with two; N = K = 5120 24.0 with one, 18.3 with
   // two); four row tiles for a vocabulary-sized N at 17 to 32 tokens
   if (rt == 0)
-    rt = mt >= 2 ? ((mt == 2 && N >= 65536) ? 4 : ((N >= 6144 || streams_weight(N, K)) ? 2 : 1))
-                 : ((N >= 8192 && M > 4) ? 2 : 1);
-  if (nw == 0) {
-    nw = (rt == 1 || N < 8192) ? 8 : 4;
-    const int64_t steps = (K + 63) / 64;
-    while (nw > 1 && steps < 4 * nw) nw /= 2;  // every wave at least four k steps (K = 1024: 4 waves, measured)
-  }
+    rt = mt >= 2 ? ((mt == 2 && N >= 65536) ? 4 : ((N >= 6144 || streams_weight(N, K)) ? 2 : 1)) : few_rows_row_tiles(M, N);
+  if (nw == 0) nw = few_rows_waves(mt, rt, N, K);
   while (nw > 1 && lds_bytes(nw, rt, mt) > 64 * 1024) nw /= 2;
   if (nw < 1 || nw > 16) return ERR_BAD_SHAPE;
   if (lds_bytes(nw, rt, mt) > 64 * 1024) return ERR_UNSUPPORTED;
