@@ -36,6 +36,8 @@ SOURCES = {
     "host": "host/api.cpp",
 }
 HEADERS = ["common.cuh"]
+# headers of single libraries (their C interface), hashed with them
+OWN_HEADERS = {"gemm_mid": ["gemm_mid.h"]}
 # libraries without device code, and the headers each is made of
 HOST_ONLY = {"host": ["host/dinfer_host.h", "host/errors.hpp", "host/block_pool.hpp", "host/cache_manager.hpp",
                       "host/step_batch.hpp", "host/scheduler.hpp"]}
@@ -97,7 +99,7 @@ def lib_dir() -> Path:
 
 def source_hash(name: str) -> str:
     h = hashlib.sha256()
-    for f in HOST_ONLY.get(name, HEADERS) + [SOURCES[name]]:
+    for f in HOST_ONLY.get(name, HEADERS) + OWN_HEADERS.get(name, []) + [SOURCES[name]]:
         h.update((CSRC / f).read_bytes())
     h.update(" ".join(HOST_FLAGS if name in HOST_ONLY else FLAGS).encode())
     return h.hexdigest()[:16]
@@ -107,11 +109,12 @@ def lib_path(name: str) -> Path:
     return lib_dir() / f"libdinfer_{name}.so"
 
 
-def find_built(name: str) -> Path | None:
-    """A library built earlier, in the package or in the per-user folder; None if absent."""
+def find_built(name: str, fresh_only: bool = True) -> Path | None:
+    """A library built earlier from today's sources, in the package or in the per-user folder; None if there
+    is none (fresh_only False: also one built from other sources)."""
     for d in (PACKAGE / "_lib", Path(tempfile.gettempdir()) / f"dinfer_amd_lib_{os.getuid()}"):
         p = d / f"libdinfer_{name}.so"
-        if p.exists():
+        if p.exists() and not (fresh_only and is_stale(name, p)):
             return p
     return None
 
@@ -170,7 +173,7 @@ def build_all(force: bool = True, jobs: int = 4, verbose: bool = True) -> dict[s
 
     def one(n):
         p = find_built(n)
-        if not force and p is not None and not is_stale(n, p):
+        if not force and p is not None:
             return n, p
         return n, build(n, verbose=verbose)
 

@@ -6,7 +6,6 @@ no GPU is present when a kernel is called, the call raises.
 from __future__ import annotations
 
 import ctypes
-import sys
 import threading
 from ctypes import c_float, c_int, c_int64, c_uint32, c_void_p
 
@@ -49,6 +48,8 @@ SIGNATURES = {
     "dinfer_gemm_small_m_sink": ("gemm", [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _F, _P, _L, _L, _L, _L, _P]),
     "dinfer_gemm_mid_m": ("gemm_mid", [_I, _P, _L, _P, _L, _P, _L, _L, _L, _L, _I, _I, _I, _P, _L, _P]),
     "dinfer_gemm_mid_m_workspace": ("gemm_mid", [_L, _L, _L, _I, _I, _I, _P]),
+    "dinfer_gemm_mid_m_static": ("gemm_mid", [_I, _P, _L, _P, _L, _P, _L, _L, _L, _L, _I, _I, _I, _P]),
+    "dinfer_gemm_mid_m_static_init": ("gemm_mid", []),
     "dinfer_argmax": ("sampling", [_P, _L, _P, _L, _L, _P]),
     "dinfer_sample": ("sampling", [_P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _P]),
     "dinfer_sample_rows": ("sampling", [_P, _L, _P, _P, _L, _P, _P, _L, _L, _I, _I, _P]),
@@ -64,6 +65,7 @@ ERRORS = {
     3: "size or option not supported by this kernel",
     4: "kernel launch failed",
     5: "workspace too small",
+    6: "sizes beyond what the library's built-in scratch array holds",
 }
 
 _libs: dict[str, ctypes.CDLL] = {}
@@ -80,12 +82,15 @@ def load_library(name: str) -> ctypes.CDLL:
         lib = _libs.get(name)
         if lib is not None:
             return lib
+        # only a library whose recorded hash equals the hash of today's sources is loaded: the argument lists
+        # above belong to those sources, and a kernel launched through another list reads past its operands
         path = _build.find_built(name)
         if path is None:
-            path = _build.build(name)
-        elif _build.is_stale(name, path):
-            print(f"[dinfer_amd] warning: {path.name} is older than its source; rebuild with "
-                  f"`python -m dinfer_amd.csrc.build`", file=sys.stderr, flush=True)
+            try:
+                path = _build.build(name)
+            except (RuntimeError, OSError) as e:
+                raise KernelError(f"libdinfer_{name}.so is missing or older than its source and cannot be "
+                                  f"built here: {e}") from e
         try:
             lib = ctypes.CDLL(str(path))
         except OSError as e:
