@@ -32,6 +32,7 @@ enum : int {
   ERR_UNSUPPORTED = 3,
   ERR_LAUNCH = 4,
   ERR_WORKSPACE = 5,
+  ERR_SCRATCH_LIMIT = 6,
 };
 
 __device__ __forceinline__ float to_f32(float v) { return v; }

@@ -27,6 +27,9 @@
 // Reference behaviour: crates/kernels/src/gemm.rs:605-647 (the product itself; the reference hands
 // these row counts to its vendor library).
 #include "common.cuh"
+#include "gemm_mid.h"
+
+#include <mutex>
 
 using namespace dinfer;
 
@@ -323,12 +326,11 @@ extern "C" int dinfer_gemm_mid_m_workspace(int64_t M, int64_t N, int64_t K, int 
   return OK;
 }
 
-// C[M,N] = A . W^T for up to 64 rows. gated: W is [2N, K] = [gate; up] and C[M,N] = silu(A . gate^T) * (A . up^T).
-// ks: k per slice (a multiple of 64; 0: as long as LDS holds), rt: tiles of 16 weight rows per wave (1, 2, 4; 0:
-// chosen from the sizes). Partial sums go through `workspace` (dinfer_gemm_mid_m_workspace bytes, 16-byte aligned).
-extern "C" int dinfer_gemm_mid_m(int out_f32, const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc,
-                                 int64_t M, int64_t N, int64_t K, int gated, int ks, int rt, void* workspace,
-                                 int64_t workspace_bytes, hipStream_t stream) {
+namespace {
+
+// The product and the pass that adds up its slices, with the partial sums in `P` (at least `capacity` bytes).
+int run_mid_m(int out_f32, const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, int64_t M, int64_t N,
+              int64_t K, int gated, int ks, int rt, void* P_, int64_t capacity, int too_small, hipStream_t stream) {
   if (M <= 0 || N <= 0) return OK;
   if (M > 64) return ERR_UNSUPPORTED;
   const int64_t rows = gated ? 2 * N : N;
@@ -339,8 +341,8 @@ extern "C" int dinfer_gemm_mid_m(int out_f32, const void* A, int64_t lda, const 
   if (!choose(M, rows, K, ks, rt, &s)) return ERR_UNSUPPORTED;
   const int mt = (int)(M + 15) / 16;
   const int64_t need = (int64_t)s.slices * rows * (mt * 16) * (int64_t)sizeof(float);
-  if (!workspace || workspace_bytes < need || ((uintptr_t)workspace % 16)) return ERR_WORKSPACE;
-  float* P = (float*)workspace;
+  if (!P_ || capacity < need || ((uintptr_t)P_ % 16)) return too_small;
+  float* P = (float*)P_;
   int st;
 #define GO(MT_) st = launch_rt<MT_>((const bf16*)A, lda, (const bf16*)W, ldw, P, (int)M, (int)rows, (int)K, s, stream)
   if (mt == 1) GO(1);
@@ -357,4 +359,68 @@ extern "C" int dinfer_gemm_mid_m(int out_f32, const void* A, int64_t lda, const 
   else
     gemm_mid_reduce_kernel<bf16, false><<<blocks, 256, 0, stream>>>(P, mt * 16, s.slices, (bf16*)C, ldc, (int)M, (int)N);
   return launch_status();
+}
+
+}  // namespace
+
+// C[M,N] = A . W^T for up to 64 rows. gated: W is [2N, K] = [gate; up] and C[M,N] = silu(A . gate^T) * (A . up^T).
+// ks: k per slice (a multiple of 64; 0: as long as LDS holds), rt: tiles of 16 weight rows per wave (1, 2, 4; 0:
+// chosen from the sizes). Partial sums go through `workspace` (dinfer_gemm_mid_m_workspace bytes, 16-byte aligned).
+extern "C" int dinfer_gemm_mid_m(int out_f32, const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc,
+                                 int64_t M, int64_t N, int64_t K, int gated, int ks, int rt, void* workspace,
+                                 int64_t workspace_bytes, hipStream_t stream) {
+  return run_mid_m(out_f32, A, lda, W, ldw, C, ldc, M, N, K, gated, ks, rt, workspace, workspace_bytes, ERR_WORKSPACE, stream);
+}
+
+// ---- the same product for callers that cannot allocate ---------------------------------------------------------
+// The partial sums go through a device array that is part of this library's code object: every GPU the library
+// runs on holds its own copy, at its own address, from the moment the code object is loaded there until the
+// process ends. In host code the array's name stands for that symbol, it is no device address: the address on
+// the current device comes from hipGetSymbolAddress, once per device, and only that pointer is ever handed to
+// a kernel.
+static __device__ __align__(256) unsigned char scratch[DINFER_GEMM_MID_STATIC_BYTES];
+
+namespace {
+
+constexpr int MAX_DEVICES = 64;
+void* scratch_ptr[MAX_DEVICES];   // by device ordinal; nullptr until that device has been set up
+std::mutex scratch_mutex;
+
+// The address of `scratch` on the current device (asked for once per device and kept).
+int scratch_on_current_device(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return ERR_LAUNCH;
+  std::lock_guard<std::mutex> guard(scratch_mutex);
+  if (!scratch_ptr[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) {
+      (void)hipGetLastError();
+      return ERR_LAUNCH;
+    }
+    scratch_ptr[dev] = p;
+  }
+  *out = scratch_ptr[dev];
+  return OK;
+}
+
+}  // namespace
+
+extern "C" int dinfer_gemm_mid_m_static_init(void) {
+  void* p;
+  return scratch_on_current_device(&p);
+}
+
+extern "C" int64_t dinfer_gemm_mid_m_static_capacity(void) { return DINFER_GEMM_MID_STATIC_BYTES; }
+
+extern "C" int dinfer_gemm_mid_m_static(int out_f32, const void* A, int64_t lda, const void* W, int64_t ldw, void* C,
+                                        int64_t ldc, int64_t M, int64_t N, int64_t K, int gated, int ks, int rt,
+                                        hipStream_t stream) {
+  if (M <= 0 || N <= 0) return OK;
+  void* p = nullptr;
+  const int st = scratch_on_current_device(&p);
+  if (st != OK) return st;
+  // Nothing of the array has to start at zero: every slice writes all of its partial sums (all rows of every
+  // token tile, all columns) before the second kernel, later on the same stream, reads them.
+  return run_mid_m(out_f32, A, lda, W, ldw, C, ldc, M, N, K, gated, ks, rt, p, DINFER_GEMM_MID_STATIC_BYTES,
+                   ERR_SCRATCH_LIMIT, stream);
 }
