@@ -28,11 +28,11 @@ from pathlib import Path
 
 sys.path.insert(0, str(Path(__file__).resolve().parent))
 
-# Qwen3-8B layer sizes (BASELINE.json configs[2])
+# Qwen3-8B layer sizes: the default run
 SIZES = dict(vocab_size=151936, hidden_size=4096, intermediate_size=12288, num_hidden_layers=36,
              num_attention_heads=32, num_key_value_heads=8, head_dim=128, rms_norm_eps=1e-6, rope_theta=1e6,
              max_position_embeddings=40960, tie_word_embeddings=False)
-# further sizes of the same architecture (BASELINE.json configs[3] and [4]); `--shape` picks one
+# further sizes of the same architecture (Qwen3-14B and 32B); `--shape` picks one
 SHAPES = {
     "8b": {},
     "14b": dict(hidden_size=5120, intermediate_size=17408, num_hidden_layers=40, num_attention_heads=40),
@@ -121,7 +121,7 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=DEFAULT_CONTEXT, help="max_model_len the engine is built for")
     ap.add_argument("--workload", default="decode", choices=["decode", "serving"],
                     help="serving: 32 requests with prompts of 512 to 3,072 tokens fed in portions of 512 beside the "
-                         "requests that decode, 256 outputs each (BASELINE.json names it for the 14B shape); its own JSON line")
+                         "requests that decode, 256 outputs each (meant for the 14B shape); its own JSON line")
     ap.add_argument("--runs", type=int, default=2,
                     help="serving: the workload runs this many times on one engine and the last run is reported")
     ap.add_argument("--sampled", action="store_true",

@@ -2,9 +2,9 @@
 
 ``allocate(n)`` is all-or-nothing and takes pages from the head of the free
 list; ``free(ids)`` puts the pages back at the head in the order given, so pages
-that were just given back are the next ones handed out (crates/core/src/kv/block_pool.rs:128-147,160-182;
-this engine has no prefix cache, so there is no LRU tail).
-A page is held by at most one owner; freeing a page that is not held raises.
+that were just given back are the next ones handed out (crates/core/src/kv/block_pool.rs:128-147,160-182).
+This bare pool names no pages; inside the cache manager the same C++ class also keeps named pages of the prefix
+cache at the tail of its list. A page is held by at most one owner; freeing a page that is not held raises.
 """
 from __future__ import annotations
 

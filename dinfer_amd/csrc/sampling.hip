@@ -111,12 +111,6 @@ __device__ float row_expsum_ge(const float* row, int vocab, float m, float t, fl
   return block_sum(s, red);
 }
 
-__device__ int row_count_ge(const float* row, int vocab, float t, float* red) {
-  float c = 0.f;
-  for (int i = threadIdx.x; i < vocab; i += BLOCK) c += row[i] >= t ? 1.f : 0.f;
-  return (int)block_sum(c, red);
-}
-
 __device__ void row_min_p(float* row, int vocab, float mp, float* red) {
   if (mp <= 0.f) return;
   const float m = row_max(row, vocab, red);
@@ -129,44 +123,76 @@ __device__ void row_min_p(float* row, int vocab, float mp, float* red) {
   __syncthreads();
 }
 
-// Keeps the k largest, then of those the smallest set of most probable tokens whose
-// mass reaches p. Both thresholds are found by bisection on the value axis.
-__device__ void row_topk_topp(float* row, int vocab, int k, float p, float* red) {
-  const bool do_k = k > 0 && k < vocab;
-  const bool do_p = p < 1.f && p > 0.f;
-  if (!do_k && !do_p) return;
-  const float m = row_max(row, vocab, red);
-  float lo_local = INFINITY;
+// Floats as unsigned keys of the same order (a larger float has a larger key; -0 counts as +0, -inf is the lowest
+// key a row holds): thresholds can then be found digit by digit, exactly, instead of by halving an interval.
+__device__ __forceinline__ uint32_t order_key(float v) {
+  const uint32_t u = __float_as_uint(v + 0.f);
+  return (u >> 31) ? ~u : (u | 0x80000000u);
+}
+
+// The key of the k-th largest entry of the row (1 <= k <= vocab): a radix selection, eight bits a pass. Each pass
+// counts, among the entries that share the digits fixed so far, how many hold each value of the next digit
+// (integer counters in LDS: the counts do not depend on the order of arrival), then walks the 256 counters from
+// the top until the k-th entry is reached.
+__device__ uint32_t row_kth_key(const float* row, int vocab, int k) {
+  __shared__ int digit_count[256];
+  __shared__ uint32_t chosen[2];   // the digit found, and how many entries are still to be skipped inside it
+  uint32_t prefix = 0;
+  int skip = k;                    // the entry looked for is the skip-th largest among those that match the prefix
+  for (int shift = 24; shift >= 0; shift -= 8) {
+    __syncthreads();
+    if (threadIdx.x < 256) digit_count[threadIdx.x] = 0;
+    __syncthreads();
+    const uint32_t fixed = shift == 24 ? 0u : 0xffffffffu << (shift + 8);
+    for (int i = threadIdx.x; i < vocab; i += BLOCK) {
+      const uint32_t key = order_key(row[i]);
+      if ((key & fixed) == prefix) atomicAdd(&digit_count[(key >> shift) & 255u], 1);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      int d = 255, left = skip;
+      while (d > 0 && digit_count[d] < left) left -= digit_count[d--];
+      chosen[0] = (uint32_t)d;
+      chosen[1] = (uint32_t)left;
+    }
+    __syncthreads();
+    prefix |= chosen[0] << shift;
+    skip = (int)chosen[1];
+  }
+  return prefix;
+}
+
+// Sum of exp(v - m) over the entries whose key is at least `least`.
+__device__ float row_mass_from_key(const float* row, int vocab, float m, uint32_t least, float* red) {
+  float s = 0.f;
   for (int i = threadIdx.x; i < vocab; i += BLOCK) {
     const float v = row[i];
-    if (v > -INFINITY) lo_local = fminf(lo_local, v);
+    if (order_key(v) >= least && v > -INFINITY) s += expf(v - m);
   }
-  const float lo = -block_max(-lo_local, red);
-  float floor_ = -INFINITY;
-  if (do_k) {
-    float a = lo, b = m;  // invariant: count(v >= a) >= k
-    for (int it = 0; it < 48 && b > a; ++it) {
-      const float mid = 0.5f * (a + b);
-      if (mid <= a || mid >= b) break;
-      if (row_count_ge(row, vocab, mid, red) >= k) a = mid; else b = mid;
+  return block_sum(s, red);
+}
+
+// top-k, then top-p on what it left: entries below the k-th largest value go, then entries below the largest value t
+// for which the entries from t up still hold the share p of the remaining mass (entries equal to a threshold stay).
+// The second threshold is built bit by bit from the top: a bit stays set if the mass from the key so formed up
+// still reaches the share.
+__device__ void row_topk_topp(float* row, int vocab, int k, float p, float* red) {
+  const bool cut_count = k > 0 && k < vocab, cut_mass = p > 0.f && p < 1.f;
+  if (!cut_count && !cut_mass) return;
+  uint32_t least = cut_count ? row_kth_key(row, vocab, k) : 0u;
+  if (cut_mass) {
+    const float m = row_max(row, vocab, red);
+    const float share = p * row_mass_from_key(row, vocab, m, least, red);
+    uint32_t t = 0;
+    for (int bit = 31; bit >= 0; --bit) {
+      const uint32_t with_bit = t | (1u << bit);
+      if (row_mass_from_key(row, vocab, m, with_bit > least ? with_bit : least, red) >= share) t = with_bit;
     }
-    floor_ = row_count_ge(row, vocab, b, red) >= k ? b : a;
-  }
-  float thresh = floor_;
-  if (do_p) {
-    const float denom = row_expsum_ge(row, vocab, m, floor_, red);
-    float a = fmaxf(lo, floor_), b = m;  // invariant: mass(v >= a) >= p
-    for (int it = 0; it < 48 && b > a; ++it) {
-      const float mid = 0.5f * (a + b);
-      if (mid <= a || mid >= b) break;
-      if (row_expsum_ge(row, vocab, m, fmaxf(mid, floor_), red) >= p * denom) a = mid; else b = mid;
-    }
-    if (row_expsum_ge(row, vocab, m, fmaxf(b, floor_), red) >= p * denom) a = b;
-    thresh = fmaxf(thresh, a);
+    if (t > least) least = t;
   }
   __syncthreads();
   for (int i = threadIdx.x; i < vocab; i += BLOCK)
-    if (row[i] < thresh) row[i] = -INFINITY;
+    if (order_key(row[i]) < least) row[i] = -INFINITY;
   __syncthreads();
 }
 

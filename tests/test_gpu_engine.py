@@ -1,5 +1,6 @@
-"""Generation through the Python entry point: greedy against the plain implementation, the workloads
-BASELINE names for the tiny configurations, sampling rules through the whole engine, preemption."""
+"""Generation through the Python entry point: greedy against the plain implementation on the small workloads
+(three prompts of 5/17/33 tokens decoded greedily; four of 1/9/40/70 prefilled in portions of 16 beside decoding
+requests and sampled at temperature 0.7), sampling rules through the whole engine, preemption."""
 import random
 
 import pytest
@@ -54,22 +55,29 @@ def test_greedy_generation_equals_plain(model_dirs, name, lens):
     eng.runner.cache.check()
 
 
-def test_bfloat16_generation_follows_plain_until_a_near_tie(model_dirs):
+def judge_greedy(cfg, w, prompt, tokens, slack=0.1):
+    """Every generated token against the plain model's logits after the tokens generated before it: it must be the
+    plain model's best, or lie within `slack` of the row's spread below it (bfloat16 logits are off by up to 0.05 of
+    the spread each, so two logits nearer than that may change places). Returns how many were the best."""
+    ids, best = list(prompt), 0
+    for i, tok in enumerate(tokens):
+        row = plain.forward(cfg, w, ids)[-1]
+        short = float((row.max() - row[tok]) / row.std())
+        assert short < slack, f"prompt of {len(prompt)}, output {i}: token {tok} lies {short:.3f} row-sigmas below the best"
+        best += short == 0.0
+        ids.append(tok)
+    return best
+
+
+def test_bfloat16_generation_follows_plain_up_to_near_ties(model_dirs):
     from dinfer_amd import SamplingParams
     name = "B"
     cfg, w = plain.load(model_dirs[name])
-    prompts = prompts_for(name, [9, 40], 8)
+    prompts = prompts_for(name, [9, 40, 70], 8)
     got = engine(model_dirs[name], name, dtype="bfloat16").generate(
-        prompts, SamplingParams(max_tokens=8, temperature=0.0, ignore_eos=True))
-    agree = 0
-    for p, g in zip(prompts, got):
-        want, margins = plain_greedy(cfg, w, p, 8)
-        for a, b, m in zip(g, want, margins):
-            if a != b:
-                assert m < 0.05, f"bf16 chose {a}, plain {b}, margin {m}"
-                break
-            agree += 1
-    assert agree >= 8
+        prompts, SamplingParams(max_tokens=12, temperature=0.0, ignore_eos=True))
+    best = sum(judge_greedy(cfg, w, p, g) for p, g in zip(prompts, got))
+    assert best >= 30, f"only {best} of 36 tokens are the plain model's first choice"
 
 
 def test_temperature_sampling_with_seed_in_mixed_batches(model_dirs):
@@ -214,9 +222,12 @@ def test_prefix_caching_changes_nothing_but_the_work(model_dirs, dtype):
     got += eng.generate(prompts, sp)        # all together: pages shared between live requests
     if dtype == "float32":
         assert got == want
-    else:  # bfloat16: a cached page was written by another kernel shape than the one that would write it now
-        same = sum(a == b for g, w_ in zip(got, want) for a, b in zip(g, w_))
-        assert same >= 0.8 * sum(len(g) for g in got), (got, want)
+    else:
+        # bfloat16: a cached page was written by another kernel shape than the one that would write it now, so two
+        # nearly equal logits may change places; every token is judged against the plain model instead
+        cfg, w = plain.load(model_dirs[name])
+        for p, g in zip(prompts + prompts, got):
+            judge_greedy(cfg, w, p, g)
     eng.runner.cache.check()
     assert eng.runner.cache.num_free(0) == 128
 
