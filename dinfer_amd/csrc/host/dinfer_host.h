@@ -77,7 +77,8 @@ int32_t dh_batch_fill(void* cache, const dh_batch_buffers* buf, int32_t n, const
 /* ---- scheduler */
 typedef struct {
     int32_t max_num_batched_tokens, max_num_seqs, max_model_len, prefill_tokens_per_step,
-        long_prefill_token_threshold, enable_chunked_prefill, decode_exempt_from_budget, enable_prefix_caching;
+        long_prefill_token_threshold, enable_chunked_prefill, decode_exempt_from_budget, enable_prefix_caching,
+        prefill_chunk_alignment;
 } dh_sched_options;
 
 typedef struct { int64_t id; int32_t start, num_new, samples; } dh_scheduled;

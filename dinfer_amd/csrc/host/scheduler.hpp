@@ -39,6 +39,7 @@ struct SchedOptions {
     int32_t enable_chunked_prefill;
     int32_t decode_exempt_from_budget;
     int32_t enable_prefix_caching;  // needs a cache manager built with a prefix cache
+    int32_t prefill_chunk_alignment;  // a portion that does not end its request's tokens ends at a multiple of this (<= 1: anywhere)
 };
 
 enum Status : int32_t { WAITING = 0, RUNNING = 1, PREEMPTED = 2, FINISHED = 3 };
@@ -125,6 +126,16 @@ public:
         if (it != reqs_.end() && it->second->status == FINISHED) reqs_.erase(it);
     }
 
+    // A portion that stops short of the request's last token is shortened so that it ends at a multiple of the
+    // alignment (layers that work in chunks of their own want portions to end where their chunks end, in the manner
+    // of crates/core/src/sched/mod.rs:146-166); 0 if not even one aligned position fits.
+    int64_t aligned(int64_t computed, int64_t n, int64_t remaining) const {
+        const int64_t a = opt_.prefill_chunk_alignment;
+        if (a <= 1 || n <= 0 || n >= remaining) return n;
+        const int64_t end = (computed + n) / a * a;
+        return end > computed ? end - computed : 0;
+    }
+
     // ---- one step
     const StepPlan& schedule() {
         plan_.scheduled.clear();
@@ -148,6 +159,7 @@ public:
             if (charged) n = std::min(n, budget);
             if (!is_decode) n = std::min(n, quota);
             if (n < remaining && !opt_.enable_chunked_prefill) n = 0;
+            n = aligned(r->num_computed, n, remaining);
             if (n <= 0) {
                 ++i;
                 continue;
@@ -194,6 +206,7 @@ public:
                 if (threshold && n > threshold) n = threshold;
                 n = std::min(n, std::min(budget, quota));
                 if (n < remaining && !opt_.enable_chunked_prefill) n = 0;
+                n = aligned(r->num_computed, n, remaining);
                 if (n <= 0 || !cache_->allocate(r->id, r->num_computed, n)) {
                     cache_->free(r->id);  // no budget or no pages now: wait (what was found stays cached)
                     if (opt_.enable_prefix_caching) r->num_computed = r->num_cached = 0;

@@ -14,7 +14,8 @@
 //
 // Padding (pad_to > B): a step of single rows that replays a captured graph of pad_to requests
 // is filled up with requests of one token at position 0 that write no cache slot (slot -1) and
-// read page 0, which always exists (crates/layers/src/exec.rs:388-426).
+// read page 0, which always exists (crates/layers/src/exec.rs:388-426). Their state slot is max_reqs,
+// one past the slots requests can hold: per-request state is allocated with that spare slot at its end.
 #pragma once
 #include <cstdint>
 #include <cstring>
@@ -116,7 +117,7 @@ inline void fill_batch(const CacheManager& cache, const BatchBuffers& buf, const
             buf.positions[b] = 0;
             buf.cu_seqlens[b + 1] = b + 1;
             buf.seq_lens[b] = 1;
-            buf.state_slots[b] = 0;
+            buf.state_slots[b] = buf.max_reqs;  // the spare slot: no request ever holds it
             buf.logits_rows[b] = b;
             for (int g = 0; g < buf.n_groups; ++g) {
                 int32_t* row = buf.block_table[g] + static_cast<int64_t>(b) * buf.max_blocks[g];

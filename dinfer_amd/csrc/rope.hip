@@ -6,7 +6,8 @@
 //   q, k:  y = x * rsqrt(mean(x^2) + eps) * (w + w_offset)   (skipped when the
 //          gain pointer is null), then rotation of the first `rot` dims by the
 //          angles of the token's position, all in float, one rounding.
-//          q is written back in place; k goes to the cache only.
+//          q is written back in place; k goes to the cache only, or, where no
+//          slot mapping is given (nothing is cached), back in place like q.
 //   v:     copied to the cache unchanged.
 //
 // Cache pages (chosen for MFMA operand loads on gfx950: both operands of
@@ -107,7 +108,7 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_kernel(
       y = first ? y * c - other * s : y * c + other * s;
     }
     const S r = from_f32<S>(y);
-    if (is_q) base[d] = r;
+    if (is_q || !slots) base[d] = r;  // without a slot mapping nothing goes to the cache and k is written back like q
     if (kd) kd[k_page_offset((int)off, d, page)] = r;
   }
 }
@@ -194,7 +195,7 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_neox_kernel(
       inv = 1.f / sqrtf(ss / (float)D + eps);
     }
     const int hk = item - H;
-    S* base = is_q ? row + q_off + (int64_t)item * D : nullptr;
+    S* base = is_q ? row + q_off + (int64_t)item * D : slots ? nullptr : row + k_off + (int64_t)hk * D;
     S* kd = (!is_q && slot >= 0) ? k_cache + (blk * Hkv + hk) * (int64_t)page * D : nullptr;  // the head's page
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
@@ -300,7 +301,7 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_vec_kernel(
   bf16x8 r;
 #pragma unroll
   for (int e = 0; e < 8; ++e) r[e] = (bf16)(first ? y[e] * c[e] - other[e] * sn[e] : y[e] * c[e] + other[e] * sn[e]);
-  if (is_q) {
+  if (is_q || !slots) {
     *(bf16x8*)(src + d0) = r;
   } else if (slot >= 0) {
     *(bf16x8*)(k_cache + (blk * Hkv + (item - H)) * (int64_t)page * D + k_page_offset((int)off, d0, page)) = r;

@@ -10,7 +10,7 @@ whole prompts, portions of prompts and single decoded tokens side by side
   cu_seqlens   [B+1] int32  prefix sums of the tokens per request
   seq_lens     [B]   int32  request length after this step (start + n)
   block_table  [B, MB] int32 per cache group, -1 where no page is held
-  state_slots  [B]   int32  the request's fixed-size state slot
+  state_slots  [B]   int32  the request's fixed-size state slot (padded rows: the spare slot max_reqs)
   logits_rows  [R]   int32  rows of the flat batch whose logits are wanted
 
 All of them live in one device allocation at fixed addresses and are filled by
@@ -82,7 +82,6 @@ class StepBatch:
         self.num_tokens = self.num_reqs = self.num_rows = 0
         self.max_q_len = self.max_seq_len = self.num_singles = 0
         self.all_decode = False
-        self.max_len_bound = 0
         self.req_ids: list = []
         self._copied = torch.cuda.Event() if pin else None
 
@@ -143,8 +142,6 @@ class StepBatch:
         self.num_tokens, self.num_reqs, self.num_rows = f.num_tokens, f.num_reqs, f.num_rows
         self.max_q_len, self.max_seq_len, self.num_singles = f.max_q_len, f.max_seq_len, f.num_singles
         self.all_decode = f.num_singles == f.num_reqs
-        # what kernels may assume about every seq_len of this step (a replayed graph fixes it to the model's limit)
-        self.max_len_bound = self.max_seq_len
 
     def upload(self) -> None:
         self._dev.copy_(self._host, non_blocking=True)

@@ -14,8 +14,8 @@ import torch
 
 from ..cache import CacheManager, GroupSpec
 from ..config import EngineOptions, load_config
-from ..kernels import ops
-from ..parts import BuildContext, CacheView, DecoderModel, KVSpec, StateSpec
+from ..kernels import blaslt, gemm, ops
+from ..parts import BuildContext, CacheView, DecoderModel
 from ..weights import WeightLoader
 from .batch import Entry, StepBatch
 
@@ -78,6 +78,7 @@ class ModelRunner:
         self.max_tokens = options.max_num_batched_tokens + (options.max_num_seqs if options.decode_exempt_from_budget else 0)
         self.ctx = BuildContext(device, self.dtype, self.max_tokens, self.max_rows, self.page_size,
                                 options.max_num_seqs, max_seq_len=options.max_model_len)
+        blaslt.configure(enabled=options.gemm_library, tuning=options.gemm_tuning, plan_file=options.gemm_plan_file)
         model.bind(self.ctx)
         self._build_caches()
         self.batch = StepBatch(device, self.max_tokens, options.max_num_seqs, self.max_rows,
@@ -91,8 +92,11 @@ class ModelRunner:
         self._graphs: dict[int, torch.cuda.CUDAGraph] = {}
         self._graph_pool = None
         self._capture_stream = None
-        if options.hip_graph and self.device.type == "cuda":
+        # a step is replayed from a graph only where every part reads what changes between steps from device memory
+        self._graphs_allowed = bool(options.hip_graph) and model.capturable()
+        if self._graphs_allowed and self.device.type == "cuda":
             _first_graph(self.device)
+        self.warm_up()
 
     # ---- construction --------------------------------------------------------------------------
     @classmethod
@@ -121,30 +125,36 @@ class ModelRunner:
         return r
 
     def _build_caches(self) -> None:
+        """Sizes and allocates what the run entries keep between steps. Every question about a cache is put to its
+        CacheSpec (group, bytes a page, bytes a request, tensors), so a mixer may bring a kind of its own."""
         opt = self.options
         needs = self.model.cache_needs()
         self.max_blocks_per_seq = -(-opt.max_model_len // self.page_size)
-        # groups: run entries whose KV needs coincide share block tables
+        # one more slot than requests: the padded rows of a replayed graph read and write the spare
+        self.num_slots = opt.max_num_seqs + 1
+        # groups: run entries whose paged needs coincide share block tables
         keys: list[tuple] = []
+        windows: list = []
         entry_group: list[int | None] = []
         for need in needs:
-            if isinstance(need, KVSpec):
-                k = need.group_key()
-                if k not in keys:
-                    keys.append(k)
-                entry_group.append(keys.index(k))
-            else:
+            k = need.group_key() if need is not None else None
+            if k is None:
                 entry_group.append(None)
-        esize = torch.empty((), dtype=self.dtype).element_size()
-        page_bytes = sum(2 * n.kv_heads * n.head_dim * self.page_size * esize for n in needs if isinstance(n, KVSpec))
-        state_bytes = 0
+                continue
+            if k not in keys:
+                keys.append(k)
+                windows.append(need.window)
+            elif windows[keys.index(k)] != need.window:
+                raise ValueError(f"cache group {k!r} is asked for with windows {windows[keys.index(k)]} and {need.window}: "
+                                 "the group key must tell them apart")
+            entry_group.append(keys.index(k))
+        # prompt portions end where every layer's own chunks end
+        import math
         for n in needs:
-            if isinstance(n, StateSpec):
-                e = torch.empty((), dtype=getattr(torch, n.dtype)).element_size()
-                numel = 1
-                for s in n.shape:
-                    numel *= s
-                state_bytes += numel * e * opt.max_num_seqs
+            if n is not None and n.chunk_alignment > 1:
+                opt.prefill_chunk_alignment = math.lcm(opt.prefill_chunk_alignment, n.chunk_alignment)
+        page_bytes = sum(n.page_bytes(self.page_size, self.dtype) for n in needs if n is not None)
+        slot_bytes = sum(n.slot_bytes(self.dtype) for n in needs if n is not None) * self.num_slots
         if opt.num_blocks is not None:
             num_blocks = opt.num_blocks
         else:
@@ -153,7 +163,7 @@ class ModelRunner:
             free, total = torch.cuda.mem_get_info(self.device)
             used = total - free
             reserve = 512 << 20
-            budget = min(free, int(total * opt.gpu_memory_utilization) - used) - reserve - state_bytes
+            budget = min(free, int(total * opt.gpu_memory_utilization) - used) - reserve - slot_bytes
             budget -= 3 * self.max_rows * self.model.spec.vocab_size * 4
             num_blocks = budget // max(page_bytes, 1) if page_bytes else 1
             if num_blocks <= 0:
@@ -162,36 +172,82 @@ class ModelRunner:
             raise RuntimeError(f"one request of max_model_len {opt.max_model_len} needs {self.max_blocks_per_seq} "
                                f"pages, the pool has {num_blocks}")
         self.num_blocks = int(num_blocks)
-        self.group_specs = [GroupSpec(self.page_size, self.num_blocks, window=k[3]) for k in keys]
+        self.group_specs = [GroupSpec(self.page_size, self.num_blocks, window=w) for w in windows]
         prefix = opt.enable_prefix_caching
+        rebuilt_from_tokens = all(n.recomputable for n in needs if n is not None)
         if prefix is None:
             # reusing pages is only the whole truth where the pages are: no layer drops keys, none keeps state of its own
-            prefix = (bool(keys) and all(g.window is None for g in self.group_specs)
-                      and not any(isinstance(n, StateSpec) for n in needs))
-        elif prefix and any(isinstance(n, StateSpec) for n in needs):
+            prefix = bool(keys) and all(g.window is None for g in self.group_specs) and rebuilt_from_tokens
+        elif prefix and not rebuilt_from_tokens:
             raise ValueError("the prefix cache cannot restore a layer's own state: switch it off for this model")
         self.cache = CacheManager(self.group_specs, opt.max_num_seqs, prefix_caching=prefix)
         self.cache_views: list[CacheView] = []
-        self.state_tensors: list[torch.Tensor] = []
+        self._slotted: list[tuple] = []     # (spec, tensors) of the entries with per-request memory
         own: dict[int, CacheView] = {}
         for i, (e, need) in enumerate(zip(self.model.run, needs)):
             if e.cache != i:
                 src = own[e.cache]
-                self.cache_views.append(CacheView(src.group, src.k, src.v, owner=False, state=src.state))
+                self.cache_views.append(CacheView(src.group, owner=False, tensors=src.tensors))
                 continue
-            if isinstance(need, KVSpec):
-                geometry = (self.num_blocks, need.kv_heads, self.page_size, need.head_dim)
-                k = torch.empty(ops.k_cache_shape(*geometry), dtype=self.dtype, device=self.device)
-                v = torch.empty(ops.v_cache_shape(*geometry), dtype=self.dtype, device=self.device)
-                view = CacheView(entry_group[i], k, v, owner=True)
-            elif isinstance(need, StateSpec):
-                st = torch.zeros((opt.max_num_seqs, *need.shape), dtype=getattr(torch, need.dtype), device=self.device)
-                self.state_tensors.append(st)
-                view = CacheView(None, None, None, owner=True, state=st)
+            if need is None:
+                view = CacheView(None, owner=True)
             else:
-                view = CacheView(None, None, None, owner=True)
+                tensors = need.allocate(self.num_blocks, self.page_size, self.num_slots, self.dtype, self.device)
+                view = CacheView(entry_group[i], owner=True, tensors=tensors)
+                if need.slot_bytes(self.dtype) > 0:
+                    self._slotted.append((need, tensors))
             own[i] = view
             self.cache_views.append(view)
+
+    @property
+    def state_tensors(self) -> list:
+        """The per-request tensors of all entries that have any (what tests and reports look at)."""
+        return [t for _, tensors in self._slotted for t in tensors.values()]
+
+    def _reset_fresh_slots(self) -> None:
+        fresh = self.cache.take_fresh_slots()
+        if fresh and self._slotted:
+            idx = torch.tensor(fresh, device=self.device, dtype=torch.long)
+            for need, tensors in self._slotted:
+                need.reset_slots(tensors, idx)
+
+    def warm_up(self) -> None:
+        """Runs one step of every row count that the library's products can meet, largest first, with made-up
+        requests that are freed again, so that every shape has its algorithm (measured now, or read from the plan
+        file) before the first real step; no later step times anything, and what a product computes does not
+        depend on when its shape first came up. Nothing to do in 32-bit (own kernels only) or without measuring."""
+        opt = self.options
+        if self.dtype != torch.bfloat16 or opt.gemm_tuning != "measured" or not blaslt.available() or not self.group_specs:
+            return
+        most = min(self.max_tokens, self.num_blocks * self.page_size, opt.max_num_seqs * opt.max_model_len)
+        bucket = gemm.ROW_BUCKET
+        sizes = sorted({min(t, most) for t in range(2 * bucket, most + bucket, bucket)}, reverse=True)
+        met = blaslt.worth_measuring_met
+        with blaslt.measuring():
+            for n, total in enumerate(sizes):
+                entries, left, i = [], total, 0
+                while left > 0:
+                    take = min(left, opt.max_model_len)
+                    rid = ("warm-up", i)
+                    if not self.reserve(rid, 0, take):
+                        self.finish(rid)
+                        break
+                    entries.append(Entry(rid, [0] * take, 0, []))
+                    left -= take
+                    i += 1
+                if left == 0:
+                    want, e = min(total, self.max_rows), 0
+                    while want > 0:     # logits at as many rows as the head can be asked for
+                        k = min(want, len(entries[e].tokens))
+                        entries[e].want = list(range(k))
+                        want -= k
+                        e += 1
+                    self.step(entries)
+                for e in entries:
+                    self.finish(e.req_id)
+                if n == 0 and blaslt.worth_measuring_met == met:
+                    break       # not even the largest step holds a product worth measuring: a small model
+        torch.cuda.synchronize(self.device)
 
     # ---- the step function ---------------------------------------------------------------------
     def step(self, entries: list[Entry]) -> torch.Tensor:
@@ -210,15 +266,11 @@ class ModelRunner:
 
     def _run(self, n: int, single_rows: bool, fill) -> torch.Tensor:
         b = self.batch
-        if self.options.hip_graph and not self.state_tensors and single_rows and 0 < n <= self._buckets[-1]:
+        if self._graphs_allowed and single_rows and 0 < n <= self._buckets[-1]:
             return self._graph_step(n, fill)
         fill(None)
         b.upload()
-        fresh = self.cache.take_fresh_slots()
-        if fresh and self.state_tensors:
-            idx = torch.tensor(fresh, device=self.device, dtype=torch.long)
-            for st in self.state_tensors:
-                st.index_fill_(0, idx, 0)
+        self._reset_fresh_slots()
         return self.model.forward(b, self.cache_views)
 
     def _graph_step(self, n: int, fill) -> torch.Tensor:
@@ -228,32 +280,33 @@ class ModelRunner:
         b = self.batch
         bucket = next(x for x in self._buckets if x >= n)
         fill(bucket)
-        b.max_len_bound = self.options.max_model_len  # the graph must hold for every later length
         b.upload()
-        self.cache.take_fresh_slots()
+        self._reset_fresh_slots()   # outside the graph: which slots are fresh changes from step to step
         g = self._graphs.get(bucket)
-        if g is None:
-            # once eagerly (first-use initialisation must not happen under capture; it writes the
-            # same cache slots with the same values as the replay will), then capture
-            self.model.forward(b, self.cache_views)
-            torch.cuda.synchronize()
-            g = torch.cuda.CUDAGraph()
-            if self._capture_stream is None:
-                self._capture_stream = torch.cuda.Stream(device=self.device)
-            side = self._capture_stream
-            side.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(side):
-                # by hand: torch's capture context would collect garbage and empty the allocator's cache first
-                g.capture_begin(pool=self._graph_pool)
-                try:
-                    self.model.forward(b, self.cache_views)
-                finally:
-                    g.capture_end()
-            torch.cuda.current_stream().wait_stream(side)
-            if self._graph_pool is None:
-                self._graph_pool = g.pool()
-            self._graphs[bucket] = g
-        g.replay()
+        if g is not None:
+            g.replay()
+            return self.model.logits[:n]
+        # The first step of a bucket runs eagerly (first-use initialisation must not happen under capture) and its
+        # result is the step's result; the capture that follows records the same launches without running them.
+        # Nothing is replayed in this step: a part with state of its own must see each step once.
+        self.model.forward(b, self.cache_views)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        if self._capture_stream is None:
+            self._capture_stream = torch.cuda.Stream(device=self.device)
+        side = self._capture_stream
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            # by hand: torch's capture context would collect garbage and empty the allocator's cache first
+            g.capture_begin(pool=self._graph_pool)
+            try:
+                self.model.forward(b, self.cache_views)
+            finally:
+                g.capture_end()
+        torch.cuda.current_stream().wait_stream(side)
+        if self._graph_pool is None:
+            self._graph_pool = g.pool()
+        self._graphs[bucket] = g
         return self.model.logits[:n]
 
     # ---- request bookkeeping shared by replay and tests ------------------------------------------

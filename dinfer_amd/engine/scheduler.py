@@ -86,7 +86,7 @@ class Scheduler:
                                 options.prefill_tokens_per_step or 0, options.long_prefill_token_threshold or 0,
                                 int(options.enable_chunked_prefill), int(options.decode_exempt_from_budget),
                                 int(cache.prefix_caching if options.enable_prefix_caching is None
-                                    else options.enable_prefix_caching))
+                                    else options.enable_prefix_caching), int(options.prefill_chunk_alignment or 1))
         eos = np.array(sorted(self.eos) or [0], dtype=np.int32)
         self._h = native.created("dh_sched_create", o, cache._h, eos.ctypes.data, len(self.eos))
         self.requests: dict = {}        # id -> Request, for every request that is not finished

@@ -72,15 +72,19 @@ def embedding(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torc
     return out
 
 
+GATED_ACTS = {"silu": 0}   # activations the gated kernels know -> their code in the C interface
+MAX_HEAD_DIM = 512         # the largest head the norm / rotation / plain attention kernels hold in registers
+
+
 def gated_act(gate_up: torch.Tensor, out: torch.Tensor, tokens: int, act: str = "silu") -> torch.Tensor:
     """out[t, i] = act(gate_up[t, i]) * gate_up[t, I + i]."""
     _need_gpu(gate_up, out)
-    if act != "silu":
-        raise lib.KernelError(f"gated activation {act!r} has no kernel (only 'silu')")
+    if act not in GATED_ACTS:
+        raise lib.KernelError(f"gated activation {act!r} has no kernel (known: {sorted(GATED_ACTS)})")
     inter = out.shape[1]
     assert gate_up.shape[1] == 2 * inter and gate_up.dtype == out.dtype and out.is_contiguous()
     assert gate_up.shape[0] >= tokens and out.shape[0] >= tokens
-    lib.call("dinfer_gated_act", dtype_code(out.dtype), 0, gate_up.data_ptr(), out.data_ptr(), tokens, inter,
+    lib.call("dinfer_gated_act", dtype_code(out.dtype), GATED_ACTS[act], gate_up.data_ptr(), out.data_ptr(), tokens, inter,
              _rows(gate_up), _stream())
     return out
 
@@ -173,7 +177,7 @@ def qkv_post(qkv: torch.Tensor, tokens: int, *, heads: int, kv_heads: int, head_
     """Per-head q/k norm, rotation, q written back in place, k and v written to the cache pages.
 
     k_cache and v_cache in the page layouts above; slot_mapping int64 [T] (None: nothing is written
-    to the cache). token_runs: the tokens come in runs of consecutive positions (prompt portions, not
+    to the cache and k is written back in place, as q is). token_runs: the tokens come in runs of consecutive positions (prompt portions, not
     single decoded tokens); it only chooses the faster of two ways of writing V.
     """
     _need_gpu(qkv, q_gain, k_gain, positions, cos_sin, k_cache, v_cache, slot_mapping)

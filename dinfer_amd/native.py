@@ -29,7 +29,7 @@ class BatchFacts(Structure):
 class SchedOptions(Structure):
     _fields_ = [(n, _I) for n in ("max_num_batched_tokens", "max_num_seqs", "max_model_len", "prefill_tokens_per_step",
                                   "long_prefill_token_threshold", "enable_chunked_prefill",
-                                  "decode_exempt_from_budget", "enable_prefix_caching")]
+                                  "decode_exempt_from_budget", "enable_prefix_caching", "prefill_chunk_alignment")]
 
 
 class Scheduled(Structure):

@@ -2,4 +2,4 @@ from . import attention, block, mlp, norm, position  # noqa: F401  (register the
 from .base import Block, BuildContext, CacheView, Carried, FeedForward, Into, Mixer, Norm, Part, PositionEncoding, Workspace
 from .model import DecoderModel, expected_tensors
 from .registry import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, Registry
-from .spec import KVSpec, LayerSpec, ModelSpec, PartSpec, RunEntry, StateSpec, TensorSpec, part
+from .spec import CacheSpec, KVSpec, LayerSpec, ModelSpec, PartSpec, RunEntry, StateSpec, TensorSpec, part

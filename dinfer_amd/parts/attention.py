@@ -20,11 +20,15 @@ from .spec import KVSpec, PartSpec, TensorSpec
 @MIXERS.register("attention")
 class Attention(Mixer):
     carries_norms = True   # the q/k/v product takes a Carried, the output product an Into
+    capturable = True      # every kernel reads tokens, positions, slots, tables and lengths from the batch's device buffers
 
     def __init__(self, hidden: int, heads: int, kv_heads: int, head_dim: int, position: PartSpec,
                  qk_norm: PartSpec | None = None, window: int | None = None, scale: float | None = None):
         if heads % kv_heads:
             raise ValueError(f"heads {heads} not divisible by kv_heads {kv_heads}")
+        if head_dim <= 0 or head_dim % 8 or head_dim > ops.MAX_HEAD_DIM:   # said at build, not at the first step
+            raise ValueError(f"attention: head_dim {head_dim} has no kernel (multiples of 8 up to {ops.MAX_HEAD_DIM}; "
+                             "the cache stores keys in pieces of 8 elements)")
         self.hidden, self.heads, self.kv_heads, self.head_dim = hidden, heads, kv_heads, head_dim
         self.window = window
         self.scale = float(scale) if scale is not None else head_dim ** -0.5
@@ -51,6 +55,8 @@ class Attention(Mixer):
         if self.q_norm is not None:
             t["q_norm.weight"] = TensorSpec((D,), init="gain")
             t["k_norm.weight"] = TensorSpec((D,), init="gain")
+        for n, spec in self.position.tensors().items():   # an encoding with parameters of its own (rotations have none)
+            t["position." + n] = spec
         return t
 
     def load(self, get):
@@ -61,6 +67,7 @@ class Attention(Mixer):
         if self.q_norm is not None:
             self.q_norm.load(lambda n, **kw: get("q_norm." + n, **kw))
             self.k_norm.load(lambda n, **kw: get("k_norm." + n, **kw))
+        self.position.load(lambda n, **kw: get("position." + n, **kw))
 
     def bind(self, ctx):
         ws = ctx.workspace
@@ -75,16 +82,28 @@ class Attention(Mixer):
         T = batch.num_tokens
         g = cache.group
         self.qkv.forward(x, self.qkv_buf, T, scratch=True)
-        qn = self.q_norm
-        ops.qkv_post(
-            self.qkv_buf, T, heads=self.heads, kv_heads=self.kv_heads, head_dim=self.head_dim,
-            q_off=0, k_off=self.q_size, v_off=self.q_size + self.kv_size,
-            q_gain=qn.weight if qn else None, k_gain=self.k_norm.weight if qn else None,
-            eps=qn.eps if qn else 0.0, gain_offset=qn.weight_offset if qn else 0.0,
-            positions=batch.positions, cos_sin=self.position.table(), rotary_dim=self.position.rotary_dim,
-            rope_style=self.position.style, k_cache=cache.k, v_cache=cache.v,
-            slot_mapping=batch.slot_mapping[g] if cache.owner else None, page_size=self.page_size,
-            token_runs=batch.max_q_len >= 8)
+        qn, pos = self.q_norm, self.position
+        geometry = dict(heads=self.heads, kv_heads=self.kv_heads, head_dim=self.head_dim, q_off=0, k_off=self.q_size,
+                        v_off=self.q_size + self.kv_size, positions=batch.positions, page_size=self.page_size)
+        norm = dict(q_gain=qn.weight if qn else None, k_gain=self.k_norm.weight if qn else None,
+                    eps=qn.eps if qn else 0.0, gain_offset=qn.weight_offset if qn else 0.0)
+        no_norm = dict(q_gain=None, k_gain=None, eps=0.0, gain_offset=0.0)
+        write = dict(k_cache=cache.k, v_cache=cache.v, slot_mapping=batch.slot_mapping[g] if cache.owner else None,
+                     token_runs=batch.max_q_len >= 8)
+        if pos.fused:
+            # per-head norm, rotation by the encoding's table and the cache write in one kernel
+            ops.qkv_post(self.qkv_buf, T, **geometry, **norm, cos_sin=pos.table(), rotary_dim=pos.rotary_dim,
+                         rope_style=pos.style, **write)
+        else:
+            # an encoding that is no rotation by a table works on q and k itself, between the norm and the cache write
+            if qn:
+                ops.qkv_post(self.qkv_buf, T, **geometry, **norm, cos_sin=None, rotary_dim=0, rope_style=0, k_cache=None,
+                             v_cache=None, slot_mapping=None, token_runs=False)
+            q = self.qkv_buf[:T, :self.q_size].view(T, self.heads, self.head_dim)
+            k = self.qkv_buf[:T, self.q_size:self.q_size + self.kv_size].view(T, self.kv_heads, self.head_dim)
+            pos.transform(q, k, batch.positions[:T])
+            if cache.owner:
+                ops.qkv_post(self.qkv_buf, T, **geometry, **no_norm, cos_sin=None, rotary_dim=0, rope_style=0, **write)
         attn_kernels.paged_attention(
             self.qkv_buf, self.attn_buf, cache.k, cache.v, batch, g, self.attn_ws, scale=self.scale,
             window=self.window or 0, heads=self.heads, kv_heads=self.kv_heads, head_dim=self.head_dim,

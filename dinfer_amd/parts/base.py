@@ -11,7 +11,7 @@ from typing import Callable
 
 import torch
 
-from .spec import KVSpec, StateSpec, TensorSpec
+from .spec import CacheSpec, TensorSpec
 
 
 class Workspace:
@@ -51,9 +51,19 @@ class BuildContext:
         self.max_tokens, self.max_rows, self.page_size, self.max_reqs = max_tokens, max_rows, page_size, max_reqs
         self.max_seq_len = max_seq_len
         self.workspace = Workspace(device, dtype, max_tokens)
+        self._shared: dict = {}
+
+    def share(self, key, make):
+        """One object for all parts that ask under the same key (a table every layer would otherwise build for itself)."""
+        if key not in self._shared:
+            self._shared[key] = make()
+        return self._shared[key]
 
 
 class Part:
+    # True: forward reads what changes from step to step from the batch's device tensors only (see Mixer.capturable)
+    capturable = True
+
     def tensors(self) -> dict[str, TensorSpec]:
         """Local tensor name -> what the weight file must hold for it."""
         return {}
@@ -109,33 +119,67 @@ class Into:
 
 
 class PositionEncoding(Part):
-    """Gives the rotation table the mixer's kernel applies to q and k."""
+    """How a mixer's queries and keys learn their positions. Two forms:
+
+    fused (the default): a rotation of q and k by a table, which the mixer's kernel applies together with the per-head
+    norm and the cache write: `table()` gives float32 [positions, rotary_dim] = [cos | sin] (None: no rotation),
+    `rotary_dim` says how many leading dims of a head turn and `style` how they pair up.
+
+    not fused (`fused = False`): anything else that acts on q and k: the mixer calls `transform(q, k, positions)`
+    between the per-head norm and the cache write, so the keys in the cache carry it.
+    """
+    fused: bool = True
     rotary_dim: int = 0
     style: int = 0  # 0: pairs (i, i + rotary_dim/2); 1: pairs (2i, 2i+1)
 
     def table(self) -> torch.Tensor | None:
-        """float32 [max_positions, rotary_dim] = [cos | sin], or None for no rotation."""
         return None
+
+    def transform(self, q: torch.Tensor, k: torch.Tensor, positions: torch.Tensor) -> None:
+        """q [T, heads, D] and k [T, kv_heads, D]: views of the step's buffer, changed in place; positions int32 [T]
+        on the device (read them there: a captured step is replayed with other contents)."""
+        raise NotImplementedError
 
 
 class CacheView:
     """The cache of one run entry as its mixer sees it.
 
-    group: index of the page group (block tables, slot mappings in the batch);
-    k, v: this entry's page tensors; owner: False if the pages belong to another
-    entry (read only); state: [max_seqs, *shape] tensor for fixed-size state.
+    group: index of the page group (block tables, slot mappings in the batch), None if the entry has no pages;
+    tensors: what the entry's CacheSpec allocated, by name, also reachable as attributes (an attention mixer reads
+    `cache.k` and `cache.v`, a mixer with per-request state `cache.state`: [slots, *shape], indexed by
+    batch.state_slots); owner: False if the memory belongs to another entry (read only).
     """
 
-    def __init__(self, group: int | None = None, k=None, v=None, owner: bool = True, state=None):
-        self.group, self.k, self.v, self.owner, self.state = group, k, v, owner, state
+    def __init__(self, group: int | None = None, k=None, v=None, owner: bool = True, state=None, tensors: dict | None = None):
+        self.group, self.owner = group, owner
+        self.tensors = dict(tensors or {})
+        for name, t in (("k", k), ("v", v), ("state", state)):
+            if t is not None:
+                self.tensors[name] = t
+
+    def __getattr__(self, name):
+        # only reached for names that are no attribute of the object: the cache's tensors, None for the usual
+        # three where the entry has none of that kind
+        tensors = self.__dict__.get("tensors", {})
+        if name in tensors:
+            return tensors[name]
+        if name in ("k", "v", "state"):
+            return None
+        raise AttributeError(name)
 
 
 class Mixer(Part):
     # True: forward also takes a Carried as x and the keyword `into` (an Into or None), and may return a Carried
     # when it has added its result to the stream itself. Parts that leave it False are given plain tensors.
     carries_norms = False
+    # True: forward reads what changes from step to step (tokens, positions, slots, tables, lengths) from the batch's
+    # device tensors only, never from host copies, and allocates nothing whose address must survive, so a step of
+    # single rows captured once may be replayed for other requests. A mixer that leaves it False keeps every step of
+    # its model eager.
+    capturable = False
 
-    def cache_spec(self) -> KVSpec | StateSpec | None:
+    def cache_spec(self) -> CacheSpec | None:
+        """What this mixer keeps between steps (a KVSpec, a StateSpec, a CacheSpec of its own), or None."""
         return None
 
     def forward(self, x: torch.Tensor, batch, cache: CacheView) -> torch.Tensor:
@@ -162,6 +206,7 @@ class Block(Part):
     `next_norm` so that it can return one. Other blocks see neither.
     """
     carries_norms = False
+    capturable = False   # an arrangement says so itself once all its parts are (see Mixer.capturable)
 
     def input_norm(self):
         """The norm this block applies to the stream first, if the block before may carry it; else None."""

@@ -44,6 +44,10 @@ class PreNormBlock(Block):
     def _parts(self):
         return zip(self.prefixes, (self.mixer, self.ff, self.norm_in, self.norm_post))
 
+    @property
+    def capturable(self):
+        return all(part.capturable for _, part in self._parts())
+
     def tensors(self):
         return {p + n: s for p, part in self._parts() for n, s in part.tensors().items()}
 

@@ -4,7 +4,7 @@ from __future__ import annotations
 
 import torch
 
-from ..kernels import gemm
+from ..kernels import gemm, ops
 from .base import Carried, FeedForward
 from .linear import Linear
 from .registry import FEED_FORWARDS
@@ -16,6 +16,8 @@ class GatedMLP(FeedForward):
     carries_norms = True   # the gate/up product takes a Carried, the down product an Into
 
     def __init__(self, hidden: int, intermediate: int, act: str = "silu"):
+        if act not in ops.GATED_ACTS:   # said when the model is built, not at its first step
+            raise ValueError(f"gated feed-forward: activation {act!r} has no kernel (known: {sorted(ops.GATED_ACTS)})")
         self.hidden, self.intermediate, self.act = hidden, intermediate, act
         self.gate_up = Linear(hidden, 2 * intermediate)
         self.down = Linear(intermediate, hidden)

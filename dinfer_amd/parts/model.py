@@ -92,11 +92,15 @@ class DecoderModel:
 
     # ---- cache needs ---------------------------------------------------------------------------
     def cache_needs(self) -> list:
-        """Per run entry: KVSpec / StateSpec / None of the cache it owns; None if it borrows one."""
+        """Per run entry: the CacheSpec of the cache it owns; None if it has none or borrows one."""
         out = []
         for i, e in enumerate(self.run):
             out.append(self.blocks[e.layer].mixer.cache_spec() if e.cache == i else None)
         return out
+
+    def capturable(self) -> bool:
+        """Whether a step of single rows may be captured once and replayed for other requests."""
+        return all(self.blocks[e.layer].capturable for e in self.run) and self.final_norm.capturable
 
     # ---- execution -----------------------------------------------------------------------------
     def bind(self, ctx: BuildContext) -> None:

@@ -36,18 +36,20 @@ class Rotary(PositionEncoding):
         self.head_dim, self.theta, self.max_positions = head_dim, float(theta), max_positions
         self.rotary_dim, self.style = rd, STYLES[style]
         self._table = None
-        self._device = None
 
     def bind(self, ctx):
-        self._device = ctx.device
+        # one table for all layers with the same rotation, as long as the longest request the engine admits
+        n = min(self.max_positions, ctx.max_seq_len or self.max_positions)
+        self._table = ctx.share(("rotary", self.theta, self.rotary_dim, self.style, n),
+                                lambda: self.host_table(n).to(ctx.device).contiguous())
 
-    def host_table(self) -> torch.Tensor:
+    def host_table(self, positions: int | None = None) -> torch.Tensor:
         i = torch.arange(0, self.rotary_dim // 2, dtype=torch.float64)
         freq = torch.pow(torch.tensor(self.theta, dtype=torch.float64), -2.0 * i / self.rotary_dim)
-        ang = torch.arange(self.max_positions, dtype=torch.float64)[:, None] * freq[None, :]
+        ang = torch.arange(positions or self.max_positions, dtype=torch.float64)[:, None] * freq[None, :]
         return torch.cat([ang.cos(), ang.sin()], dim=1).to(torch.float32)
 
     def table(self):
         if self._table is None:
-            self._table = self.host_table().to(self._device).contiguous()
+            raise RuntimeError("the rotation table is built in bind(); the part has not been bound")
         return self._table

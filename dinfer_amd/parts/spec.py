@@ -38,8 +38,46 @@ class TensorSpec:
     integer: bool = False
 
 
+class CacheSpec:
+    """What one run entry keeps between steps, and how its memory is made. The engine sizes, groups and allocates
+    every cache through these methods only, so a mixer with another kind of cache (one vector a token, unequal key
+    and value widths, a layout of its own) brings a subclass and nothing in the engine changes.
+
+    Paged memory: entries whose `group_key()` is equal share a pool of pages and one block table a request; a page id
+    is valid in the tensors of every entry of the group. `page_bytes` says what one page of this entry takes, and
+    `allocate` makes the tensors for `num_blocks` pages. Per-request memory of fixed size: `slot_bytes` a request,
+    `allocate` makes room for `num_slots` requests (one of them is a spare that padded rows of a replayed graph use),
+    `reset_slots` clears the slots of requests that have just been admitted.
+    """
+    window: int | None = None      # W: pages whose keys all lie more than W before the next token are given back
+    recomputable: bool = True      # the contents follow from the request's tokens alone (pages may be shared and refilled)
+    chunk_alignment: int = 1       # prompt portions that do not end the request must end at a multiple of this
+
+    def group_key(self) -> tuple | None:
+        """Hashable name of the page group; None if nothing here is paged."""
+        return None
+
+    def page_bytes(self, page_size: int, dtype) -> int:
+        return 0
+
+    def slot_bytes(self, dtype) -> int:
+        return 0
+
+    def allocate(self, num_blocks: int, page_size: int, num_slots: int, dtype, device) -> dict:
+        """name -> tensor; the mixer finds them as attributes of its CacheView."""
+        return {}
+
+    def reset_slots(self, tensors: dict, slots) -> None:
+        """slots: int64 tensor of request slots that start from nothing."""
+
+
+def _element_size(dtype) -> int:
+    import torch
+    return torch.empty((), dtype=dtype).element_size()
+
+
 @dataclass(frozen=True)
-class KVSpec:
+class KVSpec(CacheSpec):
     """Cache need of a mixer that stores a key and a value per token and kv head.
 
     window: None keeps every key of the request; W keeps the last W keys, so
@@ -53,12 +91,38 @@ class KVSpec:
         # Layers of equal page geometry and equal window share block tables.
         return ("kv", self.kv_heads, self.head_dim, self.window)
 
+    def page_bytes(self, page_size, dtype):
+        return 2 * self.kv_heads * self.head_dim * page_size * _element_size(dtype)
+
+    def allocate(self, num_blocks, page_size, num_slots, dtype, device):
+        import torch
+        from ..kernels import ops
+        geometry = (num_blocks, self.kv_heads, page_size, self.head_dim)
+        return {"k": torch.empty(ops.k_cache_shape(*geometry), dtype=dtype, device=device),
+                "v": torch.empty(ops.v_cache_shape(*geometry), dtype=dtype, device=device)}
+
 
 @dataclass(frozen=True)
-class StateSpec:
-    """Cache need of a mixer with per-request state of fixed size (shape per request)."""
+class StateSpec(CacheSpec):
+    """Cache need of a mixer with per-request state of fixed size (shape per request). The state cannot be rebuilt
+    from pages, so a model that has one gets no prefix cache."""
     shape: tuple
     dtype: str = "float32"
+    recomputable = False
+
+    def slot_bytes(self, dtype):
+        import torch
+        n = 1
+        for s in self.shape:
+            n *= s
+        return n * _element_size(getattr(torch, self.dtype))
+
+    def allocate(self, num_blocks, page_size, num_slots, dtype, device):
+        import torch
+        return {"state": torch.zeros((num_slots, *self.shape), dtype=getattr(torch, self.dtype), device=device)}
+
+    def reset_slots(self, tensors, slots):
+        tensors["state"].index_fill_(0, slots, 0)
 
 
 @dataclass(frozen=True)

@@ -282,3 +282,46 @@ def test_bfloat16_against_the_32bit_path_at_the_8b_layer_sizes(tmp_path):
     clear = (top2[:, 0] - top2[:, 1]) > 0.15 * spread[:, 0]
     assert int(clear.sum()) > 100
     assert bool((low.argmax(-1)[clear] == ref.argmax(-1)[clear]).all())
+
+
+_ONE_STEP = """
+import sys, random
+import torch
+from dinfer_amd.config import EngineOptions
+from dinfer_amd.engine.batch import Entry
+from dinfer_amd.engine.runner import ModelRunner
+model, tuning, plans, out = sys.argv[1:5]
+opt = EngineOptions(dtype="bfloat16", max_model_len=512, max_num_seqs=4, max_num_batched_tokens=640, block_size=16,
+                    num_blocks=48, max_logits_rows=64, gemm_tuning=tuning, gemm_plan_file=plans)
+r = ModelRunner.from_dir(model, opt)
+rng = random.Random(11)
+ids = [rng.randrange(2048) for _ in range(520)]
+assert r.reserve("a", 0, 400) and r.reserve("b", 0, 120)
+logits = r.step([Entry("a", ids[:400], 0, list(range(0, 400, 9))), Entry("b", ids[400:], 0, list(range(0, 120, 9)))])
+torch.save(logits.cpu(), out)
+from dinfer_amd.kernels import blaslt
+print("measured" if any(p and p.times for p in blaslt._plans.values()) else "not measured")
+"""
+
+
+@pytest.mark.parametrize("tuning", ["heuristic", "measured"])
+def test_two_fresh_processes_compute_the_same_bits(big_models, tmp_path, tuning):
+    """A step of 520 rows (a prompt portion beside decoding requests: the products run in the vendor library) in two
+    processes started one after the other: the bfloat16 logits are equal bit for bit. With the library's first
+    suggestion nothing is measured at all; with measured algorithms the first process measures during its warm-up
+    and keeps its choices in the plan file, the second reads them there and measures nothing."""
+    import subprocess
+    import sys
+    from pathlib import Path
+    root = Path(__file__).resolve().parent.parent
+    outs, said = [], []
+    for i in range(2):
+        out = tmp_path / f"logits{i}.pt"
+        p = subprocess.run([sys.executable, "-c", _ONE_STEP, str(big_models["8B"]), tuning, str(tmp_path / "plans.json"),
+                            str(out)], capture_output=True, text=True, timeout=600, cwd=str(root))
+        assert p.returncode == 0, p.stderr[-2000:]
+        outs.append(torch.load(out, weights_only=True))
+        said.append(p.stdout.strip().splitlines()[-1])
+    assert said == (["not measured", "not measured"] if tuning == "heuristic" else ["measured", "not measured"])
+    assert torch.equal(outs[0], outs[1])
+    assert outs[0].shape == (45 + 14, VOCAB) and bool(outs[0].isfinite().all())

@@ -584,18 +584,43 @@ def test_gemm_small_m(M, out_dtype):
             torch.testing.assert_close(out.double(), want, **t, msg=lambda m_: f"M={M} N={N} K={K} rt={rt} waves={waves}: {m_}")
 
 
-def test_library_gemm_with_measured_algorithm():
-    """Products of many rows: the vendor library called directly, its candidates timed once per shape. Rows may be
-    rounded up to a bucket inside scratch buffers: the rows asked for are right, rows past the bucket untouched."""
+def test_library_gemm_with_measured_algorithm(tmp_path):
+    """Products of many rows: the vendor library called directly. Inside `measuring()` (the engine's warm-up) the
+    candidates of a shape are timed once and the choice goes to the plan file; outside it nothing is timed: a shape
+    runs what it was given, or the library's first suggestion. Rows may be rounded up to a bucket inside scratch
+    buffers: the rows asked for are right, rows past the bucket untouched."""
+    import json
     from dinfer_amd.kernels import blaslt, gemm
+    blaslt.configure(enabled=True, tuning="measured", plan_file=str(tmp_path / "plans.json"))
+    blaslt._plans.clear()                                                    # what earlier tests of this process met
     assert blaslt.available()
+    a = torch.randn(200, 1096, device=DEV).to(torch.bfloat16)
+    w = (torch.randn(1000, 1096, device=DEV) * 0.05).to(torch.bfloat16)
+    out = torch.empty(200, 1000, device=DEV, dtype=torch.bfloat16)
+    gemm.matmul_nt(a, w, out, 200)                                           # outside: no measurement
+    assert not any(p and p.tuned for p in blaslt._plans.values())
+    with blaslt.measuring():
+        _library_gemm_cases(gemm)
+    stored = json.loads((tmp_path / "plans.json").read_text())
+    assert any(k.startswith("520,1000,1096,") for k in stored) and all(0 <= v["index"] < 32 for v in stored.values())
+    # a process that starts with the file takes its choices without measuring: forget the plans, keep the file
+    measured = {k: p.index for k, p in blaslt._plans.items() if p and p.tuned}
+    blaslt._plans.clear()
+    _library_gemm_cases(gemm)
+    again = {k: p.index for k, p in blaslt._plans.items() if p and p.tuned}
+    assert again == measured and all(p.times is None for p in blaslt._plans.values() if p)
+    blaslt.configure(plan_file=None)
+
+
+def _library_gemm_cases(gemm):
+    from dinfer_amd.kernels import blaslt
     for M, N, K in ((130, 200, 264), (520, 1000, 1096), (33, 96, 512), (257, 4096, 512), (70, 50, 100), (40, 33, 6), (35, 7, 1)):
         a = torch.randn(M + 70, K, device=DEV).to(torch.bfloat16)
         w = (torch.randn(N, K, device=DEV) * 0.05).to(torch.bfloat16)
         want = a[:M].double() @ w.double().T
         for pad in (False, True):
             out = torch.full((M + 70, N), 7.0, device=DEV, dtype=torch.bfloat16)
-            for _ in range(2):                                   # the first call measures, the second replays the choice
+            for _ in range(2):                                   # the second call replays the choice of the first
                 gemm.matmul_nt(a, w, out, M, may_pad=pad)
             torch.testing.assert_close(out[:M].double(), want, rtol=2e-2, atol=2e-2, msg=lambda m_: f"{M}x{N}x{K} pad={pad}: {m_}")
             last = -(-M // gemm.ROW_BUCKET) * gemm.ROW_BUCKET if pad else M
@@ -610,12 +635,24 @@ def test_library_gemm_with_measured_algorithm():
     torch.testing.assert_close(out.double(), a.double() @ w.double().T, rtol=1e-4, atol=1e-4)
 
 
-def test_library_gemm_adds_into_its_output():
-    """stream += a . w^T through the library: the first call of a shape times the candidates on a copy (the stream
+def test_library_gemm_adds_into_its_output(tmp_path):
+    """stream += a . w^T through the library: a shape that is measured times the candidates on a copy (the stream
     itself gets the product once), later calls add once each; rows past the bucket are untouched; the few-row and
     tall shapes are refused (other kernels serve them)."""
     from dinfer_amd.kernels import blaslt, gemm
+    blaslt.configure(enabled=True, tuning="measured", plan_file=str(tmp_path / "plans.json"))
+    blaslt._plans.clear()
     assert blaslt.available()
+    with blaslt.measuring():
+        _library_add_cases(gemm)
+    assert any(p and p.tuned for key, p in blaslt._plans.items() if key[-1])   # an adding product was measured too
+    blaslt.configure(plan_file=None)
+    a = torch.randn(32, 64, device=DEV).to(torch.bfloat16)
+    assert not gemm.add_nt(a, torch.zeros(48, 64, device=DEV, dtype=torch.bfloat16), torch.zeros(32, 48, device=DEV, dtype=torch.bfloat16), 32)
+    assert not gemm.add_nt(a.float(), torch.zeros(48, 64, device=DEV), torch.zeros(32, 48, device=DEV), 32)
+
+
+def _library_add_cases(gemm):
     for M, N, K in ((520, 1000, 1096), (130, 200, 264), (40, 33, 8), (257, 4096, 512)):
         a = torch.randn(M + 70, K, device=DEV).to(torch.bfloat16)
         w = (torch.randn(N, K, device=DEV) * 0.05).to(torch.bfloat16)
@@ -631,10 +668,6 @@ def test_library_gemm_adds_into_its_output():
             err = (stream[:M].double() - want).abs()
             assert bool((err <= 2.0 ** -8 * want.abs() + 1e-3 * prod.abs().mean()).all()), f"{M}x{N}x{K} call {call}: {err.max()}"
             assert torch.equal(stream[last:], start[last:]), f"{M}x{N}x{K}: rows past {last} were written"
-    assert any(p and p.tuned for key, p in blaslt._plans.items() if key[-1])   # an adding product was measured too
-    a = torch.randn(32, 64, device=DEV).to(torch.bfloat16)
-    assert not gemm.add_nt(a, torch.zeros(48, 64, device=DEV, dtype=torch.bfloat16), torch.zeros(32, 48, device=DEV, dtype=torch.bfloat16), 32)
-    assert not gemm.add_nt(a.float(), torch.zeros(48, 64, device=DEV), torch.zeros(32, 48, device=DEV), 32)
 
 
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 32])

@@ -367,3 +367,22 @@ def test_abort_between_schedule_and_update_drops_the_sample():
     assert [(r.id, t) for r, t, _ in res] == [(2, 8)]
     s.cache.check()
     assert s.cache.num_free() == 15
+
+
+def test_portions_end_at_multiples_of_the_alignment():
+    """With an alignment of 16 every portion that does not end its request's tokens ends at a multiple of 16: the
+    budget of 40 gives 32; what is left of it (8) is no aligned portion for the second request, which waits; the
+    last portion of a prompt may end anywhere; decoding is untouched."""
+    s = mk(8, 40, 64, prefill_chunk_alignment=16)
+    s.add_request(req(1, 70, 3))
+    s.add_request(req(2, 21, 3))
+    assert step(s, {})[0] == [(1, 32)]                       # 40 cut back to 32; 8 left: less than one aligned portion of 2
+    assert step(s, {1: 9})[0] == [(1, 38)]                   # ends the prompt: may end anywhere; 2 left, nothing for 2
+    assert step(s, {1: 9, 2: 9})[0] == [(1, 1), (2, 21)]     # a whole prompt needs no alignment either
+    assert step(s, {1: 9, 2: 9})[0] == [(1, 1), (2, 1)]
+    s = mk(8, 20, 64, prefill_chunk_alignment=16, long_prefill_token_threshold=24)
+    s.add_request(req(1, 50, 2))
+    s.add_request(req(2, 50, 2))
+    sched = step(s, {})[0]
+    assert sched == [(1, 16)]                                # 20 -> 16; the 4 left hold no aligned portion
+    assert step(s, {})[0] == [(1, 16)]
