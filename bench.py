@@ -13,7 +13,15 @@ token ids back on the host). On the same line:
             time / the dense bf16 MFMA peak (2.5 PFLOP/s; fp32: 157.3 TFLOP/s);
   roofline  the decode step against HBM: bytes it has to read (every weight it uses once,
             and the cache of the live requests) / time, against 8 TB/s;
-  points    decode tokens per second at batch 1 and 64.
+  points    decode tokens per second at batch 1 and 64;
+  and, beside the vendor's figures, what this chip delivers to a kernel that does nothing else, measured before
+  the timed region: `peak_measured` in roofline (a kernel that only reads 4 GB) and in prefill (chains of bf16
+  MFMAs on registers), with `frac_measured` against them;
+  phases    where a decode step's time goes (ms a step, from a second, instrumented run of the same steps that
+            is not the one timed): the host's schedule, fill, launch, sample, wait and update, and the model's
+            kernels on the device between two events (`gpu`);
+  gemm      which of the library's algorithms the products of many rows run with (index in its list per shape),
+            and how each was chosen.
 
 All data is synthetic: weights N(0, 0.02) / gains 1 + N(0, 0.1) drawn on the device, token
 ids uniform in the vocabulary. The reference publishes no number for this size or
@@ -53,6 +61,14 @@ def model_numbers(c, dtype_bytes):
     gains = L * (2 * Hd + 2 * D) + Hd
     return dict(linear_params=L * per_layer, head_params=V * Hd, gains=gains,
                 kv_bytes_per_token=L * 2 * Hkv * D * dtype_bytes)
+
+
+def gemm_summary(chosen):
+    """The library's algorithm per product shape, short: 'rows x n x k[+]' -> index in its list ('+': adds into its output)."""
+    measured = sum(1 for c in chosen if c["chosen"] == "measured")
+    picks = {f"{c['m']}x{c['n']}x{c['k']}{'+' if c['accumulate'] else ''}": c["algorithm"]
+             for c in chosen if c["m"] in (64, 2048)}
+    return {"shapes": len(chosen), "measured": measured, "algorithm_of": picks}
 
 
 def serving(a, torch, Engine, SamplingParams, Qwen3Config) -> int:
@@ -155,6 +171,10 @@ def main() -> int:
                  hip_graph=not a.no_hip_graph)
     rng = random.Random(0)
     V = cfg.vocab_size
+    # what the chip gives a kernel that only reads, and one that only multiplies (before anything is timed)
+    from dinfer_amd.kernels import blaslt, ops
+    hbm_measured = ops.measured_hbm_read(eng.runner.device)
+    mfma_measured = ops.measured_mfma_bf16(eng.runner.device) if a.dtype == "bfloat16" else None
 
     def prompt():
         return [rng.randrange(V) for _ in range(PROMPT)]
@@ -182,10 +202,13 @@ def main() -> int:
         attn_flops = sizes["num_hidden_layers"] * 2 * PROMPT * PROMPT * cfg.head_dim * cfg.num_attention_heads
         pre_flops = 2 * PROMPT * nums["linear_params"] + attn_flops + 2 * nums["head_params"]
         prefill = {"value": round(PROMPT / pre, 1), "tokens": PROMPT, "ms": round(pre * 1e3, 3),
-                   "frac": round(pre_flops / pre / MFMA_PEAK[a.dtype], 4)}
+                   "frac": round(pre_flops / pre / MFMA_PEAK[a.dtype], 4), "peak": MFMA_PEAK[a.dtype] / 1e12, "unit": "TFLOP/s"}
+        if mfma_measured:
+            prefill["peak_measured"] = round(mfma_measured / 1e12, 1)
+            prefill["frac_measured"] = round(pre_flops / pre / mfma_measured, 4)
 
     # ---- decode at a batch: B requests prefilled to 2,048 tokens, then timed decode steps
-    def decode(batch, steps, warmup):
+    def decode(batch, steps, warmup, phases=False):
         ids = [eng.add_request(prompt(), greedy) for _ in range(batch)]
         while any(r.num_computed < PROMPT for r in eng.scheduler.requests.values()):
             eng.step()
@@ -198,18 +221,27 @@ def main() -> int:
         sync()
         dt = (time.perf_counter() - t0) / steps
         ctx = PROMPT + 1 + warmup + steps / 2  # mean cached tokens per request over the timed steps
+        ph = None
+        if phases:      # the same steps once more with the host's clock around every phase; not the timed run
+            eng.measure_phases(True)
+            for _ in range(steps):
+                eng.step()
+            sync()
+            n = max(eng.phases.pop("steps"), 1)
+            ph = {k: round(v / n * 1e3, 4) for k, v in eng.phases.items()}
+            eng.measure_phases(False)
         for i in ids:
             eng.abort(i)
-        return dt, ctx
+        return dt, ctx, ph
 
-    dt, ctx = decode(a.batch, a.steps, a.warmup)
+    dt, ctx, phases = decode(a.batch, a.steps, a.warmup, phases=True)
     weight_bytes = (nums["linear_params"] + nums["head_params"] + nums["gains"] + a.batch * cfg.hidden_size) * dbytes
     step_bytes = weight_bytes + a.batch * ctx * nums["kv_bytes_per_token"]
     achieved = step_bytes / dt
     points = {}
     if not a.no_points:
         for b in (1, 64):
-            d, _ = decode(b, a.steps, a.warmup)
+            d, _, _ = decode(b, a.steps, a.warmup)
             points[f"decode_b{b}"] = round(b / d, 1)
 
     line = {
@@ -227,8 +259,11 @@ def main() -> int:
         },
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK, 4)},
+                     "frac": round(achieved / HBM_PEAK, 4), "peak_measured": round(hbm_measured / 1e9, 1),
+                     "frac_measured": round(achieved / hbm_measured, 4)},
         "points": points,
+        "phases": phases,
+        "gemm": gemm_summary(blaslt.chosen()),
     }
     print(json.dumps(line))
     return 0

@@ -33,6 +33,7 @@ SOURCES = {
     "gemm": "gemm.hip",
     "gemm_mid": "gemm_mid.hip",
     "sampling": "sampling.hip",
+    "ceilings": "ceilings.hip",
     "host": "host/api.cpp",
 }
 HEADERS = ["common.cuh"]

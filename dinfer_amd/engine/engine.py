@@ -51,6 +51,7 @@ class Engine:
         self.sampler = Sampler(self.runner.device, self.runner.max_rows, spec.vocab_size)
         self._ids = itertools.count()
         self._seeds = random.Random()
+        self.phases: dict | None = None     # see measure_phases
 
     # ---- requests ------------------------------------------------------------------------------
     def add_request(self, prompt_ids: list, sampling: SamplingParams | None = None, request_id=None):
@@ -72,6 +73,8 @@ class Engine:
 
     # ---- one step ------------------------------------------------------------------------------
     def step(self) -> list[StepOutput]:
+        if self.phases is not None:
+            return self._step_timed()
         so = self.scheduler.schedule()
         outs = [StepOutput(rid, None, True, reason) for rid, reason in so.force_finished]
         if not len(so):
@@ -84,6 +87,42 @@ class Engine:
         for o in outs:
             if o.finished:
                 self.sampler.forget(o.request_id)
+        return outs
+
+    def measure_phases(self, on: bool = True) -> None:
+        """From now on every step adds its host times to `phases` (seconds; the reference accounts a step the same way,
+        models/qwen3/src/executor.rs:150-157,734-748): schedule (the plan), fill (batch written and sent), launch
+        (graph replay or kernel launches issued), sample (sampling kernels issued), wait (the host waits for the tokens:
+        what the GPU still has to do once everything is issued), update (requests advanced, pages released), and
+        gpu (the model's kernels on the device, between two events); steps counts them."""
+        self.phases = {k: 0.0 for k in ("schedule", "fill", "launch", "sample", "wait", "update", "gpu")} if on else None
+        if on:
+            self.phases["steps"] = 0
+        self.runner.phases = self.sampler.phases = self.phases
+
+    def _step_timed(self) -> list[StepOutput]:
+        import time
+        ph, t = self.phases, time.perf_counter
+        t0 = t()
+        so = self.scheduler.schedule()
+        ph["schedule"] += t() - t0
+        outs = [StepOutput(rid, None, True, reason) for rid, reason in so.force_finished]
+        if not len(so):
+            return outs
+        logits = self.runner.step_planned(self.scheduler, so)          # adds to fill and launch itself
+        rows = [(r.sampling, len(r.output_ids), r.prompt_ids, r.output_ids, r.seed, r.id) for r in so.sampling_requests()]
+        tokens = self.sampler.sample(logits, rows)                     # adds to sample and wait itself
+        t0 = t()
+        for r, tok, reason in self.scheduler.update(so, tokens):
+            outs.append(StepOutput(r.id, tok, reason is not None, reason))
+        for o in outs:
+            if o.finished:
+                self.sampler.forget(o.request_id)
+        ph["update"] += t() - t0
+        ph["steps"] += 1
+        ev = self.runner.take_gpu_events()
+        if ev is not None:
+            ph["gpu"] += ev[0].elapsed_time(ev[1]) * 1e-3                # the tokens are back: both events have passed
         return outs
 
     def generate(self, prompts: list, sampling: SamplingParams | list | None = None) -> list[list[int]]:

@@ -90,6 +90,8 @@ class ModelRunner:
         sizes = {1 << i for i in range(top.bit_length() + 1)} | {24, 40, 48, 56} | {3 << i for i in range(5, top.bit_length())}
         self._buckets = sorted({min(x, top) for x in sizes})
         self._graphs: dict[int, torch.cuda.CUDAGraph] = {}
+        self.phases: dict | None = None     # Engine.measure_phases
+        self._events = None
         self._graph_pool = None
         self._capture_stream = None
         # a step is replayed from a graph only where every part reads what changes between steps from device memory
@@ -265,13 +267,38 @@ class ModelRunner:
                          lambda pad: self.batch.fill_planned(scheduler, pad_to=pad))
 
     def _run(self, n: int, single_rows: bool, fill) -> torch.Tensor:
-        b = self.batch
+        timed = self.phases is not None
+        if timed:
+            import time
+            self._began = time.perf_counter()
         if self._graphs_allowed and single_rows and 0 < n <= self._buckets[-1]:
-            return self._graph_step(n, fill)
-        fill(None)
-        b.upload()
-        self._reset_fresh_slots()
-        return self.model.forward(b, self.cache_views)
+            out = self._graph_step(n, fill)
+        else:
+            self._send(fill, None)
+            self._reset_fresh_slots()
+            out = self.model.forward(self.batch, self.cache_views)
+        if timed:
+            self._events[1].record()
+            self.phases["launch"] += time.perf_counter() - self._began
+        return out
+
+    def _send(self, fill, pad) -> None:
+        """Writes the step into the pinned buffer and starts its copy to the device. While phases are measured
+        (Engine.measure_phases) the host's time up to here counts as "fill", what follows as "launch", and two events
+        bracket the step on the device."""
+        fill(pad)
+        self.batch.upload()
+        if self.phases is not None:
+            import time
+            now = time.perf_counter()
+            self.phases["fill"] += now - self._began
+            self._began = now
+            self._events = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+            self._events[0].record()
+
+    def take_gpu_events(self):
+        ev, self._events = self._events, None
+        return ev
 
     def _graph_step(self, n: int, fill) -> torch.Tensor:
         """A step of single rows replays a HIP graph captured for its batch-size bucket
@@ -279,8 +306,7 @@ class ModelRunner:
         inputs live at fixed addresses; what varies between replays is their content."""
         b = self.batch
         bucket = next(x for x in self._buckets if x >= n)
-        fill(bucket)
-        b.upload()
+        self._send(fill, bucket)
         self._reset_fresh_slots()   # outside the graph: which slots are fresh changes from step to step
         g = self._graphs.get(bucket)
         if g is not None:

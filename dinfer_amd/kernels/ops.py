@@ -452,3 +452,39 @@ def penalties(logits: torch.Tensor, rows: int, ids: torch.Tensor, counts: torch.
     lib.call("dinfer_penalties", logits.data_ptr(), _rows(logits), ids.data_ptr(), counts.data_ptr(),
              offsets.data_ptr(), repetition.data_ptr(), frequency.data_ptr(), presence.data_ptr(), rows,
              logits.shape[1], _stream())
+
+
+# ---- measured ceilings ---------------------------------------------------------------------------
+def measured_hbm_read(device, nbytes: int = 4 << 30, repeats: int = 3) -> float:
+    """Bytes per second a kernel that only reads reaches on `nbytes` of device memory (far beyond the caches):
+    the best of `repeats` runs."""
+    buf = torch.empty(nbytes // 4, dtype=torch.float32, device=device)
+    buf.zero_()
+    blocks = 256 * 8
+    out = torch.empty(blocks * 4, dtype=torch.float32, device=device)
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    best = float("inf")
+    for _ in range(repeats + 1):      # the first run loads the kernel
+        start.record()
+        lib.call("dinfer_stream_read", buf.data_ptr(), buf.numel() * 4, blocks, out.data_ptr(), _stream())
+        end.record()
+        end.synchronize()
+        best = min(best, start.elapsed_time(end) * 1e-3)
+    del buf
+    return nbytes / best
+
+
+def measured_mfma_bf16(device, repeats: int = 3) -> float:
+    """Flops per second of chains of independent bf16 MFMAs on registers, every SIMD busy: the best of `repeats` runs."""
+    blocks, iters = 256 * 8, 2048
+    out = torch.empty(blocks * 256, dtype=torch.float32, device=device)
+    flops = ctypes.c_int64(0)
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    best = float("inf")
+    for _ in range(repeats + 1):
+        start.record()
+        lib.call("dinfer_mfma_loop", iters, blocks, out.data_ptr(), ctypes.addressof(flops), _stream())
+        end.record()
+        end.synchronize()
+        best = min(best, start.elapsed_time(end) * 1e-3)
+    return flops.value / best

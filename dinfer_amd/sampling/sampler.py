@@ -28,6 +28,7 @@ class Sampler:
         self.rows_dev: torch.Tensor | None = None
         self.history: torch.Tensor | None = None   # [max_rows, vocab] int32, made on first use of a penalty
         self._slots: dict = {}                      # request -> [history slot, outputs already counted]
+        self.phases: dict | None = None             # Engine.measure_phases: host time of the last launches and of the wait
         self._free: list = []
 
     def _buffers(self) -> None:
@@ -50,6 +51,8 @@ class Sampler:
         if R == 0:
             return []
         if all(p.is_greedy and not p.has_penalties for p, *_ in rows):
+            if self.phases is not None:
+                return self._timed(lambda: ops.argmax(logits, self.out, R), R)
             ops.argmax(logits, self.out, R)
             return self.out[:R].tolist()
         if any(p.has_penalties for p, *_ in rows):
@@ -63,8 +66,22 @@ class Sampler:
         # back (tolist) before it returned, so that copy is done
         self.rows_dev[:n].copy_(self.rows_host[:n], non_blocking=True)
         any_filter = any(p.top_k > 0 or p.top_p < 1.0 for p, *_ in rows)
+        if self.phases is not None:
+            return self._timed(lambda: ops.sample_rows(logits, self.work, self.scratch, self.rows_dev, self.out, R,
+                                                       any_filter=any_filter), R)
         ops.sample_rows(logits, self.work, self.scratch, self.rows_dev, self.out, R, any_filter=any_filter)
         return self.out[:R].tolist()   # waits for the stream, and with it for the copy out of rows_host
+
+    def _timed(self, launch, R: int) -> list[int]:
+        """The last launches of sample() with the host's time split into issuing them and waiting for the tokens."""
+        import time
+        t0 = time.perf_counter()
+        launch()
+        t1 = time.perf_counter()
+        tokens = self.out[:R].tolist()
+        self.phases["sample"] += t1 - t0
+        self.phases["wait"] += time.perf_counter() - t1
+        return tokens
 
     def forget(self, key) -> None:
         """The request is over: its history slot is free again."""

@@ -869,3 +869,12 @@ def test_add_widen_fill(dtype):
     assert torch.equal(wide, b.float())
     ops().fill_zero(wide)
     assert not wide.any()
+
+
+def test_measured_ceilings_are_plausible():
+    """The two kernels that measure what the chip gives a kernel that only reads and one that only multiplies:
+    between a fifth of the vendor's figures and the figures themselves."""
+    hbm = ops().measured_hbm_read(DEV, nbytes=1 << 30)
+    assert 1.6e12 < hbm < 8.0e12, hbm
+    mfma = ops().measured_mfma_bf16(DEV)
+    assert 0.5e15 < mfma < 2.5e15, mfma
