@@ -116,6 +116,7 @@ struct Frags {
 template <int DT, int NT, bool P2, bool STREAM = false>
 struct Tile {
   static constexpr int KS = (DT + 1) / 2;  // 32-wide steps over the head dimension
+  static constexpr float LAZY = 6.f;       // weights up to 2^6 before the reference follows the maximum
   f32x4 o[NT][DT];
   float m[NT], l[NT];
   Pages<P2> pages;
@@ -236,9 +237,20 @@ struct Tile {
       for (int e = 1; e < 8; ++e) mx = fmaxf(mx, x[e]);
       mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m[t], mx);
-      const float m_use = m_new == -INFINITY ? 0.f : m_new;  // nothing visible yet: keep everything zero
-      const float mc = m_use * scale_log2e;
+      // m is the reference the weights are taken against, not the maximum itself: it follows the maximum only
+      // when that has risen by more than LAZY (in base-2 units) for some column of the wave (a uniform branch),
+      // so weights stay below 2^LAZY and the output is rescaled rarely. Counted on random scores: among the
+      // columns of a tile some maximum rises in most blocks, and every rise used to cost a multiplication of
+      // the whole output tile. The sums and the final division use the same reference: the result is the same.
+      if (__any((mx - m[t]) * scale_log2e > LAZY)) {  // m = -inf: any visible key moves it
+        const float m_new = fmaxf(m[t], mx);
+        const float alpha = m_new == m[t] ? 1.f : exp2_raw((m[t] - m_new) * scale_log2e);  // m = -inf: 0
+        l[t] *= alpha;
+#pragma unroll
+        for (int d = 0; d < DT; ++d) o[t][d] *= alpha;
+        m[t] = m_new;
+      }
+      const float mc = (m[t] == -INFINITY ? 0.f : m[t]) * scale_log2e;  // nothing visible yet: everything stays zero
       float ps_ = 0.f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
@@ -246,15 +258,6 @@ struct Tile {
         ps_ += p;
         pf[t][e] = (bf16)p;
       }
-      // the maximum rarely moves after the first blocks; the output is rescaled only when it did for
-      // some column of the wave (a uniform branch)
-      if (__any(m_new > m[t])) {
-        const float alpha = exp2_raw(fmaf(m[t], scale_log2e, -mc));  // m = -inf: 0
-        l[t] *= alpha;
-#pragma unroll
-        for (int d = 0; d < DT; ++d) o[t][d] *= alpha;
-      }
-      m[t] = m_new;
       l[t] += ps_;  // partial over this lane's keys; lane groups are summed at the end
     }
   }
