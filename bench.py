@@ -166,6 +166,15 @@ def main() -> int:
     nums = model_numbers(sizes, dbytes)
     max_b = max(a.batch, 1 if a.no_points else 64)
     page = 16
+    # the cache of max_b requests of the whole context must fit beside the weights: at long contexts the
+    # largest point is left out rather than the run refused
+    total_mem = torch.cuda.get_device_properties(0).total_memory
+    weight_mem = (nums["linear_params"] + 2 * nums["head_params"]) * dbytes
+    fits = int((0.85 * total_mem - weight_mem) // (CONTEXT * nums["kv_bytes_per_token"]))
+    if fits < a.batch:
+        print(f"the cache of {a.batch} requests of {CONTEXT} tokens does not fit this GPU beside the weights ({fits} do)")
+        return 2
+    max_b = min(max_b, fits)
     eng = Engine(config=cfg, seed=0, dtype=a.dtype, max_model_len=CONTEXT, max_num_seqs=max_b,
                  max_num_batched_tokens=PROMPT, block_size=page, num_blocks=max_b * CONTEXT // page + 64,
                  hip_graph=not a.no_hip_graph)
@@ -241,6 +250,8 @@ def main() -> int:
     points = {}
     if not a.no_points:
         for b in (1, 64):
+            if b > max_b:
+                continue
             d, _, _ = decode(b, a.steps, a.warmup)
             points[f"decode_b{b}"] = round(b / d, 1)
 

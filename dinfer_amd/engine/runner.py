@@ -222,8 +222,7 @@ class ModelRunner:
         if self.dtype != torch.bfloat16 or opt.gemm_tuning != "measured" or not blaslt.available() or not self.group_specs:
             return
         most = min(self.max_tokens, self.num_blocks * self.page_size, opt.max_num_seqs * opt.max_model_len)
-        bucket = gemm.ROW_BUCKET
-        sizes = sorted({min(t, most) for t in range(2 * bucket, most + bucket, bucket)}, reverse=True)
+        sizes = sorted({min(t, most) for t in gemm.row_buckets(most) if t > gemm.SMALL_M}, reverse=True)
         met = blaslt.worth_measuring_met
         with blaslt.measuring():
             for n, total in enumerate(sizes):

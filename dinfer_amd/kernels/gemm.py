@@ -33,10 +33,26 @@ MID_M = 64
 TALL = 2
 TALL_BYTES = 32 << 20
 
-# Rows of a library product are rounded up to a multiple of this where the caller allows it: a prompt portion
-# beside a changing number of decoding requests then meets a handful of shapes, each with its algorithm chosen
-# once, instead of a new shape every step.
-ROW_BUCKET = 32
+# Rows of a library product are rounded up where the caller allows it: a prompt portion beside a changing number of
+# decoding requests then meets a handful of shapes, each with its algorithm chosen once, instead of a new shape
+# every step. Up to 1,024 rows to a multiple of 32; beyond, in coarser steps (at most an eighth more rows), so that
+# the shapes an engine can meet stay a few dozen however large its step budget is.
+
+
+def row_bucket(m: int) -> int:
+    """The row count a product of m rows runs with where padding is allowed."""
+    step = 32 if m <= 1024 else 128 if m <= 4096 else 512 if m <= 16384 else 2048
+    return -(-m // step) * step
+
+
+def row_buckets(most: int) -> list:
+    """Every value row_bucket takes for 1 <= m <= most, ascending (the last may exceed `most`)."""
+    out, m = [], 1
+    while m <= most:
+        b = row_bucket(m)
+        out.append(b)
+        m = b + 1
+    return out
 
 _workspace: dict = {}   # device -> float32 buffer for partial sums
 _outgrown: list = []    # earlier, smaller buffers: graphs captured with them still write there
@@ -59,7 +75,7 @@ def _mid_workspace(dev, need: int) -> torch.Tensor | None:
 def _library(a, w, out, m, may_pad):
     if blaslt.available() and a.stride(1) == 1 and w.stride(1) == 1 and out.stride(1) == 1:
         # float32 out (logits at many positions): straight from the accumulators, as the few-row kernel gives them
-        rows = min(a.shape[0], out.shape[0], -(-m // ROW_BUCKET) * ROW_BUCKET) if may_pad else m
+        rows = min(a.shape[0], out.shape[0], row_bucket(m)) if may_pad else m
         return blaslt.matmul(a, w, out, rows)
     if out.dtype == torch.float32:
         tmp = torch.mm(a[:m], w.t())
@@ -129,7 +145,7 @@ def add_nt(a: torch.Tensor, w: torch.Tensor, stream: torch.Tensor, m: int) -> bo
     if not (a.is_cuda and a.dtype == torch.bfloat16 and stream.dtype == torch.bfloat16 and m > SMALL_M
             and not _tall(m, n, k) and blaslt.available() and a.stride(1) == 1 and w.stride(1) == 1 and stream.stride(1) == 1):
         return False
-    rows = min(a.shape[0], stream.shape[0], -(-m // ROW_BUCKET) * ROW_BUCKET)
+    rows = min(a.shape[0], stream.shape[0], row_bucket(m))
     blaslt.matmul(a, w, stream, rows, accumulate=True)
     return True
 

@@ -623,7 +623,7 @@ def _library_gemm_cases(gemm):
             for _ in range(2):                                   # the second call replays the choice of the first
                 gemm.matmul_nt(a, w, out, M, may_pad=pad)
             torch.testing.assert_close(out[:M].double(), want, rtol=2e-2, atol=2e-2, msg=lambda m_: f"{M}x{N}x{K} pad={pad}: {m_}")
-            last = -(-M // gemm.ROW_BUCKET) * gemm.ROW_BUCKET if pad else M
+            last = gemm.row_bucket(M) if pad else M
             assert bool((out[last:] == 7.0).all()), f"{M}x{N}x{K} pad={pad}: rows past {last} were written"
     assert any(p and p.tuned for p in blaslt._plans.values())        # the larger shapes above were measured
     assert any(p and not p.tuned for p in blaslt._plans.values())    # the tiny ones took the library's first suggestion
@@ -659,7 +659,7 @@ def _library_add_cases(gemm):
         start = torch.randn(M + 70, N, device=DEV).to(torch.bfloat16)
         prod = a[:M].double() @ w.double().T
         stream = start.clone()
-        last = -(-M // gemm.ROW_BUCKET) * gemm.ROW_BUCKET
+        last = gemm.row_bucket(M)
         for call in (1, 2):
             before = stream[:M].double()
             assert gemm.add_nt(a, w, stream, M)
