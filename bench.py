@@ -86,35 +86,50 @@ def serving(a, torch, Engine, SamplingParams, Qwen3Config) -> int:
     lengths = [rng.randint(512, 3072) for _ in range(n_req)]
     sp = (SamplingParams(max_tokens=out_len, temperature=0.7, top_k=50, top_p=0.9, presence_penalty=0.5, seed=3, ignore_eos=True)
           if a.sampled else SamplingParams(max_tokens=out_len, temperature=0.0, ignore_eos=True))
-    def run():
+    def run(phases=False):
         for n in lengths:   # new tokens every run: the prefix cache has nothing to offer
             eng.add_request([rng.randrange(cfg.vocab_size) for _ in range(n)], sp)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         steps = mixed = outs = 0
         t_mixed = 0.0
+        split = {"with_prompt_portions": {}, "decode_only": {}}
         while eng.has_unfinished():
+            if phases:
+                eng.measure_phases(True)
             ts = time.perf_counter()
             got = eng.step()
             steps += 1
             outs += sum(1 for o in got if o.token is not None)
-            if eng.runner.batch.num_tokens != eng.runner.batch.num_reqs:
+            is_mixed = eng.runner.batch.num_tokens != eng.runner.batch.num_reqs
+            if is_mixed:
                 mixed += 1
                 t_mixed += time.perf_counter() - ts
+            if phases:
+                acc = split["with_prompt_portions" if is_mixed else "decode_only"]
+                for k, v in eng.phases.items():
+                    acc[k] = acc.get(k, 0.0) + v
         torch.cuda.synchronize()
-        return time.perf_counter() - t0, steps, mixed, outs, t_mixed
+        if phases:
+            eng.measure_phases(False)
+            for acc in split.values():
+                n = max(acc.pop("steps", 0), 1)
+                for k in acc:
+                    acc[k] = round(acc[k] / n * 1e3, 3)
+        return time.perf_counter() - t0, steps, mixed, outs, t_mixed, split
 
-    # the first run pays for first uses: kernels load, product shapes are measured, graphs are captured
+    # the first run pays for first uses: kernels load, graphs are captured
     results = [run() for _ in range(max(1, a.runs))]
     cold = results[0][0]
-    dt, steps, mixed, outs, t_mixed = results[-1]
+    dt, steps, mixed, outs, t_mixed, _ = results[-1]
+    phase_ms = run(phases=True)[5]   # once more with the host's clock around every phase (ms a step); not the timed run
     ptoks = sum(lengths)
     print(json.dumps({
         "metric": f"tokens/s, prompt and output (Qwen3-{a.shape.upper()} shape, 32 requests, prompts 512-3072 in portions of 512, 256 outputs each)",
         "value": round((ptoks + outs) / dt, 1), "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True,
         "vs_baseline": None, "dtype": "bf16" if a.dtype == "bfloat16" else "fp32", "data": "synthetic",
         "seconds": round(dt, 3), "runs": len(results), "seconds_first_run": round(cold, 3), "prompt_tokens": ptoks, "output_tokens": outs, "output_tokens_per_s": round(outs / dt, 1),
-        "steps": steps, "steps_with_prompt_portions": mixed, "seconds_in_those": round(t_mixed, 3),
+        "steps": steps, "steps_with_prompt_portions": mixed, "seconds_in_those": round(t_mixed, 3), "phases_ms": phase_ms,
         "sampling": "temperature 0.7, top-k 50, top-p 0.9, presence penalty 0.5" if a.sampled else "greedy",
         "config": {"model": f"Qwen3-{a.shape.upper()} shape, random weights", "layers": sizes["num_hidden_layers"],
                    "requests": n_req, "token_budget": budget, "context": ctx, "parallelism": "single GPU"}}))

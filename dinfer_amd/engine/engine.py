@@ -122,7 +122,8 @@ class Engine:
         ph["steps"] += 1
         ev = self.runner.take_gpu_events()
         if ev is not None:
-            ph["gpu"] += ev[0].elapsed_time(ev[1]) * 1e-3                # the tokens are back: both events have passed
+            ev[1].synchronize()        # a step in which nobody samples has not waited for the device yet
+            ph["gpu"] += ev[0].elapsed_time(ev[1]) * 1e-3
         return outs
 
     def generate(self, prompts: list, sampling: SamplingParams | list | None = None) -> list[list[int]]:
