@@ -304,6 +304,37 @@ def test_attention_finds_one_far_key(kernel):
         assert (got[hk * (H // Hkv)] - vv[5, hk]).abs().max() < 0.1
 
 
+@pytest.mark.parametrize("kernel", ["plain", "flash", "decode"])
+@pytest.mark.parametrize("inside", [True, False], ids=["first_key_inside", "last_key_outside"])
+def test_attention_window_edge(kernel, inside):
+    """A window of W keys ends exactly W - 1 keys before the row: the key at that place is made to dominate the last
+    row's softmax and must decide the output; the key one place earlier, made to dominate instead, must not count
+    at all (with random scores one key more or less among 150 changes the output by less than the tolerance).
+    The edge lies in the middle of a 32-key block and of a page, and the window starts in another split."""
+    H, Hkv, D, page, W = 8, 2, 64, 16, 150
+    total = 700
+    pos = total - 1                                   # the last row's position
+    key = pos - W + 1 if inside else pos - W          # first key inside the window / last key outside it
+    hist, new = ([total - 1], [1]) if kernel != "flash" else ([total - 40], [40])
+    q, kc, vc, m, outs = paged_case(torch.bfloat16, H, Hkv, D, page, hist, new, seed=21, spike=(key, 3.0))
+    out = torch.zeros(new[0], H * D, device=DEV, dtype=torch.bfloat16)
+    geo = dict(scale=D ** -0.5, window=W, heads=H, kv_heads=Hkv, head_dim=D, page_size=page)
+    if kernel == "plain":
+        ops().attn_paged_ref(q, out, kc, vc, m["bt"], m["cu"], m["sl"], 1, new[0], **geo)
+    elif kernel == "flash":
+        ops().attn_flash(q, out, kc, vc, m["bt"], m["cu"], m["sl"], 1, new[0], new[0], **geo)
+    else:
+        part = torch.zeros(H * 7 * (D + 4), device=DEV)
+        ops().attn_decode(q, out, part, kc, vc, m["bt"], None, m["sl"], 1, 7, **geo)
+    want = expected_attention(outs, hist, D ** -0.5, W)
+    torch.testing.assert_close(out.double().cpu().view(-1, H, D), want, rtol=2e-2, atol=2e-2)
+    (qq, kk, vv) = outs[0]
+    got = out.double().cpu().view(-1, H, D)[-1]
+    for hk in range(Hkv):
+        near = (got[hk * (H // Hkv)] - vv[key, hk]).abs().max()
+        assert (near < 0.1) == inside, f"kv head {hk}: the spiked key {'does not decide' if inside else 'decides'} the output"
+
+
 # ---- sampling -------------------------------------------------------------------------------------
 def test_argmax_ties_to_lowest_index():
     V = 163841
