@@ -296,12 +296,15 @@ struct Tile {
   // A block's loads are issued right before its use and other waves hide the latency: reading a
   // block ahead was measured and does not pay (neither with a second set of registers nor by
   // refilling each fragment as soon as its last reader has issued).
+  // fence_last: the wave has stored the key and value at k_hi - 1 itself (other lanes than those that read them);
+  // before the last block is loaded, those stores are waited for.
   template <bool TWO_BODIES, class MaskFn>
   __device__ __forceinline__ void walk(const bf16x8 (&qf)[NT][KS], const int (&col_lo)[NT], const int (&col_hi)[NT],
-                                       MaskFn mask) {
+                                       MaskFn mask, bool fence_last = false) {
     Frags<DT> f;
 #pragma nounroll
     for (int kb = k_lo & ~31; kb < k_hi; kb += 32) {
+      if (fence_last && kb + 32 >= k_hi) __threadfence_block();
       if (!TWO_BODIES || mask(kb)) {
         load<true>(f, kb);
         compute<true>(f, qf, kb, col_lo, col_hi);
@@ -441,6 +444,97 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))
   }
 }
 
+// What the decode kernel does itself in a step of single rows only, so that no kernel runs between the q|k|v product
+// and the attention: the per-head norm of q and k, the rotation (pairs (i, i + D/2), whole head, angles of the row's
+// position), and the new key and value into their pages. Same arithmetic, in the same order, as qkv_post_vec_kernel.
+struct DecodePost {
+  const bf16* wq;        // gains of the q and k norms (null: no norm)
+  const bf16* wk;
+  float eps, w_offset;
+  const int32_t* pos;    // [rows] position of each row
+  const float* cos_sin;  // [positions][D]: cos of the D/2 angles, then sin (null: no rotation)
+  const int64_t* slots;  // [rows] block * page + offset of the new key; negative or null: nothing is written
+  const bf16* k_new;     // the rows' new keys and values, [rows, ld_q] like q
+  const bf16* v_new;
+  bf16* k_cache;         // the same pages the kernel reads
+  bf16* v_cache;
+};
+
+// One head of D = 16 DT dims (DT % 4 == 0) in MFMA operand order: a lane holds the pieces d = 32 ks + 8 g4 .. + 8,
+// ks < KS, of the head its lane group of 16 selects; the partner of a pair lies KS / 2 pieces further in the same lane.
+// In three steps, so that the kernel can issue every load whose address it knows before it waits for any: load (the
+// head and the gains: addresses known at once), Angles::load (needs the position), finish (arithmetic only).
+template <int DT>
+struct HeadPost {
+  static constexpr int KS = DT / 2, D = DT * 16, HALF = D / 2;
+  struct Angles {
+    f32x4 c[KS / 2][2], s[KS / 2][2];
+    __device__ __forceinline__ void load(const float* cs) {
+      const int g4 = (threadIdx.x & 63) >> 4;
+#pragma unroll
+      for (int ks = 0; ks < KS / 2; ++ks) {
+        const int pi = ks * 32 + g4 * 8;
+        c[ks][0] = *(const f32x4*)(cs + pi);
+        c[ks][1] = *(const f32x4*)(cs + pi + 4);
+        s[ks][0] = *(const f32x4*)(cs + HALF + pi);
+        s[ks][1] = *(const f32x4*)(cs + HALF + pi + 4);
+      }
+    }
+  };
+  bf16x8 x[KS];
+  bf16x8 g[KS];  // the gains (bf16)
+
+  __device__ __forceinline__ void load(const bf16* src, bool active) {
+    const int g4 = (threadIdx.x & 63) >> 4;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) x[ks] = active ? *(const bf16x8*)(src + ks * 32 + g4 * 8) : zero8();
+  }
+  __device__ __forceinline__ void load_gains(const bf16* w) {
+    const int g4 = (threadIdx.x & 63) >> 4;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) g[ks] = *(const bf16x8*)(w + ks * 32 + g4 * 8);
+  }
+
+  // normed: gains were loaded; rotate: a holds the angles of the row's position
+  __device__ __forceinline__ void finish(const Angles& a, bool normed, float eps, float w_offset, bool rotate,
+                                         bf16x8 (&r)[KS]) const {
+    float inv = 1.f;
+    if (normed) {
+      float s[KS];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        s[ks] = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s[ks] = add_square(s[ks], (float)x[ks][e]);
+      }
+      // the sum of squares over the head's D / 8 pieces as a butterfly over the piece index, highest bit first
+#pragma unroll
+      for (int o = KS / 2; o > 0; o >>= 1)
+#pragma unroll
+        for (int ks = 0; ks < o; ++ks) s[ks] = s[ks] + s[ks + o];
+      float ss = s[0];
+      ss += __shfl_xor(ss, 32, 64);
+      ss += __shfl_xor(ss, 16, 64);
+      inv = 1.f / sqrtf(ss / (float)D + eps);
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS / 2; ++ks) {
+      const int k2 = ks + KS / 2;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float y1 = (float)x[ks][e], y2 = (float)x[k2][e];
+        if (normed) {
+          y1 = y1 * inv * ((float)g[ks][e] + w_offset);
+          y2 = y2 * inv * ((float)g[k2][e] + w_offset);
+        }
+        const float c = rotate ? a.c[ks][e >> 2][e & 3] : 1.f, sn = rotate ? a.s[ks][e >> 2][e & 3] : 0.f;
+        r[ks][e] = (bf16)rotated_first(y1, y2, c, sn);
+        r[k2][e] = (bf16)rotated_second(y1, y2, c, sn);
+      }
+    }
+  }
+};
+
 // The keys a request's row sees, [first, seq), are cut into `splits` equal parts of a multiple of
 // 32 keys; short requests leave the last parts empty. Computed alike by the decode and merge kernels.
 __device__ __forceinline__ void split_range(int seq, int window, int splits, int sp, int* k_lo, int* k_hi, int* kps) {
@@ -458,16 +552,23 @@ __device__ __forceinline__ void split_range(int seq, int window, int splits, int
 // meet in LDS and are combined there as attn_decode_merge_kernel combines them, so that kernel does not run.
 constexpr int JOIN_SPLITS = 4;
 
-template <int DT, bool P2, bool STREAM, bool JOIN = false>
-// (JOIN runs where requests are many and parts few: a CU holds 4 to 8 of its waves, registers are no limit there)
-__global__ void __launch_bounds__(JOIN ? 64 * JOIN_SPLITS : 64) __attribute__((amdgpu_waves_per_eu(JOIN ? 2 : 4, 8)))
+// POST: q arrives as the product left it; the kernel norms and rotates it on the way into its registers (every part
+// for itself: the head is 2 D bytes), and the wave whose part ends with the row's own position norms and rotates the
+// new key and stores it and the new value into their pages before it reads its last block.
+// (The pages are written through post.k_cache / v_cache and read through kc / vc: no __restrict__ on those.)
+template <int DT, bool P2, bool STREAM, bool JOIN = false, bool POST = false>
+// (JOIN runs where requests are many and parts few: a CU holds 4 to 8 of its waves, registers are no limit there;
+// POST without JOIN runs with about one wave per SIMD, and its prologue holds a head, gains and angles at once)
+__global__ void __launch_bounds__(JOIN ? 64 * JOIN_SPLITS : 64)
+__attribute__((amdgpu_waves_per_eu(JOIN || POST ? 2 : 4, 8)))
 attn_decode_kernel(
-    const bf16* __restrict__ q, int64_t ld_q, float* __restrict__ part, const bf16* __restrict__ kc,
-    const bf16* __restrict__ vc, const int32_t* __restrict__ block_table, int64_t max_blocks,
-    const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ seq_lens, int splits, float scale_log2e,
-    int window, int H, int Hkv, int ps, bf16* __restrict__ out = nullptr, int64_t ld_out = 0) {
+    const bf16* __restrict__ q, int64_t ld_q, float* __restrict__ part, const bf16* kc, const bf16* vc,
+    const int32_t* __restrict__ block_table, int64_t max_blocks, const int32_t* __restrict__ cu_seqlens,
+    const int32_t* __restrict__ seq_lens, int splits, float scale_log2e, int window, int H, int Hkv, int ps,
+    bf16* __restrict__ out = nullptr, int64_t ld_out = 0, DecodePost post = DecodePost{}) {
   constexpr int D = DT * 16;
   constexpr int KS = (DT + 1) / 2;
+  static_assert(!POST || DT % 4 == 0, "the fused norm and rotation keep both elements of a pair in one lane");
   const int sp = JOIN ? (int)(threadIdx.x >> 6) : (int)blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
   const int G = H / Hkv;
   int row = b;  // without cu_seqlens every request has exactly one row
@@ -475,28 +576,73 @@ attn_decode_kernel(
     row = cu_seqlens[b];
     if (cu_seqlens[b + 1] - row != 1) return;  // a longer run of rows belongs to the flash kernel
   }
-  int k_lo, k_hi, kps;
-  split_range(seq_lens[b], window, splits, sp, &k_lo, &k_hi, &kps);
-  // an empty part writes nothing; the merge kernel skips it by the same rule. (JOIN: it walks no block and
-  // leaves m = -inf, which weighs nothing; its wave must reach the barrier below.)
-  if (!JOIN && k_lo >= k_hi) return;
   const int lane = threadIdx.x & 63, i16 = lane & 15, g4 = lane >> 4;
   const int32_t* bt = block_table + (int64_t)b * max_blocks;
-
+  const bf16* qp = q + (int64_t)row * ld_q + (int64_t)(hk * G + (i16 < G ? i16 : 0)) * D;
+  int k_lo, k_hi, kps;
   bf16x8 qf[1][KS];
-  {
-    const int hh = i16 < G ? i16 : 0;
-    const bf16* qp = q + (int64_t)row * ld_q + (int64_t)(hk * G + hh) * D;
+  Tile<DT, 1, P2, STREAM> tl;
+  bool writer = false;
+  if constexpr (POST) {
+    // in the order of what is known when: the head, its gains, the row's position and slot at once; ...
+    HeadPost<DT> qh;
+    qh.load(qp, i16 < G);
+    if (post.wq) qh.load_gains(post.wq);
+    const int pos_row = post.cos_sin ? post.pos[row] : 0;
+    const int64_t slot = post.slots ? post.slots[row] : -1;
+    const int seq = seq_lens[b];
+    split_range(seq, window, splits, sp, &k_lo, &k_hi, &kps);
+    if (!JOIN && k_lo >= k_hi) return;
+    // ... with the length the block table, with the position the angles; the part that ends with the row's own
+    // position (wave-uniform) also takes the new key and value
+    tl.init(kc, vc, bt, (int)max_blocks, hk, Hkv, ps, k_lo, k_hi, scale_log2e);
+    typename HeadPost<DT>::Angles ang;
+    if (post.cos_sin) ang.load(post.cos_sin + (int64_t)pos_row * D);
+    writer = slot >= 0 && k_lo < k_hi && k_hi == seq;
+    qh.finish(ang, post.wq != nullptr, post.eps, post.w_offset, post.cos_sin != nullptr, qf[0]);
+    if (i16 >= G) {  // columns beyond the group stay zero whatever the norm made of nothing
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) qf[0][ks] = zero8();
+    }
+    if (writer) {
+      const int64_t blk = slot / ps;
+      const int off = (int)(slot - blk * ps);
+      const int64_t head = (blk * Hkv + hk) * (int64_t)ps * D;
+      // (asked for only now, when the registers of q's head are free: this part is on average half as long as the
+      // others, so its wave has the time)
+      HeadPost<DT> kh;
+      bf16x8 vv;
+      kh.load(post.k_new + (int64_t)row * ld_q + (int64_t)hk * D, i16 == 0);
+      if (post.wk) kh.load_gains(post.wk);
+      if (lane < D / 8) vv = *(const bf16x8*)(post.v_new + (int64_t)row * ld_q + (int64_t)hk * D + lane * 8);
+      bf16x8 kr[KS];
+      kh.finish(ang, post.wk != nullptr, post.eps, post.w_offset, post.cos_sin != nullptr, kr);
+      if (i16 == 0) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+          *(bf16x8*)(post.k_cache + head + k_page_offset(off, ks * 32 + g4 * 8, ps)) = kr[ks];
+      }
+      if (lane < D / 8) {  // V pages are transposed: the 8 dims of a piece go to 8 rows of keys
+        bf16* vd = post.v_cache + head + (int64_t)(lane * 8) * ps + off;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) vd[(int64_t)e * ps] = vv[e];
+      }
+    }
+  } else {
+    split_range(seq_lens[b], window, splits, sp, &k_lo, &k_hi, &kps);
+    // an empty part writes nothing; the merge kernel skips it by the same rule. (JOIN: it walks no block and
+    // leaves m = -inf, which weighs nothing; its wave must reach the barrier below.)
+    if (!JOIN && k_lo >= k_hi) return;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int d = ks * 32 + g4 * 8;
       qf[0][ks] = (d < D && i16 < G) ? *(const bf16x8*)(qp + d) : zero8();
     }
+    tl.init(kc, vc, bt, (int)max_blocks, hk, Hkv, ps, k_lo, k_hi, scale_log2e);
   }
   const int col_lo[1] = {k_lo}, col_hi[1] = {k_hi};
-  Tile<DT, 1, P2, STREAM> tl;
-  tl.init(kc, vc, bt, (int)max_blocks, hk, Hkv, ps, k_lo, k_hi, scale_log2e);
-  tl.template walk<false>(qf, col_lo, col_hi, [&](int kb) { return kb < k_lo || kb + 32 > k_hi; });
+  // (reading the first block before q is normed, or two blocks ahead, was measured at 1 and 8 requests: no gain)
+  tl.template walk<false>(qf, col_lo, col_hi, [&](int kb) { return kb < k_lo || kb + 32 > k_hi; }, writer);
   const float lt = tl.sum_l(0);
   if constexpr (JOIN) {
     __shared__ __attribute__((aligned(16))) float joined[JOIN_SPLITS][16][D + 4];
@@ -656,10 +802,11 @@ inline int compute_units() {
   return cached[dev];
 }
 
-template <int DT>
+template <int DT, bool POST>
 int launch_decode(const bf16* q, int64_t ld_q, bf16* out, int64_t ld_out, float* part, const bf16* kc, const bf16* vc,
                   const int32_t* bt, int64_t max_blocks, const int32_t* cu, const int32_t* sl, int num_reqs,
-                  int splits, float scale, int window, int H, int Hkv, int ps, hipStream_t stream) {
+                  int splits, float scale, int window, int H, int Hkv, int ps, const DecodePost& post,
+                  hipStream_t stream) {
   // many requests: the keys of a step exceed the caches and each is used once, so they are read past
   // them (measured at 64 requests of 2k-4k keys: 10% faster; at 8 or fewer, slightly slower)
   const bool p2 = (ps & (ps - 1)) == 0, stream_kv = num_reqs >= 32;
@@ -669,17 +816,22 @@ int launch_decode(const bf16* q, int64_t ld_q, bf16* out, int64_t ld_out, float*
     // lesser cost. Measured at 8 kv heads: 32, 56 and 64 requests gain 0.12 to 0.17 ms a step, 40 and 48 lose.
     const double per_cu = (double)Hkv * num_reqs / compute_units();
     if (splits <= JOIN_SPLITS && (per_cu <= 1. || ceil(per_cu) <= 1.15 * per_cu)) {
-      auto kernel = p2 ? (stream_kv ? attn_decode_kernel<DT, true, true, true> : attn_decode_kernel<DT, true, false, true>)
-                       : (stream_kv ? attn_decode_kernel<DT, false, true, true> : attn_decode_kernel<DT, false, false, true>);
+      auto kernel = p2 ? (stream_kv ? attn_decode_kernel<DT, true, true, true, POST>
+                                    : attn_decode_kernel<DT, true, false, true, POST>)
+                       : (stream_kv ? attn_decode_kernel<DT, false, true, true, POST>
+                                    : attn_decode_kernel<DT, false, false, true, POST>);
       kernel<<<dim3(1, (unsigned)Hkv, (unsigned)num_reqs), 64 * splits, 0, stream>>>(
-          q, ld_q, part, kc, vc, bt, max_blocks, cu, sl, splits, scale * LOG2E, window, H, Hkv, ps, out, ld_out);
+          q, ld_q, part, kc, vc, bt, max_blocks, cu, sl, splits, scale * LOG2E, window, H, Hkv, ps, out, ld_out, post);
       return launch_status();
     }
   }
-  auto kernel = p2 ? (stream_kv ? attn_decode_kernel<DT, true, true> : attn_decode_kernel<DT, true, false>)
-                   : (stream_kv ? attn_decode_kernel<DT, false, true> : attn_decode_kernel<DT, false, false>);
+  auto kernel = p2 ? (stream_kv ? attn_decode_kernel<DT, true, true, false, POST>
+                                : attn_decode_kernel<DT, true, false, false, POST>)
+                   : (stream_kv ? attn_decode_kernel<DT, false, true, false, POST>
+                                : attn_decode_kernel<DT, false, false, false, POST>);
   kernel<<<dim3((unsigned)splits, (unsigned)Hkv, (unsigned)num_reqs), 64, 0, stream>>>(
-      q, ld_q, part, kc, vc, bt, max_blocks, cu, sl, splits, scale * LOG2E, window, H, Hkv, ps, (bf16*)nullptr, (int64_t)0);
+      q, ld_q, part, kc, vc, bt, max_blocks, cu, sl, splits, scale * LOG2E, window, H, Hkv, ps, (bf16*)nullptr,
+      (int64_t)0, post);
   const int D = DT * 16;
   attn_decode_merge_kernel<<<dim3((unsigned)H, (unsigned)num_reqs), 64, 0, stream>>>(part, out, ld_out, cu, sl, splits,
                                                                                      window, H, D);
@@ -742,7 +894,49 @@ extern "C" int dinfer_attn_decode(const void* q, int64_t ld_q, void* out, int64_
       !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(part) || num_reqs > 65535 || kv_heads > 65535)
     return ERR_BAD_SHAPE;
   if ((int64_t)num_reqs * heads * splits * (head_dim + 4) > part_elems) return 5;
-  DINFER_DISPATCH_HEAD_DIM(head_dim, return launch_decode<DT>(
+  DINFER_DISPATCH_HEAD_DIM(head_dim, return (launch_decode<DT, false>(
       (const bf16*)q, ld_q, (bf16*)out, ld_out, part, (const bf16*)k_cache, (const bf16*)v_cache, block_table,
-      max_blocks, cu_seqlens, seq_lens, num_reqs, splits, scale, window, heads, kv_heads, page_size, stream));
+      max_blocks, cu_seqlens, seq_lens, num_reqs, splits, scale, window, heads, kv_heads, page_size, DecodePost{},
+      stream)));
+}
+
+// 1 if dinfer_attn_decode_post takes this head size (both elements of a rotated pair must lie in one lane).
+extern "C" int dinfer_attn_decode_post_supports(int head_dim) { return head_dim == 64 || head_dim == 128 || head_dim == 256; }
+
+// dinfer_attn_decode for a step in which every request brings exactly one row, with what otherwise runs as a kernel of
+// its own before it: q [rows, ld_q], k_new and v_new (rows of the same stride) come as the q|k|v product left them.
+// q and k get their per-head RMSNorm (gains q_gain and k_gain of head_dim bf16 elements; null: none) and are
+// rotated by the angles of positions[row] (cos_sin [positions, head_dim] float: cos of the head_dim / 2 angles, then
+// sin; pairs (i, i + head_dim / 2); null: no rotation); the new key and value go to slot_mapping[row] of the pages
+// (null or negative: nowhere; then the pages must already hold them). q, k_new and v_new are left as they were.
+extern "C" int dinfer_attn_decode_post(const void* q, const void* k_new, const void* v_new, int64_t ld_q, void* out,
+                                       int64_t ld_out, float* part, int64_t part_elems, void* k_cache, void* v_cache,
+                                       const int32_t* block_table, int64_t max_blocks, const int32_t* seq_lens,
+                                       int num_reqs, int splits, float scale, int window, int heads, int kv_heads,
+                                       int head_dim, int page_size, const void* q_gain, const void* k_gain,
+                                       float eps, float gain_offset, const int32_t* positions,
+                                       const float* cos_sin, const int64_t* slot_mapping, hipStream_t stream) {
+  if (num_reqs <= 0) return OK;
+  if (!dinfer_attn_mfma_supports(head_dim, page_size, heads, kv_heads) || !dinfer_attn_decode_post_supports(head_dim))
+    return ERR_UNSUPPORTED;
+  if (heads / kv_heads > 16) return ERR_UNSUPPORTED;
+  if (window < 0 || max_blocks <= 0 || splits <= 0 || splits > MAX_SPLITS || ld_q % 8 || !aligned16(q) ||
+      !aligned16(k_new) || !aligned16(v_new) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(part) ||
+      !aligned16(q_gain) || !aligned16(k_gain) || !aligned16(cos_sin) || num_reqs > 65535 || kv_heads > 65535 ||
+      (cos_sin && !positions) || (!q_gain != !k_gain))
+    return ERR_BAD_SHAPE;
+  if ((int64_t)num_reqs * heads * splits * (head_dim + 4) > part_elems) return 5;
+  DecodePost post{(const bf16*)q_gain, (const bf16*)k_gain, eps, gain_offset, positions, cos_sin, slot_mapping,
+                  (const bf16*)k_new, (const bf16*)v_new, (bf16*)k_cache, (bf16*)v_cache};
+  switch (head_dim) {
+    case 64: return launch_decode<4, true>((const bf16*)q, ld_q, (bf16*)out, ld_out, part, (const bf16*)k_cache,
+                                           (const bf16*)v_cache, block_table, max_blocks, nullptr, seq_lens, num_reqs,
+                                           splits, scale, window, heads, kv_heads, page_size, post, stream);
+    case 128: return launch_decode<8, true>((const bf16*)q, ld_q, (bf16*)out, ld_out, part, (const bf16*)k_cache,
+                                            (const bf16*)v_cache, block_table, max_blocks, nullptr, seq_lens, num_reqs,
+                                            splits, scale, window, heads, kv_heads, page_size, post, stream);
+    default: return launch_decode<16, true>((const bf16*)q, ld_q, (bf16*)out, ld_out, part, (const bf16*)k_cache,
+                                            (const bf16*)v_cache, block_table, max_blocks, nullptr, seq_lens, num_reqs,
+                                            splits, scale, window, heads, kv_heads, page_size, post, stream);
+  }
 }

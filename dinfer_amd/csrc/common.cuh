@@ -90,6 +90,21 @@ __device__ __forceinline__ float block_max(float v, float* red) {
 
 static inline int launch_status() { return hipGetLastError() == hipSuccess ? OK : ERR_LAUNCH; }
 
+// One rotated pair (a, b) -> (a cos - b sin, b cos + a sin) and one step of a sum of squares, with their roundings
+// spelled out: the kernels that norm and rotate a head (alone, or on the way into an attention kernel) must leave the
+// same bits, whatever the compiler would fuse in each of them.
+__device__ __forceinline__ float rotated_first(float a, float b, float c, float s) {
+#pragma clang fp contract(off)
+  const float t = b * s;
+  return __builtin_fmaf(a, c, -t);
+}
+__device__ __forceinline__ float rotated_second(float a, float b, float c, float s) {
+#pragma clang fp contract(off)
+  const float t = a * s;
+  return __builtin_fmaf(b, c, t);
+}
+__device__ __forceinline__ float add_square(float sum, float x) { return __builtin_fmaf(x, x, sum); }
+
 // K pages. One kv head of one page is [D / 8][page][8]: the 8-element pieces of consecutive keys lie
 // next to each other, so lanes that read the same piece of consecutive keys (the rows of an MFMA
 // operand) read contiguous memory. Needs D % 8 == 0. Offset of element d of the key at `off`:

@@ -285,7 +285,7 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_vec_kernel(
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
     x[e] = (float)xv[e];
-    ss += x[e] * x[e];
+    ss = add_square(ss, x[e]);
   }
   // every lane takes part in the cross-lane steps, whatever its head is
 #pragma unroll
@@ -300,7 +300,8 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_vec_kernel(
   const bool first = l < LPH / 2;  // this lane holds the first elements of its pairs
   bf16x8 r;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) r[e] = (bf16)(first ? y[e] * c[e] - other[e] * sn[e] : y[e] * c[e] + other[e] * sn[e]);
+  for (int e = 0; e < 8; ++e)
+    r[e] = (bf16)(first ? rotated_first(y[e], other[e], c[e], sn[e]) : rotated_second(other[e], y[e], c[e], sn[e]));
   if (is_q || !slots) {
     *(bf16x8*)(src + d0) = r;
   } else if (slot >= 0) {

@@ -30,6 +30,8 @@ class Workspace:
         self.split_k = self.mfma and heads // kv_heads <= 16
         self.part = None
         self.kv_heads = kv_heads
+        # a step of single rows: the split-K kernel can take the per-head norms, the rotation and the cache write along
+        self.decode_takes_post = self.split_k and ops.attn_decode_post_supports(head_dim)
         if self.split_k:
             max_units = max(self.splits(n) * n for n in range(1, ctx.max_reqs + 1)) * kv_heads
             elems = max_units * (heads // kv_heads) * (head_dim + 4)
@@ -38,6 +40,14 @@ class Workspace:
     def splits(self, num_reqs: int) -> int:
         """Parts per request: a function of the batch size only, so a captured graph stays valid."""
         return max(1, min(self.max_splits, TARGET_WAVES // (num_reqs * self.kv_heads)))
+
+
+def decode_with_post(qkv, out, k_cache, v_cache, batch, group: int, ws: Workspace, *, write: bool, **kw):
+    """A step in which every request brings one row (ws.decode_takes_post): norms, rotation, cache write and attention
+    in one kernel (and the merge of its parts). kw: geometry, norm and rotation as ops.attn_decode_post takes them."""
+    B = batch.num_reqs
+    return ops.attn_decode_post(qkv, out, ws.part, k_cache, v_cache, batch.block_table[group], batch.seq_lens, B,
+                                ws.splits(B), slot_mapping=batch.slot_mapping[group] if write else None, **kw)
 
 
 def paged_attention(qkv: torch.Tensor, out: torch.Tensor, k_cache, v_cache, batch, group: int, ws: Workspace, *,

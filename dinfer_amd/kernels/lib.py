@@ -41,6 +41,12 @@ SIGNATURES = {
         "attention",
         [_P, _L, _P, _L, _P, _L, _P, _P, _P, _L, _P, _P, _I, _I, _F, _I, _I, _I, _I, _I, _P],
     ),
+    "dinfer_attn_decode_post_supports": ("attention", [_I]),
+    "dinfer_attn_decode_post": (
+        "attention",
+        [_P, _P, _P, _L, _P, _L, _P, _L, _P, _P, _P, _L, _P, _I, _I, _F, _I, _I, _I, _I, _I, _P, _P, _F, _F, _P, _P,
+         _P, _P],
+    ),
     "dinfer_gemm_ref": ("gemm_ref", [_I, _I, _P, _L, _P, _L, _P, _L, _L, _L, _L, _P]),
     "dinfer_gemm_small_m": ("gemm", [_I, _P, _L, _P, _L, _P, _L, _L, _L, _L, _I, _I, _P]),
     "dinfer_gemm_small_m_gated": ("gemm", [_P, _L, _P, _L, _P, _L, _L, _L, _L, _I, _P]),

@@ -266,6 +266,39 @@ def attn_decode(q, out, part, k_cache, v_cache, block_table, cu_seqlens, seq_len
     return out
 
 
+def attn_decode_post_supports(head_dim: int) -> bool:
+    return bool(lib.get("dinfer_attn_decode_post_supports")(head_dim))
+
+
+def attn_decode_post(qkv, out, part, k_cache, v_cache, block_table, seq_lens, num_reqs: int, splits: int, *,
+                     scale: float, window: int, heads: int, kv_heads: int, head_dim: int, page_size: int, q_off: int,
+                     k_off: int, v_off: int, q_gain, k_gain, eps: float, gain_offset: float, positions, cos_sin,
+                     slot_mapping):
+    """attn_decode for a step in which every request brings one row, straight from the q|k|v product: the per-head
+    norms, the rotation (pairs (i, i + head_dim/2), the whole head) and the write of the new key and value into their
+    pages happen inside the attention kernel. qkv stays as the product left it. slot_mapping None: nothing is written."""
+    _need_gpu(qkv, out, part, k_cache, v_cache, block_table, seq_lens, q_gain, k_gain, positions, cos_sin, slot_mapping)
+    _check_paged(qkv, out, k_cache, v_cache, block_table, seq_lens, num_reqs, heads, kv_heads, head_dim, page_size)
+    assert part.dtype == torch.float32 and part.is_contiguous() and qkv.shape[0] >= num_reqs
+    assert max(q_off + heads * head_dim, k_off + kv_heads * head_dim, v_off + kv_heads * head_dim) <= qkv.shape[1]
+    assert q_off % 8 == 0 and k_off % 8 == 0 and v_off % 8 == 0
+    assert positions.dtype == torch.int32 and positions.numel() >= num_reqs
+    if q_gain is not None:   # (gains kept in 32-bit go through qkv_post)
+        assert k_gain is not None and q_gain.numel() == k_gain.numel() == head_dim
+        assert q_gain.dtype == k_gain.dtype == torch.bfloat16
+    if cos_sin is not None:
+        assert cos_sin.dtype == torch.float32 and cos_sin.is_contiguous() and cos_sin.shape[1] == head_dim
+    if slot_mapping is not None:
+        assert slot_mapping.dtype == torch.int64 and slot_mapping.numel() >= num_reqs
+    base, es = qkv.data_ptr(), qkv.element_size()
+    lib.call("dinfer_attn_decode_post", base + q_off * es, base + k_off * es, base + v_off * es, _rows(qkv),
+             out.data_ptr(), _rows(out), part.data_ptr(), part.numel(), k_cache.data_ptr(), v_cache.data_ptr(),
+             block_table.data_ptr(), block_table.shape[1], seq_lens.data_ptr(), num_reqs, splits, float(scale),
+             int(window), heads, kv_heads, head_dim, page_size, _ptr(q_gain), _ptr(k_gain), float(eps),
+             float(gain_offset), positions.data_ptr(), _ptr(cos_sin), _ptr(slot_mapping), _stream())
+    return out
+
+
 def gemm_ref(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int) -> torch.Tensor:
     """out[:m] = a[:m] @ w.T on the vector ALUs with float accumulation (true 32-bit for float operands)."""
     _need_gpu(a, w, out)

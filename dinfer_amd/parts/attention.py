@@ -90,6 +90,15 @@ class Attention(Mixer):
         no_norm = dict(q_gain=None, k_gain=None, eps=0.0, gain_offset=0.0)
         write = dict(k_cache=cache.k, v_cache=cache.v, slot_mapping=batch.slot_mapping[g] if cache.owner else None,
                      token_runs=batch.max_q_len >= 8)
+        if (pos.fused and batch.all_decode and self.attn_ws.decode_takes_post and pos.style == 0
+                and pos.rotary_dim == self.head_dim and (qn is None or qn.weight.dtype == torch.bfloat16)):
+            # only single rows: norm, rotation and cache write ride in the attention kernel, one launch fewer a layer
+            attn_kernels.decode_with_post(
+                self.qkv_buf, self.attn_buf, cache.k, cache.v, batch, g, self.attn_ws, write=cache.owner,
+                scale=self.scale, window=self.window or 0, heads=self.heads, kv_heads=self.kv_heads,
+                head_dim=self.head_dim, page_size=self.page_size, q_off=0, k_off=self.q_size,
+                v_off=self.q_size + self.kv_size, positions=batch.positions, cos_sin=pos.table(), **norm)
+            return self._project_out(T, into)
         if pos.fused:
             # per-head norm, rotation by the encoding's table and the cache write in one kernel
             ops.qkv_post(self.qkv_buf, T, **geometry, **norm, cos_sin=pos.table(), rotary_dim=pos.rotary_dim,
@@ -108,6 +117,9 @@ class Attention(Mixer):
             self.qkv_buf, self.attn_buf, cache.k, cache.v, batch, g, self.attn_ws, scale=self.scale,
             window=self.window or 0, heads=self.heads, kv_heads=self.kv_heads, head_dim=self.head_dim,
             page_size=self.page_size)
+        return self._project_out(T, into)
+
+    def _project_out(self, T, into):
         if into is not None:
             done = self.o.forward_into(self.attn_buf, into, T)
             if done is not None:

@@ -251,6 +251,73 @@ def test_attention_decode_split_k(H, Hkv, D, page, window):
         torch.testing.assert_close(out.double().cpu().view(-1, H, D), want, rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("gains", ["bf16", "none"])
+@pytest.mark.parametrize("window", [0, 100])
+@pytest.mark.parametrize("H,Hkv,D,page", [(16, 8, 128, 16), (5, 1, 64, 64), (16, 2, 256, 16), (8, 8, 64, 24)])
+def test_attention_decode_takes_norm_rotation_and_cache_write_along(H, Hkv, D, page, window, gains):
+    """A step of single rows straight from the q|k|v product: one kernel norms and rotates q and the new key, writes
+    key and value into their pages and attends. Against the plain functions, and against the two kernels it stands for
+    (whose page contents it must reproduce bit for bit). The slot of the new key holds stale content beforehand; one
+    request writes nothing (slot -1: its pages hold the key already)."""
+    theta, eps, scale = 1e4, 1e-5, D ** -0.5
+    # parts of several blocks, a part of one block (the store is waited for at once), a single key, many short ones
+    rng = random.Random(3)
+    for hist, splits in (([299, 69, 0, 1000], 7), ([rng.randrange(64) for _ in range(32)], 2),
+                         ([0, 45, 1000, 130], 4), ([100, 31, 32, 33], 1)):
+        B = len(hist)
+        _, kc, vc, m, outs = paged_case(torch.bfloat16, H, Hkv, D, page, hist, [1] * B, seed=11)
+        g = torch.Generator().manual_seed(B)
+        raw = torch.randn(B, (H + 2 * Hkv) * D, generator=g).to(torch.bfloat16)
+        wq = wk = None
+        if gains != "none":
+            wq = (torch.rand(D, generator=g) + 0.5).to(torch.bfloat16)
+            wk = (torch.rand(D, generator=g) + 0.5).to(torch.bfloat16)
+        pos = [h for h in hist]
+        table = rope_table(1024, D, theta).to(DEV)
+        slots = []
+        for b in range(B):
+            blk = int(m["bt"][b, hist[b] // page])
+            slots.append(blk * page + hist[b] % page)
+        slots[1] = -1
+        # what the plain functions make of the rows
+        x = raw.double()
+        ang = plain.rope_angles(pos, D, theta)
+        norm = (lambda t, w: plain.rms_norm(t, w.double(), eps)) if wq is not None else (lambda t, w: t)
+        q = plain.rope_neox(norm(x[:, :H * D].view(B, H, D), wq), ang).to(torch.bfloat16).double()
+        k = plain.rope_neox(norm(x[:, H * D:(H + Hkv) * D].view(B, Hkv, D), wk), ang).to(torch.bfloat16).double()
+        v = x[:, (H + Hkv) * D:].view(B, Hkv, D)
+        want_outs = []
+        for b, (_, kk, vv) in enumerate(outs):
+            kk, vv = kk.clone(), vv.clone()
+            if slots[b] >= 0:
+                kk[-1], vv[-1] = k[b], v[b]
+            want_outs.append((q[b:b + 1], kk, vv))
+        want = expected_attention(want_outs, hist, scale, window)
+        dev = lambda t: None if t is None else t.to(DEV)
+        args = dict(heads=H, kv_heads=Hkv, head_dim=D, page_size=page)
+        post = dict(q_off=0, k_off=H * D, v_off=(H + Hkv) * D, q_gain=dev(wq), k_gain=dev(wk), eps=eps, gain_offset=0.0,
+                    positions=torch.tensor(pos, dtype=torch.int32, device=DEV))
+        slot_t = torch.tensor(slots, dtype=torch.int64, device=DEV)
+        part = torch.full((B * H * splits * (D + 4),), float("nan"), device=DEV)
+        # the two kernels
+        kc2, vc2, qkv2 = kc.clone(), vc.clone(), raw.to(DEV)
+        out2 = torch.zeros(B, H * D, device=DEV, dtype=torch.bfloat16)
+        ops().qkv_post(qkv2, B, **args, **post, cos_sin=table, rotary_dim=D, rope_style=0, k_cache=kc2, v_cache=vc2,
+                       slot_mapping=slot_t, token_runs=False)
+        ops().attn_decode(qkv2, out2, part, kc2, vc2, m["bt"], None, m["sl"], B, splits, scale=scale, window=window,
+                          **args)
+        # the one
+        kc1, vc1, qkv1 = kc.clone(), vc.clone(), raw.to(DEV)
+        out1 = torch.zeros(B, H * D, device=DEV, dtype=torch.bfloat16)
+        part.fill_(float("nan"))
+        ops().attn_decode_post(qkv1, out1, part, kc1, vc1, m["bt"], m["sl"], B, splits, scale=scale, window=window,
+                               **args, **post, cos_sin=table, slot_mapping=slot_t)
+        assert torch.equal(qkv1.cpu(), raw), "the product's rows are left as they were"
+        assert torch.equal(vc1, vc2) and torch.equal(kc1, kc2), "the pages hold the same bits as after the two kernels"
+        torch.testing.assert_close(out1.double().cpu().view(-1, H, D), want, rtol=2e-2, atol=2e-2)
+        assert torch.equal(out1, out2), f"differs from the two kernels by {float((out1.float() - out2.float()).abs().max())}"
+
+
 @pytest.mark.parametrize("window", [0, 200])
 @pytest.mark.parametrize("H,Hkv,D,page", [(8, 2, 128, 16), (5, 5, 64, 8), (6, 1, 128, 24), (4, 2, 256, 16)])
 def test_attention_flash_long_portions(H, Hkv, D, page, window):
