@@ -55,6 +55,9 @@ FLAGS = [
     "-shared",
     "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the first kernel arguments arrive in scalar registers with the wave instead of by a load that every kernel's
+    # first addresses would wait for (a decode step is a chain of some 200 short kernels)
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
     "-Wno-unused-result",
 ]
 

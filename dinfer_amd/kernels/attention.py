@@ -14,6 +14,7 @@ from . import ops
 TARGET_WAVES = 1024   # split-K aims at about this many waves (measured: more, shorter waves cost more than they hide)
 MAX_SPLITS = 128      # the kernels take up to 256
 MIN_KEYS_PER_SPLIT = 512   # of the longest request the engine admits, beyond 32 parts
+SHORTEST_PART = 64         # keys of the longest request in one part, at least
 
 
 class Workspace:
@@ -26,6 +27,10 @@ class Workspace:
         # graph must stay valid), so it is bounded by the longest request the engine admits
         longest = ctx.max_seq_len or 4096
         self.max_splits = min(MAX_SPLITS, max(32, longest // MIN_KEYS_PER_SPLIT))
+        # an engine for short requests: no part shorter than 64 keys of the longest, so up to 256 keys there are at
+        # most four parts, which meet inside the workgroup and need no merge kernel (28 layers of 1,024 wide, 256
+        # keys: 1.17 -> 1.0x ms a step at one request)
+        self.max_splits = max(1, min(self.max_splits, -(-longest // SHORTEST_PART)))
         self.mfma = (ctx.dtype == torch.bfloat16 and ops.attn_mfma_supports(head_dim, ctx.page_size, heads, kv_heads))
         self.split_k = self.mfma and heads // kv_heads <= 16
         self.part = None
