@@ -32,6 +32,8 @@ def _engine_flags(p: argparse.ArgumentParser) -> None:
                    help="most prompt tokens of all requests per step (0: no limit)")
     p.add_argument("--no-hip-graph", "--no-cuda-graph", dest="no_graph", action="store_true",
                    help="run decode steps eagerly instead of replaying captured graphs")
+    p.add_argument("--no-async-scheduling", dest="no_async", action="store_true",
+                   help="plan each step only after the tokens of the one before have been read")
     p.add_argument("--gemm-tuning", choices=["measured", "heuristic"], default="measured",
                    help="library products: time the library's candidates once per shape at start-up and keep the "
                         "choices in a file (measured), or take its first suggestion (heuristic)")
@@ -46,7 +48,8 @@ def _options(a):
         gpu_memory_utilization=a.gpu_memory_utilization, decode_exempt_from_budget=not a.no_decode_exempt,
         enable_prefix_caching=a.prefix_caching,
         long_prefill_token_threshold=a.long_prefill_token_threshold,
-        prefill_tokens_per_step=a.prefill_tokens_per_step, hip_graph=not a.no_graph, device=a.device,
+        prefill_tokens_per_step=a.prefill_tokens_per_step, hip_graph=not a.no_graph, async_scheduling=not a.no_async,
+        device=a.device,
         gemm_tuning=a.gemm_tuning)
 
 

@@ -28,6 +28,10 @@ class EngineOptions:
     # of the reference implies (bins/dinfer/src/main.rs:30-131: the cache is on unless switched off)
     enable_prefix_caching: bool | None = None
     hip_graph: bool = True              # replay decode steps from captured HIP graphs
+    # while a step of single decode rows runs, the next one is planned and launched already (its input tokens stay on
+    # the device), and only then the running step's tokens are read: the host's work between two steps is hidden
+    # (the reference's engine does so by default too: crates/core/src/engine.rs:153-154,209)
+    async_scheduling: bool = True
     # bfloat16 products of more than 32 rows: the vendor library called directly (False: through torch.mm)
     gemm_library: bool = True
     # "measured": the engine's warm-up times the library's candidates once per shape, keeps the choices in

@@ -13,9 +13,16 @@ namespace {
 
 template <class S>
 __global__ void __launch_bounds__(256) embedding_kernel(const int32_t* __restrict__ ids, const S* __restrict__ table,
-                                                        S* __restrict__ out, int64_t vocab, int64_t width, int vec_ok) {
+                                                        S* __restrict__ out, int64_t vocab, int64_t width, int vec_ok,
+                                                        const int32_t* __restrict__ from,
+                                                        const int32_t* __restrict__ last) {
   const int64_t t = blockIdx.x;
+  // from[t] >= 0: the token is not known to the host yet, it is that one of the tokens the step before sampled
   int64_t id = ids[t];
+  if (from) {
+    const int32_t at = from[t];
+    if (at >= 0) id = last[at];
+  }
   if (id < 0 || id >= vocab) id = 0;
   const S* src = table + id * width;
   S* dst = out + t * width;
@@ -87,13 +94,16 @@ inline unsigned blocks_for(int64_t n, int per_block, unsigned cap) {
 
 }  // namespace
 
+// src, last (both or neither): where src[t] >= 0, token t's id is last[src[t]] instead of ids[t].
 extern "C" int dinfer_embedding(int dtype, const int32_t* ids, const void* table, void* out, int64_t tokens,
-                                int64_t vocab, int64_t width, hipStream_t stream) {
+                                int64_t vocab, int64_t width, const int32_t* src, const int32_t* last,
+                                hipStream_t stream) {
   if (tokens <= 0) return OK;
-  if (vocab <= 0 || width <= 0 || tokens > 0x7fffffff) return ERR_BAD_SHAPE;
+  if (vocab <= 0 || width <= 0 || tokens > 0x7fffffff || (!src != !last)) return ERR_BAD_SHAPE;
   DINFER_DISPATCH_DTYPE(dtype, {
     const bool vec = (width * sizeof(S)) % 16 == 0 && ((uintptr_t)table % 16 == 0) && ((uintptr_t)out % 16 == 0);
-    embedding_kernel<S><<<(unsigned)tokens, 256, 0, stream>>>(ids, (const S*)table, (S*)out, vocab, width, vec ? 1 : 0);
+    embedding_kernel<S><<<(unsigned)tokens, 256, 0, stream>>>(ids, (const S*)table, (S*)out, vocab, width, vec ? 1 : 0,
+                                                              src, last);
   });
   return launch_status();
 }

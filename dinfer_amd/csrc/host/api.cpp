@@ -252,6 +252,18 @@ int32_t dh_sched_schedule(void* sched, int32_t* n_out) {
         return 0;
     });
 }
+int32_t dh_sched_can_look_ahead(void* sched) {
+    return guarded([&] { return S(sched)->sched.can_look_ahead() ? 1 : 0; });
+}
+int32_t dh_sched_schedule_ahead(void* sched, int32_t* n_out) {
+    return guarded([&] {
+        const StepPlan& p = S(sched)->sched.schedule_ahead();
+        n_out[0] = static_cast<int32_t>(p.scheduled.size());
+        n_out[1] = static_cast<int32_t>(p.preempted.size());
+        n_out[2] = static_cast<int32_t>(p.force_finished.size());
+        return 0;
+    });
+}
 int32_t dh_sched_plan(void* sched, dh_scheduled* scheduled, int64_t* preempted, int64_t* finished_ids,
                       int32_t* finished_reasons) {
     const StepPlan& p = S(sched)->sched.plan();

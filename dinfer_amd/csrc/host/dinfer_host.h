@@ -59,6 +59,7 @@ typedef struct {
     int32_t* seq_lens;
     int32_t* state_slots;
     int32_t* logits_rows;
+    int32_t* feedback_src; /* per token: -1, or which of the last step's sampled tokens (on the device) it is */
     int64_t* slot_mapping[DH_MAX_GROUPS];
     int32_t* block_table[DH_MAX_GROUPS];
     int32_t max_blocks[DH_MAX_GROUPS];
@@ -97,6 +98,12 @@ int32_t dh_sched_request_info(void* sched, int64_t rid, dh_request_info* out);
 int32_t dh_sched_queue(void* sched, int32_t running, int64_t* out, int32_t capacity);  /* ids in queue order */
 /* plans a step; counts of the three lists go to n_out[3]; read them with dh_sched_plan */
 int32_t dh_sched_schedule(void* sched, int32_t* n_out);
+/* 1 if the next step can be planned while the last planned step still runs (before its dh_sched_update) */
+int32_t dh_sched_can_look_ahead(void* sched);
+/* plans that next step: every request of the running step that goes on decodes once more, its input token being
+ * the one the running step samples (a placeholder on the host; the batch names its place among those tokens).
+ * The next dh_sched_update is the running step's, the one after it this step's. */
+int32_t dh_sched_schedule_ahead(void* sched, int32_t* n_out);
 int32_t dh_sched_plan(void* sched, dh_scheduled* scheduled, int64_t* preempted, int64_t* finished_ids,
                       int32_t* finished_reasons);
 /* writes the planned step into the batch buffers straight from the requests' tokens */

@@ -57,6 +57,12 @@ struct Request {
     std::vector<int32_t> stop_ids;
     int32_t preemptions = 0;
     int32_t num_cached = 0;  // tokens of the prompt found in the prefix cache at the last admission
+    // Look-ahead: the step that samples this request's next token is still running and the step after it is planned
+    // already. `tokens` then ends with a placeholder (-1) whose value that running step brings; pending_src is the
+    // place of this request among the running step's sampled tokens. ending: the running step's token is the
+    // request's last whatever it is (max_tokens or max_model_len), so no further step is planned for it.
+    int32_t pending = 0, pending_src = -1;
+    bool ending = false;
 
     int32_t num_tokens() const { return static_cast<int32_t>(tokens.size()); }
     int32_t num_output() const { return num_tokens() - num_prompt; }
@@ -69,10 +75,14 @@ struct Scheduled {
     int32_t samples;  // the step reaches the end of the known tokens, so a token is sampled
 };
 
+// (feedback: for each scheduled request, the place among the sampled tokens of the step before whose value its last
+// token is, or -1: known only where that step was still running when this one was planned)
 struct StepPlan {
     std::vector<Scheduled> scheduled;  // running first, then newly admitted
     std::vector<int64_t> preempted;
     std::vector<std::pair<int64_t, Reason>> force_finished;  // ended by the scheduler itself
+    std::vector<int32_t> feedback;
+    bool open = false;  // planned and not yet updated
 };
 
 struct UpdateResult {
@@ -138,9 +148,52 @@ public:
 
     // ---- one step
     const StepPlan& schedule() {
+        if (plan_.open || prev_.open)
+            throw Error(ERR_VALUE, "a planned step has not been updated (plan ahead with schedule_ahead)");
+        return plan(false);
+    }
+
+    // ---- looking one step ahead (in the manner of crates/core/src/sched/mod.rs:8-9,646-670,690-760: the next step
+    // is planned and launched while the last one still runs, with a placeholder for the token it will bring) ----
+    // Only the plain case is taken ahead: the running step feeds one token of every request and samples each, nobody
+    // waits, and every cache group has a free page for every running request, so the step ahead is "everyone decodes
+    // once more" and preempts nobody. Anything else is planned after the running step's update, as before.
+    bool can_look_ahead() const {
+        if (!plan_.open || prev_.open || !waiting_.empty() || plan_.scheduled.empty()) return false;
+        for (const Scheduled& s : plan_.scheduled)
+            if (s.num_new != 1 || !s.samples) return false;
+        for (int g = 0; g < cache_->num_groups(); ++g)
+            if (cache_->pool(g).num_free() < static_cast<int64_t>(running_.size())) return false;
+        return true;
+    }
+
+    const StepPlan& schedule_ahead() {
+        if (!can_look_ahead()) throw Error(ERR_VALUE, "this step cannot be planned ahead");
+        prev_ = std::move(plan_);
+        plan_ = StepPlan{};
+        int32_t k = 0;
+        for (const Scheduled& s : prev_.scheduled) {
+            const int32_t at = k++;  // every row of the running step samples
+            auto it = reqs_.find(s.id);
+            if (it == reqs_.end() || it->second->status != RUNNING) continue;
+            Request* r = it->second.get();
+            if (r->num_output() + 1 >= r->max_tokens || r->num_tokens() + 1 >= opt_.max_model_len) {
+                r->ending = true;
+                continue;
+            }
+            r->tokens.push_back(-1);
+            r->pending = 1;
+            r->pending_src = at;
+        }
+        return plan(true);
+    }
+
+private:
+    const StepPlan& plan(bool ahead) {
         plan_.scheduled.clear();
         plan_.preempted.clear();
         plan_.force_finished.clear();
+        plan_.feedback.clear();
         int64_t budget = opt_.max_num_batched_tokens;
         int64_t quota = opt_.prefill_tokens_per_step > 0 ? opt_.prefill_tokens_per_step : (int64_t(1) << 62);
         const size_t eligible = running_.size() + waiting_.size();
@@ -150,6 +203,10 @@ public:
         size_t i = 0;
         while (i < running_.size()) {
             Request* r = running_[i];
+            if (r->ending) {  // its last token is on its way
+                ++i;
+                continue;
+            }
             const int64_t remaining = r->num_tokens() - r->num_computed;
             const bool is_decode = remaining == 1 && r->num_computed > 0;
             const bool charged = !(opt_.decode_exempt_from_budget && is_decode);
@@ -170,6 +227,7 @@ public:
                     got = true;
                     break;
                 }
+                if (ahead) break;  // the running step reads everyone's pages: nobody is preempted under it
                 Request* victim = running_.back();
                 if (victim == r) {
                     if (running_.size() > 1) break;  // others hold the pages; try again next step, never preempt oneself
@@ -185,12 +243,13 @@ public:
             if (!got) break;
             plan_.scheduled.push_back({r->id, r->num_computed, static_cast<int32_t>(n),
                                        r->num_computed + n == r->num_tokens()});
+            plan_.feedback.push_back(r->pending && r->num_computed + n == r->num_tokens() ? r->pending_src : -1);
             if (charged) budget -= n;
             if (!is_decode) quota -= n;
             ++i;
         }
 
-        if (!preempted_any) {
+        if (!preempted_any && !ahead) {
             while (budget > 0 && !waiting_.empty() && static_cast<int>(running_.size()) < opt_.max_num_seqs) {
                 Request* r = waiting_.front();
                 if (!cache_->can_admit()) break;
@@ -217,6 +276,7 @@ public:
                 running_.push_back(r);
                 plan_.scheduled.push_back({r->id, r->num_computed, static_cast<int32_t>(n),
                                            r->num_computed + n == r->num_tokens()});
+                plan_.feedback.push_back(-1);
                 budget -= n;
                 quota -= n;
             }
@@ -226,29 +286,44 @@ public:
             Request* r = reqs_.at(s.id).get();
             if (r->status == RUNNING) r->num_computed = s.start + s.num_new;
         }
+        plan_.open = !plan_.scheduled.empty();
         return plan_;
     }
 
-    // sampled: one token for every scheduled request that samples, in the plan's order.
+public:
+
+    // sampled: one token for every scheduled request that samples, in the plan's order; of the oldest plan that is
+    // not updated yet (the running step's, where the next one was planned ahead).
     // Appends one result for every scheduled request that is still running.
     void update(const int32_t* sampled, int n_sampled, std::vector<UpdateResult>& results) {
+        StepPlan& p = prev_.open ? prev_ : plan_;
+        if (!p.open) return;  // an empty plan, or one that was updated already: nothing to apply
+        p.open = false;
         int k = 0;
-        for (const Scheduled& s : plan_.scheduled) {
+        for (const Scheduled& s : p.scheduled) {
             const int at = s.samples ? k++ : -1;
             auto it = reqs_.find(s.id);
-            if (it == reqs_.end() || it->second->status != RUNNING) continue;  // preempted or aborted meanwhile
+            if (it == reqs_.end() || it->second->status != RUNNING) continue;  // preempted, aborted or ended meanwhile
             Request* r = it->second.get();
-            cache_->release_passed(r->id, r->num_computed);
-            if (opt_.enable_prefix_caching) cache_->commit(r->id, r->tokens.data(), r->num_computed);
             int32_t tok = -1;
             Reason reason = NO_REASON;
             if (s.samples) {
                 if (at >= n_sampled) throw Error(ERR_VALUE, "fewer sampled tokens than sampling requests");
                 tok = sampled[at];
-                r->tokens.push_back(tok);
+                if (r->pending) {  // the step ahead was planned around this token: its placeholder gets its value
+                    r->tokens.back() = tok;
+                    r->pending = 0;
+                    r->pending_src = -1;
+                } else {
+                    r->tokens.push_back(tok);
+                }
                 reason = check_stop(*r, tok);
-                if (reason != NO_REASON) finish(r, reason);
             }
+            // (the tokens counted as computed may include the one a step ahead is computing now: what is released
+            // or committed here is used again only by steps launched later, which run after it)
+            cache_->release_passed(r->id, r->num_computed);
+            if (opt_.enable_prefix_caching) cache_->commit(r->id, r->tokens.data(), r->num_computed);
+            if (reason != NO_REASON) finish(r, reason);
             results.push_back({r->id, tok, reason});
         }
     }
@@ -261,7 +336,8 @@ public:
         for (const Scheduled& s : plan_.scheduled) {
             const Request* r = reqs_.at(s.id).get();
             want_store[i] = s.num_new - 1;
-            entries.push_back({s.id, s.start, s.num_new, r->tokens.data() + s.start, &want_store[i], s.samples ? 1 : 0});
+            entries.push_back({s.id, s.start, s.num_new, r->tokens.data() + s.start, &want_store[i], s.samples ? 1 : 0,
+                               plan_.feedback[i]});
             ++i;
         }
     }
@@ -299,7 +375,8 @@ private:
     std::deque<Request*> waiting_;
     std::vector<Request*> running_;
     std::unordered_map<int64_t, std::unique_ptr<Request>> reqs_;
-    StepPlan plan_;
+    StepPlan plan_;  // the newest plan
+    StepPlan prev_;  // the plan before it while that one's step still runs (open), else spent
 };
 
 }  // namespace dinfer

@@ -11,6 +11,7 @@
 //   block_table  [B, MB] per cache group, -1 where no page is held
 //   state_slots  [B]     the request's fixed-size state slot
 //   logits_rows  [R]     rows of the flat batch whose logits are wanted
+//   feedback_src [T]     -1, or: the token's id is the feedback_src-th token the last step sampled (still on the device)
 //
 // Padding (pad_to > B): a step of single rows that replays a captured graph of pad_to requests
 // is filled up with requests of one token at position 0 that write no cache slot (slot -1) and
@@ -36,6 +37,7 @@ struct BatchBuffers {
     int32_t* seq_lens;
     int32_t* state_slots;
     int32_t* logits_rows;
+    int32_t* feedback_src;
     int64_t* slot_mapping[MAX_GROUPS];
     int32_t* block_table[MAX_GROUPS];
     int32_t max_blocks[MAX_GROUPS];
@@ -53,6 +55,8 @@ struct EntryView {
     const int32_t* tokens;
     const int32_t* want;
     int32_t n_want;
+    int32_t feedback_src = -1;  // >= 0: the entry's last token is not known on the host yet; it is this one of the
+                                // tokens the last step samples (its id in `tokens` is a placeholder)
 };
 
 inline void fill_batch(const CacheManager& cache, const BatchBuffers& buf, const EntryView* entries, int n_entries,
@@ -80,7 +84,14 @@ inline void fill_batch(const CacheManager& cache, const BatchBuffers& buf, const
         const EntryView& e = entries[b];
         const int n = e.count;
         std::memcpy(buf.input_ids + t, e.tokens, sizeof(int32_t) * n);
-        for (int i = 0; i < n; ++i) buf.positions[t + i] = e.start + i;
+        for (int i = 0; i < n; ++i) {
+            buf.positions[t + i] = e.start + i;
+            buf.feedback_src[t + i] = -1;
+        }
+        if (e.feedback_src >= 0) {
+            buf.input_ids[t + n - 1] = 0;
+            buf.feedback_src[t + n - 1] = e.feedback_src;
+        }
         for (int g = 0; g < buf.n_groups; ++g) {
             const std::vector<int32_t>& tab = cache.block_table(e.rid, g);
             const int mb = buf.max_blocks[g];
@@ -114,6 +125,7 @@ inline void fill_batch(const CacheManager& cache, const BatchBuffers& buf, const
             throw Error(ERR_VALUE, "only a step of single rows that all want logits can be padded");
         for (int b = B; b < P; ++b) {
             buf.input_ids[b] = 0;
+            buf.feedback_src[b] = -1;
             buf.positions[b] = 0;
             buf.cu_seqlens[b + 1] = b + 1;
             buf.seq_lens[b] = 1;

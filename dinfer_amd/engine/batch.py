@@ -12,6 +12,8 @@ whole prompts, portions of prompts and single decoded tokens side by side
   block_table  [B, MB] int32 per cache group, -1 where no page is held
   state_slots  [B]   int32  the request's fixed-size state slot (padded rows: the spare slot max_reqs)
   logits_rows  [R]   int32  rows of the flat batch whose logits are wanted
+  feedback_src [T]   int32  -1, or: the token's id is not in input_ids but is the feedback_src-th of the tokens the
+                            step before sampled (last_tokens, on the device): a step planned before that one ended
 
 All of them live in one device allocation at fixed addresses and are filled by
 one host-to-device copy from one pinned buffer (crates/layers/src/exec.rs:338-467),
@@ -44,7 +46,8 @@ class StepBatch:
         layout = [("slot_mapping%d" % g, np.int64, (max_tokens,)) for g in range(len(max_blocks))]
         layout += [("input_ids", np.int32, (max_tokens,)), ("positions", np.int32, (max_tokens,)),
                    ("cu_seqlens", np.int32, (max_reqs + 1,)), ("seq_lens", np.int32, (max_reqs,)),
-                   ("state_slots", np.int32, (max_reqs,)), ("logits_rows", np.int32, (max(max_rows, 1),))]
+                   ("state_slots", np.int32, (max_reqs,)), ("logits_rows", np.int32, (max(max_rows, 1),)),
+                   ("feedback_src", np.int32, (max_tokens,))]
         layout += [("block_table%d" % g, np.int32, (max_reqs, mb)) for g, mb in enumerate(max_blocks)]
         off = 0
         spans = {}
@@ -65,13 +68,16 @@ class StepBatch:
         self.input_ids, self.positions = d["input_ids"], d["positions"]
         self.cu_seqlens, self.seq_lens = d["cu_seqlens"], d["seq_lens"]
         self.state_slots, self.logits_rows = d["state_slots"], d["logits_rows"]
+        self.feedback_src = d["feedback_src"]
+        # the tokens the last step sampled, one per sampling request in the step's order: the sampler writes them here
+        self.last_tokens = torch.zeros(max(max_rows, 1), dtype=torch.int32, device=device)
         self.slot_mapping = [d["slot_mapping%d" % g] for g in range(len(max_blocks))]
         self.block_table = [d["block_table%d" % g] for g in range(len(max_blocks))]
         # where the C++ core writes: addresses inside the pinned buffer
         self._buffers = native.BatchBuffers()
         bb = self._buffers
         bb.n_groups, bb.max_tokens, bb.max_reqs, bb.max_rows = len(max_blocks), max_tokens, max_reqs, max_rows
-        for name in ("input_ids", "positions", "cu_seqlens", "seq_lens", "state_slots", "logits_rows"):
+        for name in ("input_ids", "positions", "cu_seqlens", "seq_lens", "state_slots", "logits_rows", "feedback_src"):
             setattr(bb, name, self.h[name].ctypes.data)
         for g, mb in enumerate(max_blocks):
             bb.slot_mapping[g] = self.h["slot_mapping%d" % g].ctypes.data

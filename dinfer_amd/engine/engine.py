@@ -12,6 +12,7 @@ from __future__ import annotations
 
 import itertools
 import random
+import time
 from dataclasses import dataclass
 
 from ..config import EngineOptions
@@ -28,6 +29,16 @@ class StepOutput:
     token: int | None          # None: a portion of a prompt was computed, nothing sampled
     finished: bool
     finish_reason: str | None
+
+
+class _Ready:
+    """Tokens that are on the host already, in the shape of what Sampler.launch returns."""
+
+    def __init__(self, tokens):
+        self._tokens = tokens
+
+    def tokens(self):
+        return self._tokens
 
 
 class Engine:
@@ -48,7 +59,11 @@ class Engine:
         spec = self.runner.model.spec
         self.vocab_size = spec.vocab_size
         self.scheduler = Scheduler(self.options, self.runner.cache, spec.eos_token_ids)
-        self.sampler = Sampler(self.runner.device, self.runner.max_rows, spec.vocab_size)
+        # the sampled tokens land where the next step can take them from as its input, if it is launched before
+        # the host has read them
+        last = getattr(getattr(self.runner, "batch", None), "last_tokens", None)
+        self.sampler = Sampler(self.runner.device, self.runner.max_rows, spec.vocab_size, out=last)
+        self._running = None                # (plan, tokens on their way, device events) of the step in flight
         self._ids = itertools.count()
         self._seeds = random.Random()
         self.phases: dict | None = None     # see measure_phases
@@ -69,62 +84,81 @@ class Engine:
         self.sampler.forget(request_id)
 
     def has_unfinished(self) -> bool:
-        return self.scheduler.has_unfinished()
+        return self.scheduler.has_unfinished() or self._running is not None
 
     # ---- one step ------------------------------------------------------------------------------
     def step(self) -> list[StepOutput]:
-        if self.phases is not None:
-            return self._step_timed()
-        so = self.scheduler.schedule()
-        outs = [StepOutput(rid, None, True, reason) for rid, reason in so.force_finished]
-        if not len(so):
-            return outs
-        logits = self.runner.step_planned(self.scheduler, so)
-        rows = [(r.sampling, len(r.output_ids), r.prompt_ids, r.output_ids, r.seed, r.id) for r in so.sampling_requests()]
-        tokens = self.sampler.sample(logits, rows)
+        """Plans, runs and samples one step and returns what it brought. With async_scheduling, where that step is
+        one of single decode rows, the step after it is planned and launched before this one's tokens are read, and
+        stays in flight when this call returns (crates/core/src/engine.rs:538-729)."""
+        ph = self.phases
+        outs: list = []
+        if self._running is None:
+            outs = self._launch(ahead=False)
+            if self._running is None:
+                return outs               # nothing was scheduled
+        nxt = None
+        if self._may_look_ahead():
+            self._running, held = None, self._running
+            outs += self._launch(ahead=True)            # (a plan ahead ends nobody: nothing is added)
+            self._running, nxt = held, self._running
+        so, sampled, events = self._running
+        tokens = sampled.tokens()
+        t0 = time.perf_counter() if ph is not None else 0.0
         for r, tok, reason in self.scheduler.update(so, tokens):
             outs.append(StepOutput(r.id, tok, reason is not None, reason))
         for o in outs:
             if o.finished:
                 self.sampler.forget(o.request_id)
+        self._running = nxt
+        if ph is not None:
+            ph["update"] += time.perf_counter() - t0
+            ph["steps"] += 1
+            if events is not None:
+                events[1].synchronize()        # a step in which nobody samples has not waited for the device yet
+                ph["gpu"] += events[0].elapsed_time(events[1]) * 1e-3
+        return outs
+
+    def _may_look_ahead(self) -> bool:
+        """The step after the running one can be launched before the running one's tokens are read: the scheduler
+        can plan it (everyone decodes once more), and no row needs the token on the host to sample the next (a
+        penalty counts the tokens seen so far)."""
+        if not self.options.async_scheduling or not self.scheduler.can_look_ahead():
+            return False
+        return not any(r.sampling.has_penalties for r in self._running[0].requests)
+
+    def _launch(self, ahead: bool) -> list[StepOutput]:
+        """Plans a step and issues it and its sampling; what is in flight afterwards is in _running (None: nothing
+        was scheduled). Returns the outputs of requests the scheduler itself ended while planning."""
+        ph = self.phases
+        t0 = time.perf_counter() if ph is not None else 0.0
+        so = self.scheduler.schedule(ahead=ahead)
+        if ph is not None:
+            ph["schedule"] += time.perf_counter() - t0
+        outs = [StepOutput(rid, None, True, reason) for rid, reason in so.force_finished]
+        if not len(so):
+            self._running = None
+            return outs
+        logits = self.runner.step_planned(self.scheduler, so)          # adds to fill and launch itself
+        # a request whose last token is still on its way has produced one more than its list says
+        rows = [(r.sampling, len(r.output_ids) + (1 if ahead else 0), r.prompt_ids, r.output_ids, r.seed, r.id)
+                for r in so.sampling_requests()]
+        launch = getattr(self.sampler, "launch", None)                 # (a stand-in may only know how to sample())
+        sampled = launch(logits, rows) if launch else _Ready(self.sampler.sample(logits, rows))   # adds to sample (and wait)
+        self._running = (so, sampled, self.runner.take_gpu_events() if ph is not None else None)
         return outs
 
     def measure_phases(self, on: bool = True) -> None:
         """From now on every step adds its host times to `phases` (seconds; the reference accounts a step the same way,
         models/qwen3/src/executor.rs:150-157,734-748): schedule (the plan), fill (batch written and sent), launch
-        (graph replay or kernel launches issued), sample (sampling kernels issued), wait (the host waits for the tokens:
-        what the GPU still has to do once everything is issued), update (requests advanced, pages released), and
-        gpu (the model's kernels on the device, between two events); steps counts them."""
+        (graph replay or kernel launches issued), sample (sampling kernels issued), wait (from there until the host
+        has the tokens: what the GPU still had to do, and, where the next step was launched meanwhile, that work of
+        the host as well), update (requests advanced, pages released), and gpu (the model's kernels on the device,
+        between two events); steps counts them."""
         self.phases = {k: 0.0 for k in ("schedule", "fill", "launch", "sample", "wait", "update", "gpu")} if on else None
         if on:
             self.phases["steps"] = 0
         self.runner.phases = self.sampler.phases = self.phases
-
-    def _step_timed(self) -> list[StepOutput]:
-        import time
-        ph, t = self.phases, time.perf_counter
-        t0 = t()
-        so = self.scheduler.schedule()
-        ph["schedule"] += t() - t0
-        outs = [StepOutput(rid, None, True, reason) for rid, reason in so.force_finished]
-        if not len(so):
-            return outs
-        logits = self.runner.step_planned(self.scheduler, so)          # adds to fill and launch itself
-        rows = [(r.sampling, len(r.output_ids), r.prompt_ids, r.output_ids, r.seed, r.id) for r in so.sampling_requests()]
-        tokens = self.sampler.sample(logits, rows)                     # adds to sample and wait itself
-        t0 = t()
-        for r, tok, reason in self.scheduler.update(so, tokens):
-            outs.append(StepOutput(r.id, tok, reason is not None, reason))
-        for o in outs:
-            if o.finished:
-                self.sampler.forget(o.request_id)
-        ph["update"] += t() - t0
-        ph["steps"] += 1
-        ev = self.runner.take_gpu_events()
-        if ev is not None:
-            ev[1].synchronize()        # a step in which nobody samples has not waited for the device yet
-            ph["gpu"] += ev[0].elapsed_time(ev[1]) * 1e-3
-        return outs
 
     def generate(self, prompts: list, sampling: SamplingParams | list | None = None) -> list[list[int]]:
         """Runs the prompts (lists of token ids) to the end; returns the generated ids of each."""

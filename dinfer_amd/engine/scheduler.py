@@ -157,8 +157,16 @@ class Scheduler:
         return [self._by_number[h] for h in out[:n].tolist()]
 
     # ---- one step ------------------------------------------------------------------------------
-    def schedule(self) -> SchedulerOutput:
-        native.checked("dh_sched_schedule", self._h, self._counts)
+    def can_look_ahead(self) -> bool:
+        """The step planned last has not been updated yet (it is running), and the one after it can be planned now:
+        it feeds one token of every request and samples each, nobody waits to be admitted, and pages are at hand, so
+        the next step is every request decoding once more (crates/core/src/sched/mod.rs:8-9,646-670)."""
+        return bool(native.checked("dh_sched_can_look_ahead", self._h))
+
+    def schedule(self, ahead: bool = False) -> SchedulerOutput:
+        """ahead: plan the step after the one that still runs (can_look_ahead()); each request's input token is then
+        the one the running step samples, a placeholder here. update() then applies to the running step first."""
+        native.checked("dh_sched_schedule_ahead" if ahead else "dh_sched_schedule", self._h, self._counts)
         n, n_pre, n_fin = self._counts
         rows = np.zeros(n, dtype=_SCHEDULED)
         pre = np.zeros(max(n_pre, 1), dtype=np.int64)

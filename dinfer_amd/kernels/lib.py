@@ -18,7 +18,7 @@ _F = c_float
 
 # function name -> (library, argument types). Every function returns an int status.
 SIGNATURES = {
-    "dinfer_embedding": ("elementwise", [_I, _P, _P, _P, _L, _L, _L, _P]),
+    "dinfer_embedding": ("elementwise", [_I, _P, _P, _P, _L, _L, _L, _P, _P, _P]),
     "dinfer_gated_act": ("elementwise", [_I, _I, _P, _P, _L, _L, _L, _P]),
     "dinfer_add_inplace": ("elementwise", [_I, _P, _P, _L, _P]),
     "dinfer_widen": ("elementwise", [_I, _P, _P, _L, _P]),

@@ -59,16 +59,21 @@ def _is_param_f32(w: torch.Tensor, act_dtype: torch.dtype) -> int:
     return 0
 
 
-def embedding(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out[t] = table[ids[t]]; ids int32 [T], table [V, W], out [T, W]."""
-    _need_gpu(ids, table, out)
+def embedding(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, src: torch.Tensor | None = None,
+              last: torch.Tensor | None = None) -> torch.Tensor:
+    """out[t] = table[ids[t]]; ids int32 [T], table [V, W], out [T, W]. src, last (int32, both or neither): where
+    src[t] >= 0 the id is last[src[t]], a token the step before sampled, which only the device knows so far."""
+    _need_gpu(ids, table, out, src, last)
     assert ids.dtype == torch.int32 and ids.is_contiguous()
+    assert (src is None) == (last is None)
+    if src is not None:
+        assert src.dtype == last.dtype == torch.int32 and src.numel() >= ids.numel()
     assert table.is_contiguous() and out.is_contiguous() and table.dtype == out.dtype
     T = ids.numel()
     V, W = table.shape
     assert out.shape[0] >= T and out.shape[1] == W
     lib.call("dinfer_embedding", dtype_code(table.dtype), ids.data_ptr(), table.data_ptr(), out.data_ptr(), T, V, W,
-             _stream())
+             _ptr(src), _ptr(last), _stream())
     return out
 
 

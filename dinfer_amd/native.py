@@ -17,7 +17,7 @@ _PI, _PL = POINTER(c_int32), POINTER(c_int64)
 class BatchBuffers(Structure):
     _fields_ = [("n_groups", _I), ("max_tokens", _I), ("max_reqs", _I), ("max_rows", _I),
                 ("input_ids", _P), ("positions", _P), ("cu_seqlens", _P), ("seq_lens", _P),
-                ("state_slots", _P), ("logits_rows", _P),
+                ("state_slots", _P), ("logits_rows", _P), ("feedback_src", _P),
                 ("slot_mapping", _P * MAX_GROUPS), ("block_table", _P * MAX_GROUPS),
                 ("max_blocks", _I * MAX_GROUPS)]
 
@@ -83,6 +83,8 @@ _SIGNATURES = {
     "dh_sched_request_info": (_I, [_P, _L, POINTER(RequestInfo)]),
     "dh_sched_queue": (_I, [_P, _I, _P, _I]),
     "dh_sched_schedule": (_I, [_P, _P]),
+    "dh_sched_can_look_ahead": (_I, [_P]),
+    "dh_sched_schedule_ahead": (_I, [_P, _P]),
     "dh_sched_plan": (_I, [_P, _P, _P, _P, _P]),
     "dh_sched_fill": (_I, [_P, POINTER(BatchBuffers), _I, POINTER(BatchFacts)]),
     "dh_sched_update": (_I, [_P, _P, _I, _P, _I]),

@@ -116,7 +116,8 @@ class DecoderModel:
         """Runs the batch's tokens through all run entries; returns float32 logits [num_rows, vocab]
         at batch.logits_rows (a view of a fixed buffer)."""
         T, R = batch.num_tokens, batch.num_rows
-        ops.embedding(batch.input_ids[:T], self.embed, self.hidden)
+        ops.embedding(batch.input_ids[:T], self.embed, self.hidden, getattr(batch, "feedback_src", None),
+                      getattr(batch, "last_tokens", None))
         pending = None
         for i, e in enumerate(self.run):
             # the input norm of the block that runs next, if that block lets the one before carry it

@@ -16,15 +16,40 @@ import torch
 from ..kernels import ops
 
 
+class Sampled:
+    """The tokens of one launch(): on their way to pinned host memory until tokens() has waited for them."""
+
+    def __init__(self, sampler, n: int, host, event, launched: float | None):
+        self._sampler, self._n, self._host, self._event, self._launched = sampler, n, host, event, launched
+
+    def tokens(self) -> list[int]:
+        if self._n == 0:
+            return []
+        self._event.synchronize()
+        ph = self._sampler.phases
+        if ph is not None and self._launched is not None:
+            import time
+            ph["wait"] += time.perf_counter() - self._launched
+        return self._host[:self._n].tolist()
+
+
 class Sampler:
-    def __init__(self, device, max_rows: int, vocab: int):
+    def __init__(self, device, max_rows: int, vocab: int, out: torch.Tensor | None = None):
+        """out: int32 [>= max_rows] on the device where the sampled tokens are to land (the engine names the buffer
+        that the next step may take its input tokens from); made here if absent."""
         self.device, self.max_rows, self.vocab = device, max_rows, vocab
-        self.out = torch.empty(max_rows, dtype=torch.int32, device=device)
+        self.out = out if out is not None else torch.empty(max_rows, dtype=torch.int32, device=device)
+        assert self.out.dtype == torch.int32 and self.out.numel() >= max_rows
+        # two launches may be in flight (a step planned ahead of the one that runs): what the host fills or reads
+        # alternates between two pinned buffers (made at the first launch)
+        self._tokens_host: list | None = None
+        self._read: list | None = None
+        self._turn = 0
         # made on first non-greedy use: [max_rows, vocab] float32 for rows that take the one-workgroup path,
-        # the kernels' scratch, and the rows' options (filled in pinned host memory, copied once per step)
+        # the kernels' scratch, and the rows' options (filled in pinned host memory, copied once per launch)
         self.work: torch.Tensor | None = None
         self.scratch: torch.Tensor | None = None
-        self.rows_host: torch.Tensor | None = None
+        self.rows_host: list | None = None
         self.rows_dev: torch.Tensor | None = None
         self.history: torch.Tensor | None = None   # [max_rows, vocab] int32, made on first use of a penalty
         self._slots: dict = {}                      # request -> [history slot, outputs already counted]
@@ -38,50 +63,54 @@ class Sampler:
         self.work = torch.empty((self.max_rows, self.vocab), dtype=torch.float32, device=self.device)
         self.scratch = torch.empty(ops.sample_scratch_bytes(self.max_rows, self.vocab), dtype=torch.uint8,
                                    device=self.device)
-        self.rows_host = torch.empty(nbytes, dtype=torch.uint8, pin_memory=True)
+        self.rows_host = [torch.empty(nbytes, dtype=torch.uint8, pin_memory=True) for _ in range(2)]
         self.rows_dev = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
-        self._rows_np = self.rows_host.numpy().view(ops.SAMPLE_ROW)
+        self._rows_np = [h.numpy().view(ops.SAMPLE_ROW) for h in self.rows_host]
 
     def sample(self, logits: torch.Tensor, rows: list) -> list[int]:
-        """rows: per logits row (SamplingParams, num_output_tokens, prompt_ids, output_ids, seed[, request]).
+        """launch() and the wait for its tokens in one."""
+        return self.launch(logits, rows).tokens()
+
+    def launch(self, logits: torch.Tensor, rows: list) -> Sampled:
+        """Issues the sampling of one token per logits row and the copy of the tokens to the host; returns at once.
+        rows: per logits row (SamplingParams, num_output_tokens, prompt_ids, output_ids, seed[, request]).
         request: any hashable name of the request, under which its history is kept from step to step
-        (forget() when it is over); without it a row with penalties sends its whole history every time."""
+        (forget() when it is over); without it a row with penalties sends its whole history every time.
+        At most two launches may be waiting for their tokens() at a time."""
+        import time
         R = len(rows)
         assert logits.shape[0] == R and R <= self.max_rows
         if R == 0:
-            return []
+            return Sampled(self, 0, None, None, None)
+        t0 = time.perf_counter() if self.phases is not None else None
+        if self._tokens_host is None:
+            self._tokens_host = [torch.empty(self.max_rows, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+            self._read = [torch.cuda.Event(), torch.cuda.Event()]
+        turn = self._turn
+        self._turn ^= 1
         if all(p.is_greedy and not p.has_penalties for p, *_ in rows):
-            if self.phases is not None:
-                return self._timed(lambda: ops.argmax(logits, self.out, R), R)
             ops.argmax(logits, self.out, R)
-            return self.out[:R].tolist()
-        if any(p.has_penalties for p, *_ in rows):
-            self._penalties(logits, rows)
-        self._buffers()
-        rec = self._rows_np
-        for i, (p, n_out, _prompt, _output, seed, *_key) in enumerate(rows):
-            rec[i] = (p.temperature, p.top_k, p.top_p, p.min_p, seed & 0xFFFFFFFFFFFFFFFF, n_out)
-        n = R * ops.SAMPLE_ROW.itemsize
-        # pinned memory the device may still be reading from the step before: this step's tokens were read
-        # back (tolist) before it returned, so that copy is done
-        self.rows_dev[:n].copy_(self.rows_host[:n], non_blocking=True)
-        any_filter = any(p.top_k > 0 or p.top_p < 1.0 for p, *_ in rows)
-        if self.phases is not None:
-            return self._timed(lambda: ops.sample_rows(logits, self.work, self.scratch, self.rows_dev, self.out, R,
-                                                       any_filter=any_filter), R)
-        ops.sample_rows(logits, self.work, self.scratch, self.rows_dev, self.out, R, any_filter=any_filter)
-        return self.out[:R].tolist()   # waits for the stream, and with it for the copy out of rows_host
-
-    def _timed(self, launch, R: int) -> list[int]:
-        """The last launches of sample() with the host's time split into issuing them and waiting for the tokens."""
-        import time
-        t0 = time.perf_counter()
-        launch()
-        t1 = time.perf_counter()
-        tokens = self.out[:R].tolist()
-        self.phases["sample"] += t1 - t0
-        self.phases["wait"] += time.perf_counter() - t1
-        return tokens
+        else:
+            if any(p.has_penalties for p, *_ in rows):
+                self._penalties(logits, rows)
+            self._buffers()
+            rec = self._rows_np[turn]
+            for i, (p, n_out, _prompt, _output, seed, *_key) in enumerate(rows):
+                rec[i] = (p.temperature, p.top_k, p.top_p, p.min_p, seed & 0xFFFFFFFFFFFFFFFF, n_out)
+            n = R * ops.SAMPLE_ROW.itemsize
+            # (the pinned buffer of this turn was last read by the launch before the last, whose tokens have been
+            # waited for since)
+            self.rows_dev[:n].copy_(self.rows_host[turn][:n], non_blocking=True)
+            any_filter = any(p.top_k > 0 or p.top_p < 1.0 for p, *_ in rows)
+            ops.sample_rows(logits, self.work, self.scratch, self.rows_dev, self.out, R, any_filter=any_filter)
+        host = self._tokens_host[turn]
+        host[:R].copy_(self.out[:R], non_blocking=True)
+        self._read[turn].record()
+        t1 = None
+        if t0 is not None:
+            t1 = time.perf_counter()
+            self.phases["sample"] += t1 - t0
+        return Sampled(self, R, host, self._read[turn], t1)
 
     def forget(self, key) -> None:
         """The request is over: its history slot is free again."""

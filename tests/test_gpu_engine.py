@@ -294,3 +294,46 @@ def test_random_workloads_equal_the_plain_continuations(seed, tmp_path):
         for _ in range(n):
             ids.append(int(plain.forward(cfg, w, ids)[-1].argmax()))
         assert got[rid] == ids[len(p):], f"request {rid} (prompt of {len(p)}): {got[rid]} != {ids[len(p):]}"
+
+
+@pytest.mark.parametrize("dtype,graph", [("float32", False), ("bfloat16", True), ("bfloat16", False)])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_steps_launched_ahead_give_the_same_tokens(model_dirs, name, dtype, graph):
+    """async_scheduling launches a decode step before the tokens of the one before it are read (its input tokens stay
+    on the device). Greedy and seeded sampling, ends by length and by a stop token nobody can foresee, requests that
+    arrive while others decode: token for token what the engine gives step by step (the same kernels on the same
+    inputs: equal, not close)."""
+    from dinfer_amd import SamplingParams
+    prompts = prompts_for(name, [5, 17, 33, 9, 3, 21], 11)
+
+    def run(ahead, stop=()):
+        eng = engine(model_dirs[name], name, dtype=dtype, hip_graph=graph, async_scheduling=ahead, max_num_seqs=4)
+        sps = [SamplingParams(max_tokens=n, temperature=t, top_k=k, seed=100 + i, ignore_eos=True, stop_token_ids=list(stop))
+               for i, (n, t, k) in enumerate([(24, 0.0, -1), (7, 0.8, -1), (30, 0.0, -1), (13, 1.0, 5), (1, 0.0, -1), (18, 0.7, -1)])]
+        ids = [eng.add_request(p, sp) for p, sp in zip(prompts[:4], sps[:4])]
+        got, reasons, steps, looked = {}, {}, 0, 0
+        while eng.has_unfinished():
+            if steps == 9:                       # two more arrive while the first four decode
+                ids += [eng.add_request(p, sp) for p, sp in zip(prompts[4:], sps[4:])]
+            looked += eng._running is not None   # a step was in flight when this call began
+            for o in eng.step():
+                if o.token is not None:
+                    got.setdefault(o.request_id, []).append(o.token)
+                if o.finished:
+                    reasons[o.request_id] = o.finish_reason
+            steps += 1
+            assert steps < 400
+        assert eng.runner.cache.num_free(0) == 128
+        eng.runner.cache.check()
+        return [got[i] for i in ids], [reasons[i] for i in ids], looked
+
+    plain_tokens, plain_reasons, none_ahead = run(False)
+    assert none_ahead == 0
+    ahead_tokens, ahead_reasons, looked = run(True)
+    assert looked > 15, "the decode steps were not launched ahead"
+    assert ahead_tokens == plain_tokens and ahead_reasons == plain_reasons
+    # a stop token in the middle of the longest output: that request ends while its next step is in flight already
+    stop = plain_tokens[2][11]
+    a, ra, _ = run(False, stop=[stop])
+    b, rb, _ = run(True, stop=[stop])
+    assert a == b and ra == rb and "stop" in ra

@@ -386,3 +386,156 @@ def test_portions_end_at_multiples_of_the_alignment():
     sched = step(s, {})[0]
     assert sched == [(1, 16)]                                # 20 -> 16; the 4 left hold no aligned portion
     assert step(s, {})[0] == [(1, 16)]
+
+
+# ---- planning one step ahead (crates/core/src/sched/mod.rs:8-9,646-670,690-760: placeholders for tokens on their way) ----
+def ahead_run(s, tokens_of, steps):
+    """Drives s with one step always planned ahead where that is allowed. tokens_of(request id, its output count)
+    gives the token a step samples. Returns {id: outputs} and how many steps were planned ahead."""
+    got, running, ahead_count = {}, None, 0
+    for _ in range(steps):
+        if running is None:
+            out = s.schedule()
+            if not len(out):
+                if not s.has_unfinished():
+                    break
+                continue
+            running = out
+        nxt = None
+        if s.can_look_ahead():
+            nxt = s.schedule(ahead=True)
+            ahead_count += 1
+            assert all(x.num_new == 1 and x.samples for x in nxt.scheduled) and not nxt.preempted
+            nxt = nxt if len(nxt) else None
+        toks = {r.id: tokens_of(r.id, len(got.get(r.id, []))) for r in running.sampling_requests()}
+        for r, tok, reason in s.update(running, toks):
+            if tok is not None:
+                got.setdefault(r.id, []).append(tok)
+        s.cache.check()
+        running = nxt
+    return got, ahead_count
+
+
+def plain_run(s, tokens_of, steps):
+    got = {}
+    for _ in range(steps):
+        if not s.has_unfinished():
+            break
+        out = s.schedule()
+        toks = {r.id: tokens_of(r.id, len(got.get(r.id, []))) for r in out.sampling_requests()}
+        for r, tok, reason in s.update(out, toks):
+            if tok is not None:
+                got.setdefault(r.id, []).append(tok)
+    return got
+
+
+def test_a_step_planned_ahead_feeds_the_token_that_is_on_its_way():
+    s = mk(8, 64, 32)
+    r1 = req(1, 10, 100)
+    s.add_request(r1)
+    out = s.schedule()
+    assert not s.can_look_ahead()                      # a prompt portion runs: not the plain case
+    s.update(out, {1: 7})
+    out = s.schedule()                                 # the first decode step, planned after its input was known
+    assert [(x.start, x.num_new) for x in out.scheduled] == [(10, 1)] and s.can_look_ahead()
+    nxt = s.schedule(ahead=True)
+    assert [(x.start, x.num_new, x.samples) for x in nxt.scheduled] == [(11, 1, True)]
+    assert s.request_info(r1).num_tokens == 12          # prompt, one output, one placeholder
+    assert not s.can_look_ahead()                       # two steps are out already
+    res = s.update(out, {1: 8})                         # the running step's token fills the placeholder
+    assert [(r.id, t, why) for r, t, why in res] == [(1, 8, None)] and r1.output_ids == [7, 8]
+    assert s.request_info(r1).num_tokens == 12
+    assert s.can_look_ahead()                           # now the plan ahead is the running one
+    res = s.update(nxt, {1: 9})
+    assert r1.output_ids == [7, 8, 9] and s.request_info(r1).num_tokens == 13
+    s.cache.check()
+
+
+def test_planned_ahead_gives_the_same_tokens_and_ends_as_step_by_step():
+    def tokens_of(rid, n):                              # request 2 meets the end-of-sequence token as its 6th
+        return 2 if (rid == 2 and n == 5) else 10 + rid + n
+    runs = []
+    for drive in (plain_run, lambda s, t, n: ahead_run(s, t, n)[0]):
+        s = mk(8, 64, 64)
+        for i, (plen, mx) in enumerate([(10, 9), (20, 30), (5, 4)], start=1):
+            s.add_request(req(i, plen, mx))
+        runs.append(drive(s, tokens_of, 100))
+        assert not s.has_unfinished() and s.cache.num_free() == 64
+        s.cache.check()
+    assert runs[0] == runs[1]
+    assert len(runs[0][1]) == 9 and runs[0][2][-1] == 2 and len(runs[0][2]) == 6 and len(runs[0][3]) == 4
+
+
+def test_a_request_that_ends_unforeseen_leaves_a_row_nobody_waits_for():
+    s = mk(8, 64, 32)
+    r1, r2 = req(1, 10, 100), req(2, 10, 100)
+    s.add_request(r1)
+    s.add_request(r2)
+    s.update(s.schedule(), {1: 5, 2: 5})
+    run = s.schedule()
+    nxt = s.schedule(ahead=True)
+    assert [x.request.id for x in nxt.scheduled] == [1, 2]
+    res = s.update(run, {1: 2, 2: 6})                   # request 1 samples the end-of-sequence token
+    assert [(r.id, why) for r, _, why in res] == [(1, STOP), (2, None)] and 1 not in s.requests
+    free = s.cache.num_free()
+    res = s.update(nxt, {1: 99, 2: 7})                  # its row in the step ahead was computed in vain
+    assert [(r.id, t) for r, t, _ in res] == [(2, 7)] and r1.output_ids == [5, 2] and r2.output_ids == [5, 6, 7]
+    assert s.cache.num_free() == free
+    s.cache.check()
+
+
+def test_no_step_is_planned_ahead_for_the_last_token_of_a_request():
+    s = mk(8, 64, 32)
+    r1, r2 = req(1, 10, 2), req(2, 10, 100)
+    s.add_request(r1)
+    s.add_request(r2)
+    s.update(s.schedule(), {1: 5, 2: 5})
+    run = s.schedule()
+    nxt = s.schedule(ahead=True)                        # request 1's second token is its last whatever it is
+    assert [x.request.id for x in nxt.scheduled] == [2]
+    res = s.update(run, {1: 6, 2: 6})
+    assert [(r.id, why) for r, _, why in res] == [(1, LENGTH), (2, None)]
+    s.update(nxt, {2: 7})
+    assert r2.output_ids == [5, 6, 7]
+    s.cache.check()
+
+
+def test_nothing_is_planned_ahead_when_someone_waits_or_pages_are_short():
+    s = mk(1, 64, 32)                                   # one request slot: the second request waits
+    s.add_request(req(1, 10, 100))
+    s.add_request(req(2, 10, 100))
+    s.update(s.schedule(), {1: 5})
+    s.schedule()
+    assert not s.can_look_ahead()
+    s = mk(8, 64, 3)                                    # three pages of 16: the prompts take two
+    s.add_request(req(1, 16, 100))
+    s.add_request(req(2, 15, 100))
+    s.update(s.schedule(), {1: 5, 2: 5})
+    out = s.schedule()                                  # request 1's decode takes the last free page
+    assert [x.request.id for x in out.scheduled] == [1, 2] and not out.preempted and s.cache.num_free() == 0
+    assert not s.can_look_ahead()                       # a step ahead might have to preempt: it waits
+
+
+def test_random_loads_planned_ahead_match_step_by_step():
+    import random
+    looked = 0
+    for seed in range(6):
+        rng = random.Random(seed)
+        spec = [(rng.randrange(1, 60), rng.randrange(1, 40)) for _ in range(rng.randrange(2, 10))]
+        stop_at = {i: rng.randrange(1, 40) for i in range(1, len(spec) + 1) if rng.random() < 0.4}
+        tokens_of = lambda rid, n: 2 if stop_at.get(rid) == n else 10 + (rid * 31 + n * 7) % 1000
+        blocks = rng.choice([8, 16, 64])
+        # the same engine sizes for both ways of driving
+        seqs, budget = rng.choice([2, 4, 8]), rng.choice([16, 64])
+        outs = []
+        for drive in (plain_run, ahead_run):
+            s = mk(seqs, budget, blocks)
+            for i, (plen, mx) in enumerate(spec, start=1):
+                s.add_request(req(i, plen, mx))
+            res = drive(s, tokens_of, 2000)
+            outs.append(res if drive is plain_run else res[0])
+            assert not s.has_unfinished() and s.cache.num_free() == blocks
+            s.cache.check()
+        assert outs[0] == outs[1], f"seed {seed}"
+        looked += res[1]
+    assert looked > 50                                  # the loads do spend most decode steps planned ahead
