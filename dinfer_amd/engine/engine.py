@@ -139,12 +139,16 @@ class Engine:
         if not len(so):
             self._running = None
             return outs
-        logits = self.runner.step_planned(self.scheduler, so)          # adds to fill and launch itself
+        greedy = all(r.sampling.is_greedy and not r.sampling.has_penalties for r in so.sampling_requests())
+        logits = self.runner.step_planned(self.scheduler, so, greedy=greedy)      # adds to fill and launch itself
         # a request whose last token is still on its way has produced one more than its list says
         rows = [(r.sampling, len(r.output_ids) + (1 if ahead else 0), r.prompt_ids, r.output_ids, r.seed, r.id)
                 for r in so.sampling_requests()]
         launch = getattr(self.sampler, "launch", None)                 # (a stand-in may only know how to sample())
-        sampled = launch(logits, rows) if launch else _Ready(self.sampler.sample(logits, rows))   # adds to sample (and wait)
+        if launch:      # adds to sample (and, later, to wait); a replayed graph may have found the best tokens already
+            sampled = launch(logits, rows, done=getattr(self.runner, "argmax_done", False))
+        else:
+            sampled = _Ready(self.sampler.sample(logits, rows))
         self._running = (so, sampled, self.runner.take_gpu_events() if ph is not None else None)
         return outs
 

@@ -89,7 +89,7 @@ class ModelRunner:
         top = min(options.max_num_seqs, self.max_rows, self.max_tokens)
         sizes = {1 << i for i in range(top.bit_length() + 1)} | {24, 40, 48, 56} | {3 << i for i in range(5, top.bit_length())}
         self._buckets = sorted({min(x, top) for x in sizes})
-        self._graphs: dict[int, torch.cuda.CUDAGraph] = {}
+        self._graphs: dict[tuple, torch.cuda.CUDAGraph] = {}   # (bucket, finds the best tokens itself) -> graph
         self.phases: dict | None = None     # Engine.measure_phases
         self._events = None
         self._graph_pool = None
@@ -258,20 +258,23 @@ class ModelRunner:
         single_rows = all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)
         return self._run(len(entries), single_rows, lambda pad: self.batch.fill(entries, self.cache, pad_to=pad))
 
-    def step_planned(self, scheduler, plan) -> torch.Tensor:
+    def step_planned(self, scheduler, plan, greedy: bool = False) -> torch.Tensor:
         """The same step function for the step a scheduler has just planned: the batch is written
         straight from the tokens and tables the host core holds. Logits come back for the
-        requests of the plan that sample, in the plan's order."""
+        requests of the plan that sample, in the plan's order.
+        greedy: every row will take its best token; a step that replays a graph then finds them itself
+        (batch.last_tokens, `argmax_done` says so afterwards), one launch and one gap fewer after the graph."""
         return self._run(len(plan), plan.single_rows_that_sample,
-                         lambda pad: self.batch.fill_planned(scheduler, pad_to=pad))
+                         lambda pad: self.batch.fill_planned(scheduler, pad_to=pad), greedy)
 
-    def _run(self, n: int, single_rows: bool, fill) -> torch.Tensor:
+    def _run(self, n: int, single_rows: bool, fill, greedy: bool = False) -> torch.Tensor:
         timed = self.phases is not None
         if timed:
             import time
             self._began = time.perf_counter()
+        self.argmax_done = False
         if self._graphs_allowed and single_rows and 0 < n <= self._buckets[-1]:
-            out = self._graph_step(n, fill)
+            out = self._graph_step(n, fill, greedy)
         else:
             self._send(fill, None)
             self._reset_fresh_slots()
@@ -299,7 +302,7 @@ class ModelRunner:
         ev, self._events = self._events, None
         return ev
 
-    def _graph_step(self, n: int, fill) -> torch.Tensor:
+    def _graph_step(self, n: int, fill, greedy: bool = False) -> torch.Tensor:
         """A step of single rows replays a HIP graph captured for its batch-size bucket
         (crates/layers/src/exec.rs:83-222, models/qwen3/src/executor.rs:995-1014). All step
         inputs live at fixed addresses; what varies between replays is their content."""
@@ -307,14 +310,21 @@ class ModelRunner:
         bucket = next(x for x in self._buckets if x >= n)
         self._send(fill, bucket)
         self._reset_fresh_slots()   # outside the graph: which slots are fresh changes from step to step
-        g = self._graphs.get(bucket)
+        greedy = greedy and bucket <= b.last_tokens.numel()
+        self.argmax_done = greedy
+        g = self._graphs.get((bucket, greedy))
         if g is not None:
             g.replay()
             return self.model.logits[:n]
         # The first step of a bucket runs eagerly (first-use initialisation must not happen under capture) and its
         # result is the step's result; the capture that follows records the same launches without running them.
         # Nothing is replayed in this step: a part with state of its own must see each step once.
-        self.model.forward(b, self.cache_views)
+        def forward():
+            logits = self.model.forward(b, self.cache_views)
+            if greedy:      # (padded rows find a token as well; nobody reads it)
+                ops.argmax(logits, b.last_tokens, bucket)
+
+        forward()
         torch.cuda.synchronize()
         g = torch.cuda.CUDAGraph()
         if self._capture_stream is None:
@@ -325,13 +335,13 @@ class ModelRunner:
             # by hand: torch's capture context would collect garbage and empty the allocator's cache first
             g.capture_begin(pool=self._graph_pool)
             try:
-                self.model.forward(b, self.cache_views)
+                forward()
             finally:
                 g.capture_end()
         torch.cuda.current_stream().wait_stream(side)
         if self._graph_pool is None:
             self._graph_pool = g.pool()
-        self._graphs[bucket] = g
+        self._graphs[(bucket, greedy)] = g
         return self.model.logits[:n]
 
     # ---- request bookkeeping shared by replay and tests ------------------------------------------

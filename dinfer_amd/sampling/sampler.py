@@ -71,11 +71,12 @@ class Sampler:
         """launch() and the wait for its tokens in one."""
         return self.launch(logits, rows).tokens()
 
-    def launch(self, logits: torch.Tensor, rows: list) -> Sampled:
+    def launch(self, logits: torch.Tensor, rows: list, done: bool = False) -> Sampled:
         """Issues the sampling of one token per logits row and the copy of the tokens to the host; returns at once.
         rows: per logits row (SamplingParams, num_output_tokens, prompt_ids, output_ids, seed[, request]).
         request: any hashable name of the request, under which its history is kept from step to step
         (forget() when it is over); without it a row with penalties sends its whole history every time.
+        done: the tokens are in `out` already (every row is greedy and the step found them itself).
         At most two launches may be waiting for their tokens() at a time."""
         import time
         R = len(rows)
@@ -89,8 +90,10 @@ class Sampler:
         turn = self._turn
         self._turn ^= 1
         if all(p.is_greedy and not p.has_penalties for p, *_ in rows):
-            ops.argmax(logits, self.out, R)
+            if not done:
+                ops.argmax(logits, self.out, R)
         else:
+            assert not done
             if any(p.has_penalties for p, *_ in rows):
                 self._penalties(logits, rows)
             self._buffers()

@@ -122,7 +122,7 @@ def test_engine_loop_with_a_stand_in_runner():
             self.cache = CacheManager([GroupSpec(4, 32)], 3)
             self.model, self.device, self.max_rows, self.steps = FakeModel, torch.device("cpu"), 3, []
 
-        def step_planned(self, scheduler, plan):
+        def step_planned(self, scheduler, plan, greedy=False):
             self.steps.append([(x.request.id, x.num_new, x.start) for x in plan.scheduled])
             rows = [(x.start + x.num_new) % 50 for x in plan.scheduled if x.samples]
             return torch.nn.functional.one_hot(torch.tensor(rows, dtype=torch.long), 50).float()
