@@ -228,9 +228,12 @@ class _Plan:
         self.asked = False   # True once the plan file was asked about this shape
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)   # the handle alone: building a Stream object costs 4 us a call
+
+
 def _run(handle, plan, algo, a, w, out, workspace, beta=_zero) -> None:
     """out = a . w^T + beta * out (the library reads and writes the same matrix)."""
-    stream = torch.cuda.current_stream(a.device).cuda_stream
+    stream = _raw_stream(a.device.index) if _raw_stream is not None else torch.cuda.current_stream(a.device).cuda_stream
     _ok(_lib.hipblasLtMatmul(handle, plan.desc, byref(_one), w.data_ptr(), plan.lw, a.data_ptr(), plan.la, byref(beta),
                              out.data_ptr(), plan.lc, out.data_ptr(), plan.lc, byref(algo), workspace.data_ptr(),
                              WORKSPACE_BYTES, stream), "matmul")
