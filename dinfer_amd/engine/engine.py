@@ -100,8 +100,10 @@ class Engine:
         nxt = None
         if self._may_look_ahead():
             self._running, held = None, self._running
-            outs += self._launch(ahead=True)            # (a plan ahead ends nobody: nothing is added)
-            self._running, nxt = held, self._running
+            try:
+                outs += self._launch(ahead=True)        # (a plan ahead ends nobody: nothing is added)
+            finally:                                    # whatever happened, the running step is still the running step
+                self._running, nxt = held, self._running
         so, sampled, events = self._running
         tokens = sampled.tokens()
         t0 = time.perf_counter() if ph is not None else 0.0
