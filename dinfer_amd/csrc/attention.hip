@@ -53,6 +53,8 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
+__device__ __forceinline__ int lane_of() { return threadIdx.x & 63; }
+
 // 2^x by the hardware instruction alone: results below 2^-126 become 0, which a softmax weight may
 __device__ __forceinline__ float exp2_raw(float x) { return __builtin_amdgcn_exp2f(x); }
 
@@ -341,8 +343,15 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))
   constexpr int D = DT * 16;
   constexpr int KS = (DT + 1) / 2;
   constexpr int QW = 16 * QT;  // query rows per workgroup
-  __shared__ f32x4 part_o[3][QT][DT][64];
-  __shared__ float part_m[3][QT][64], part_l[3][QT][64];
+  // what waves 1..3 hand to wave 0 (dynamic: three row tiles of head size 128 need more than the 64 KB a kernel
+  // may declare): part_o[3][QT][DT][64] of f32x4, then part_m and part_l [3][QT][64] of float
+  extern __shared__ __attribute__((aligned(16))) char flash_smem[];
+  f32x4* const part_o_ = (f32x4*)flash_smem;
+  float* const part_m_ = (float*)(flash_smem + sizeof(f32x4) * 3 * QT * DT * 64);
+  float* const part_l_ = part_m_ + 3 * QT * 64;
+  auto part_o = [&](int r, int t, int d) -> f32x4& { return part_o_[((r * QT + t) * DT + d) * 64 + lane_of()]; };
+  auto part_m = [&](int r, int t) -> float& { return part_m_[(r * QT + t) * 64 + lane_of()]; };
+  auto part_l = [&](int r, int t) -> float& { return part_l_[(r * QT + t) * 64 + lane_of()]; };
   // Block order: the head index runs fastest and visits kv heads round-robin, so that the
   // workgroups an XCD receives (linear id modulo 8) share kv heads, and with them the L2 lines
   // of K and V. Late query tiles (most keys) are issued first.
@@ -397,10 +406,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))
   if (wave > 0) {
 #pragma unroll
     for (int t = 0; t < QT; ++t) {
-      part_m[wave - 1][t][lane] = tl.m[t];
-      part_l[wave - 1][t][lane] = tl.l[t];
+      part_m(wave - 1, t) = tl.m[t];
+      part_l(wave - 1, t) = tl.l[t];
 #pragma unroll
-      for (int d = 0; d < DT; ++d) part_o[wave - 1][t][d][lane] = tl.o[t][d];
+      for (int d = 0; d < DT; ++d) part_o(wave - 1, t, d) = tl.o[t][d];
     }
   }
   __syncthreads();
@@ -412,7 +421,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))
     float mr[3], M = tl.m[t];
 #pragma unroll
     for (int r = 0; r < 3; ++r) {
-      mr[r] = part_m[r][t][lane];
+      mr[r] = part_m(r, t);
       M = fmaxf(M, mr[r]);
     }
     const float mc = (M == -INFINITY ? 0.f : M) * scale_log2e;
@@ -423,9 +432,9 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8))
 #pragma unroll
     for (int r = 0; r < 3; ++r) {
       const float ar = exp2_raw(fmaf(mr[r], scale_log2e, -mc));
-      lsum += part_l[r][t][lane] * ar;
+      lsum += part_l(r, t) * ar;
 #pragma unroll
-      for (int d = 0; d < DT; ++d) tl.o[t][d] += part_o[r][t][d][lane] * ar;
+      for (int d = 0; d < DT; ++d) tl.o[t][d] += part_o(r, t, d) * ar;
     }
     tl.l[t] = lsum;
     const float lt = tl.sum_l(t);
@@ -771,21 +780,39 @@ int launch_flash(const bf16* q, int64_t ld_q, bf16* out, int64_t ld_out, const b
   const bool p2 = (ps & (ps - 1)) == 0;
   // 32 rows per workgroup where the head size leaves room for two row tiles (registers, and the LDS the
   // waves meet in), and the portions are longer than one tile; otherwise 16
-  if (DT <= 8 && max_q_len > 16) {
+  auto lds_of = [](int qt) { return (size_t)3 * qt * 64 * (sizeof(f32x4) * DT + 2 * sizeof(float)); };
+  // 48 rows per workgroup at head size 128: every K and V fragment a wave loads serves three row tiles instead of two
+  // (the path on which loads return is what this kernel fills first), at 256 registers, still two waves a SIMD.
+  // It pays where the rows still make several rounds of workgroups over the chip (measured, 32 heads: 3,072 rows
+  // 135 -> 121 us, 8,192 rows 783 -> 642 us = 34 % of the MFMA peak, 32,768 rows 37 %; 2,048 rows, 1,376 workgroups, level; a portion
+  // of 512 rows behind 30,000 keys, 352 workgroups instead of 512, loses 17 %). Head size 64 gains nothing.
+  constexpr bool WIDE_OK = DT == 8;
+  const int64_t wide_blocks = (int64_t)((max_q_len + 47) / 48) * H * num_reqs;
+  if (WIDE_OK && wide_blocks >= 2000) {
+    constexpr int QT = WIDE_OK ? 3 : 1;
+    const int tiles = (max_q_len + 16 * QT - 1) / (16 * QT);
+    if (wide_blocks > 0x7fffffff) return ERR_UNSUPPORTED;
+    auto kernel = p2 ? attn_flash_kernel<DT, QT, true> : attn_flash_kernel<DT, QT, false>;
+    // (more than the 64 KB of LDS a launch may ask for without saying so)
+    if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_of(QT)) != hipSuccess)
+      return ERR_LAUNCH;
+    kernel<<<(unsigned)wide_blocks, 256, lds_of(QT), stream>>>(q, ld_q, out, ld_out, kc, vc, bt, max_blocks, cu, sl, tiles,
+                                                              sl2, window, H, Hkv, ps, skip_single);
+  } else if (DT <= 8 && max_q_len > 16) {
     constexpr int QT = DT <= 8 ? 2 : 1;
     const int tiles = (max_q_len + 16 * QT - 1) / (16 * QT);
     const int64_t blocks = (int64_t)tiles * H * num_reqs;
     if (blocks > 0x7fffffff) return ERR_UNSUPPORTED;
     auto kernel = p2 ? attn_flash_kernel<DT, QT, true> : attn_flash_kernel<DT, QT, false>;
-    kernel<<<(unsigned)blocks, 256, 0, stream>>>(q, ld_q, out, ld_out, kc, vc, bt, max_blocks, cu, sl, tiles, sl2,
-                                                 window, H, Hkv, ps, skip_single);
+    kernel<<<(unsigned)blocks, 256, lds_of(QT), stream>>>(q, ld_q, out, ld_out, kc, vc, bt, max_blocks, cu, sl, tiles, sl2,
+                                                         window, H, Hkv, ps, skip_single);
   } else {
     const int tiles = (max_q_len + 15) / 16;
     const int64_t blocks = (int64_t)tiles * H * num_reqs;
     if (blocks > 0x7fffffff) return ERR_UNSUPPORTED;
     auto kernel = p2 ? attn_flash_kernel<DT, 1, true> : attn_flash_kernel<DT, 1, false>;
-    kernel<<<(unsigned)blocks, 256, 0, stream>>>(q, ld_q, out, ld_out, kc, vc, bt, max_blocks, cu, sl, tiles, sl2,
-                                                 window, H, Hkv, ps, skip_single);
+    kernel<<<(unsigned)blocks, 256, lds_of(1), stream>>>(q, ld_q, out, ld_out, kc, vc, bt, max_blocks, cu, sl, tiles, sl2,
+                                                        window, H, Hkv, ps, skip_single);
   }
   return launch_status();
 }

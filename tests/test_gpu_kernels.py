@@ -332,6 +332,20 @@ def test_attention_flash_long_portions(H, Hkv, D, page, window):
     torch.testing.assert_close(out.double().cpu().view(-1, H, D), want, rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("window", [0, 300])
+def test_attention_flash_three_row_tiles_a_workgroup(window):
+    """Head size 128 with enough rows for several rounds of workgroups: 48 rows a workgroup (three row tiles share every
+    key and value fragment). Rows with and without history, a request that ends inside a tile, one shorter than a tile."""
+    H, Hkv, D, page = 16, 4, 128, 16
+    hist, new = [0, 100, 555, 31, 7, 0], [1000, 700, 300, 49, 120, 33]     # ceil(1000 / 48) x 16 heads x 6 requests = 2,016 workgroups
+    q, kc, vc, m, outs = paged_case(torch.bfloat16, H, Hkv, D, page, hist, new, seed=9)
+    out = torch.zeros(sum(new), H * D, device=DEV, dtype=torch.bfloat16)
+    ops().attn_flash(q, out, kc, vc, m["bt"], m["cu"], m["sl"], len(hist), sum(new), max(new), scale=D ** -0.5,
+                     window=window, heads=H, kv_heads=Hkv, head_dim=D, page_size=page)
+    want = expected_attention(outs, hist, D ** -0.5, window)
+    torch.testing.assert_close(out.double().cpu().view(-1, H, D), want, rtol=2e-2, atol=2e-2)
+
+
 @pytest.mark.parametrize("splits", [5, 3])   # parts merged by a kernel of their own, and inside the workgroup
 def test_attention_mixed_routes_single_rows_to_split_k(splits):
     H, Hkv, D, page = 16, 4, 128, 16
