@@ -332,11 +332,13 @@ def test_attention_flash_long_portions(H, Hkv, D, page, window):
     torch.testing.assert_close(out.double().cpu().view(-1, H, D), want, rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("page", [16, 24])
 @pytest.mark.parametrize("window", [0, 300])
-def test_attention_flash_three_row_tiles_a_workgroup(window):
+def test_attention_flash_three_row_tiles_a_workgroup(window, page):
     """Head size 128 with enough rows for several rounds of workgroups: 48 rows a workgroup (three row tiles share every
-    key and value fragment). Rows with and without history, a request that ends inside a tile, one shorter than a tile."""
-    H, Hkv, D, page = 16, 4, 128, 16
+    key and value fragment). Rows with and without history, a request that ends inside a tile, one shorter than a tile;
+    pages of a power of two and not."""
+    H, Hkv, D = 16, 4, 128
     hist, new = [0, 100, 555, 31, 7, 0], [1000, 700, 300, 49, 120, 33]     # ceil(1000 / 48) x 16 heads x 6 requests = 2,016 workgroups
     q, kc, vc, m, outs = paged_case(torch.bfloat16, H, Hkv, D, page, hist, new, seed=9)
     out = torch.zeros(sum(new), H * D, device=DEV, dtype=torch.bfloat16)
