@@ -157,10 +157,9 @@ class Engine:
     def measure_phases(self, on: bool = True) -> None:
         """From now on every step adds its host times to `phases` (seconds; the reference accounts a step the same way,
         models/qwen3/src/executor.rs:150-157,734-748): schedule (the plan), fill (batch written and sent), launch
-        (graph replay or kernel launches issued), sample (sampling kernels issued), wait (from there until the host
-        has the tokens: what the GPU still had to do, and, where the next step was launched meanwhile, that work of
-        the host as well), update (requests advanced, pages released), and gpu (the model's kernels on the device,
-        between two events); steps counts them."""
+        (graph replay or kernel launches issued), sample (sampling kernels issued), wait (the host stands still until
+        the tokens of the oldest step in flight are there), update (requests advanced, pages released), and gpu (the
+        model's kernels on the device, between two events); steps counts them."""
         self.phases = {k: 0.0 for k in ("schedule", "fill", "launch", "sample", "wait", "update", "gpu")} if on else None
         if on:
             self.phases["steps"] = 0

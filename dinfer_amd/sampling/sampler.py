@@ -25,11 +25,14 @@ class Sampled:
     def tokens(self) -> list[int]:
         if self._n == 0:
             return []
-        self._event.synchronize()
         ph = self._sampler.phases
-        if ph is not None and self._launched is not None:
+        if ph is None:
+            self._event.synchronize()
+        else:
             import time
-            ph["wait"] += time.perf_counter() - self._launched
+            t0 = time.perf_counter()
+            self._event.synchronize()
+            ph["wait"] += time.perf_counter() - t0     # what the host stands still for
         return self._host[:self._n].tolist()
 
 
