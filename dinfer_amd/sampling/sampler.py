@@ -19,8 +19,8 @@ from ..kernels import ops
 class Sampled:
     """The tokens of one launch(): on their way to pinned host memory until tokens() has waited for them."""
 
-    def __init__(self, sampler, n: int, host, event, launched: float | None):
-        self._sampler, self._n, self._host, self._event, self._launched = sampler, n, host, event, launched
+    def __init__(self, sampler, n: int, host, event):
+        self._sampler, self._n, self._host, self._event = sampler, n, host, event
 
     def tokens(self) -> list[int]:
         if self._n == 0:
@@ -85,7 +85,7 @@ class Sampler:
         R = len(rows)
         assert logits.shape[0] == R and R <= self.max_rows
         if R == 0:
-            return Sampled(self, 0, None, None, None)
+            return Sampled(self, 0, None, None)
         t0 = time.perf_counter() if self.phases is not None else None
         if self._tokens_host is None:
             self._tokens_host = [torch.empty(self.max_rows, dtype=torch.int32, pin_memory=True) for _ in range(2)]
@@ -112,11 +112,9 @@ class Sampler:
         host = self._tokens_host[turn]
         host[:R].copy_(self.out[:R], non_blocking=True)
         self._read[turn].record()
-        t1 = None
         if t0 is not None:
-            t1 = time.perf_counter()
-            self.phases["sample"] += t1 - t0
-        return Sampled(self, R, host, self._read[turn], t1)
+            self.phases["sample"] += time.perf_counter() - t0
+        return Sampled(self, R, host, self._read[turn])
 
     def forget(self, key) -> None:
         """The request is over: its history slot is free again."""
