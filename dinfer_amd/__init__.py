@@ -1,9 +1,9 @@
 """dinfer_amd: a small, whole LLM inference engine for one MI355X GPU."""
 from .config import EngineOptions
-from .sampling.params import SamplingParams
+from .sampling.params import SamplingParams, TokenLogprobs
 
 __version__ = "0.1.0"
-__all__ = ["Engine", "EngineOptions", "SamplingParams"]
+__all__ = ["Engine", "EngineOptions", "SamplingParams", "TokenLogprobs"]
 
 
 def __getattr__(name):

@@ -20,7 +20,8 @@
 //
 // Reference behaviour: crates/kernels/cuda/sampling.cu:13-56 (argmax),
 // :85-133 (top-k / top-p by threshold search), :137-157 (Philox), :159-263
-// (draw), :266-283 (fused order), :318-349 (penalties), :352-364 (min_p).
+// (draw), :266-283 (fused order), :318-349 (penalties), :352-364 (min_p),
+// :290-316 (logit_bias), :380-430 (log-probabilities of the chosen and the most probable tokens).
 #include "common.cuh"
 
 using namespace dinfer;
@@ -858,6 +859,83 @@ __global__ void __launch_bounds__(256) penalties_dense_kernel(float* __restrict_
   logits[(int64_t)blockIdx.y * ld + i] = v;
 }
 
+// ---- what a request may add to its logits, and what it may ask about the token that was chosen -------
+// entries [n][2] int32 = (row, token), vals [n]: logits[row][token] += val. A token occurs once a row.
+__global__ void __launch_bounds__(256) logit_bias_kernel(float* __restrict__ logits, int64_t ld,
+                                                         const int32_t* __restrict__ entries,
+                                                         const float* __restrict__ vals, int n, int rows, int vocab) {
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= n) return;
+  const int row = entries[2 * e], tok = entries[2 * e + 1];
+  if (row < 0 || row >= rows || tok < 0 || tok >= vocab) return;
+  logits[(int64_t)row * ld + tok] += vals[e];
+}
+
+constexpr int MAX_TOP = 32;
+
+// (value, index) pairs in falling order of value, rising index among equals: is (v, i) behind (pv, pi)?
+__device__ __forceinline__ bool behind(float v, int i, float pv, int pi) { return v < pv || (v == pv && i > pi); }
+
+// One workgroup a row; k_of[row] < 0: nothing is asked about the row. log-softmax of the row as it is given:
+// column 0 of out_ids / out_lp [rows][stride] takes the chosen token and its log-probability, columns 1..k the k
+// most probable tokens in falling order (equal values: lower index first), rank[row] the number of tokens
+// whose logit is larger than the chosen one's. The k best come from a tournament: every thread names the
+// best of its own entries, the workgroup picks among 1024 names, and only the thread whose entry won
+// looks for its next.
+__global__ void __launch_bounds__(BLOCK) logprobs_kernel(const float* __restrict__ logits, int64_t ld,
+                                                         const int32_t* __restrict__ chosen,
+                                                         const int32_t* __restrict__ k_of, int stride,
+                                                         int32_t* __restrict__ out_ids, float* __restrict__ out_lp,
+                                                         int32_t* __restrict__ rank, int vocab) {
+  __shared__ Red red;
+  __shared__ float fred[NWAVE];
+  const int b = blockIdx.x;
+  const int k = k_of[b] < stride - 1 ? k_of[b] : stride - 1;
+  if (k < 0) return;
+  const float* row = logits + (int64_t)b * ld;
+  int c = chosen[b];
+  c = c < 0 ? 0 : (c >= vocab ? vocab - 1 : c);
+  const float cv = row[c];
+  float best = -INFINITY;
+  int besti = 0x7fffffff, larger = 0;
+  for (int i = threadIdx.x; i < vocab; i += BLOCK) {
+    const float v = row[i];
+    better(best, besti, v, i);
+    larger += v > cv;
+  }
+  float top = 0.f;
+  int wi = block_argmax(best, besti, red, &top);
+  float sum = 0.f;
+  for (int i = threadIdx.x; i < vocab; i += BLOCK) sum += expf(row[i] - top);
+  sum = block_sum(sum, fred);
+  const float lse = top + logf(sum);
+  const float n_larger = block_sum((float)larger, fred);  // (a count below 2^24 is exact in a float)
+  int32_t* ids = out_ids + (int64_t)b * stride;
+  float* lps = out_lp + (int64_t)b * stride;
+  if (threadIdx.x == 0) {
+    ids[0] = c;
+    lps[0] = cv - lse;
+    rank[b] = (int)n_larger;
+  }
+  float wv = top;
+  for (int j = 0; j < k; ++j) {
+    if (j > 0) wi = block_argmax(best, besti, red, &wv);
+    if (threadIdx.x == 0) {
+      const bool none = wi == 0x7fffffff;  // fewer tokens than k
+      ids[1 + j] = none ? -1 : wi;
+      lps[1 + j] = none ? -INFINITY : wv - lse;
+    }
+    if (wi != 0x7fffffff && wi % BLOCK == (int)threadIdx.x) {  // the winner was this thread's: its next one
+      best = -INFINITY;
+      besti = 0x7fffffff;
+      for (int i = threadIdx.x; i < vocab; i += BLOCK) {
+        const float v = row[i];
+        if (behind(v, i, wv, wi)) better(best, besti, v, i);
+      }
+    }
+  }
+}
+
 }  // namespace
 
 extern "C" int dinfer_argmax(const float* logits, int64_t ld, int32_t* out, int64_t rows, int64_t vocab,
@@ -948,5 +1026,36 @@ extern "C" int dinfer_penalties_dense(float* logits, int64_t ld, const int32_t* 
     return ERR_BAD_SHAPE;
   const dim3 grid((unsigned)((vocab + 255) / 256), (unsigned)rows);
   penalties_dense_kernel<<<grid, 256, 0, stream>>>(logits, ld, history, (const PenaltyRow*)rows_packed, (int)vocab);
+  return launch_status();
+}
+
+
+// logits[row][token] += val for n entries (row, token) [n][2] int32 with vals [n] float (a request's logit_bias,
+// crates/kernels/cuda/sampling.cu:290-316 without the grammar mask). Tokens outside the vocabulary and rows
+// outside [0, rows) are ignored; a (row, token) pair must not occur twice.
+extern "C" int dinfer_logit_bias(float* logits, int64_t ld, const int32_t* entries, const float* vals, int64_t n,
+                                 int64_t rows, int64_t vocab, hipStream_t stream) {
+  if (n <= 0 || rows <= 0) return OK;
+  if (!logits || !entries || !vals || vocab <= 0 || ld < vocab || n > 0x7fffffff || rows > 0x7fffffff ||
+      vocab > 0x7fffffff)
+    return ERR_BAD_SHAPE;
+  logit_bias_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(logits, ld, entries, vals, (int)n, (int)rows,
+                                                                     (int)vocab);
+  return launch_status();
+}
+
+// Log-probabilities of the chosen tokens and of the k most probable ones per row (k_of[row], < 0: none asked,
+// at most stride - 1 <= 32), from the log-softmax of logits as given (the caller passes the logits the model
+// produced, before penalties and temperature): out_ids / out_lp [rows][stride], rank [rows]
+// (crates/kernels/cuda/sampling.cu:380-430).
+extern "C" int dinfer_logprobs(const float* logits, int64_t ld, const int32_t* chosen, const int32_t* k_of,
+                               int64_t stride, int32_t* out_ids, float* out_lp, int32_t* rank, int64_t rows,
+                               int64_t vocab, hipStream_t stream) {
+  if (rows <= 0) return OK;
+  if (!logits || !chosen || !k_of || !out_ids || !out_lp || !rank) return ERR_BAD_SHAPE;
+  if (vocab <= 0 || vocab > (1 << 24) || ld < vocab || rows > 0x7fffffff) return ERR_BAD_SHAPE;
+  if (stride < 1 || stride > MAX_TOP + 1) return ERR_UNSUPPORTED;
+  logprobs_kernel<<<(unsigned)rows, BLOCK, 0, stream>>>(logits, ld, chosen, k_of, (int)stride, out_ids, out_lp, rank,
+                                                        (int)vocab);
   return launch_status();
 }

@@ -29,6 +29,7 @@ class StepOutput:
     token: int | None          # None: a portion of a prompt was computed, nothing sampled
     finished: bool
     finish_reason: str | None
+    logprobs: object = None    # TokenLogprobs of the token, for a request that asked for them
 
 
 class _Ready:
@@ -39,6 +40,9 @@ class _Ready:
 
     def tokens(self):
         return self._tokens
+
+    def logprobs(self):
+        return [None] * len(self._tokens)
 
 
 class Engine:
@@ -63,7 +67,8 @@ class Engine:
         # the host has read them
         last = getattr(getattr(self.runner, "batch", None), "last_tokens", None)
         self.sampler = Sampler(self.runner.device, self.runner.max_rows, spec.vocab_size, out=last)
-        self._running = None                # (plan, tokens on their way, device events) of the step in flight
+        # the step in flight: (plan, tokens on their way, device events, the sampled rows' requests if any wants logprobs)
+        self._running = None
         self._ids = itertools.count()
         self._seeds = random.Random()
         self.phases: dict | None = None     # see measure_phases
@@ -72,6 +77,7 @@ class Engine:
     def add_request(self, prompt_ids: list, sampling: SamplingParams | None = None, request_id=None):
         sampling = sampling or SamplingParams()
         bad = [t for t in prompt_ids if not (isinstance(t, int) and 0 <= t < self.vocab_size)]
+        bad += [t for t in sampling.logit_bias if not 0 <= t < self.vocab_size]
         if bad:
             raise ValueError(f"token {bad[0]!r} is outside the vocabulary of {self.vocab_size}")
         rid = next(self._ids) if request_id is None else request_id
@@ -104,11 +110,14 @@ class Engine:
                 outs += self._launch(ahead=True)        # (a plan ahead ends nobody: nothing is added)
             finally:                                    # whatever happened, the running step is still the running step
                 self._running, nxt = held, self._running
-        so, sampled, events = self._running
+        so, sampled, events, asking = self._running
         tokens = sampled.tokens()
         t0 = time.perf_counter() if ph is not None else 0.0
+        about = {}
+        if asking is not None:      # the requests of the sampled rows, where one of them wants log-probabilities
+            about = {r.id: lp for r, lp in zip(asking, sampled.logprobs()) if lp is not None}
         for r, tok, reason in self.scheduler.update(so, tokens):
-            outs.append(StepOutput(r.id, tok, reason is not None, reason))
+            outs.append(StepOutput(r.id, tok, reason is not None, reason, about.get(r.id) if tok is not None else None))
         for o in outs:
             if o.finished:
                 self.sampler.forget(o.request_id)
@@ -141,17 +150,19 @@ class Engine:
         if not len(so):
             self._running = None
             return outs
-        greedy = all(r.sampling.is_greedy and not r.sampling.has_penalties for r in so.sampling_requests())
+        sampling = so.sampling_requests()
+        greedy = all(r.sampling.picks_largest_logit for r in sampling)
         logits = self.runner.step_planned(self.scheduler, so, greedy=greedy)      # adds to fill and launch itself
         # a request whose last token is still on its way has produced one more than its list says
         rows = [(r.sampling, len(r.output_ids) + (1 if ahead else 0), r.prompt_ids, r.output_ids, r.seed, r.id)
-                for r in so.sampling_requests()]
+                for r in sampling]
         launch = getattr(self.sampler, "launch", None)                 # (a stand-in may only know how to sample())
         if launch:      # adds to sample (and, later, to wait); a replayed graph may have found the best tokens already
             sampled = launch(logits, rows, done=getattr(self.runner, "argmax_done", False))
         else:
             sampled = _Ready(self.sampler.sample(logits, rows))
-        self._running = (so, sampled, self.runner.take_gpu_events() if ph is not None else None)
+        asking = sampling if any(r.sampling.logprobs is not None for r in sampling) else None
+        self._running = (so, sampled, self.runner.take_gpu_events() if ph is not None else None, asking)
         return outs
 
     def measure_phases(self, on: bool = True) -> None:
@@ -165,13 +176,17 @@ class Engine:
             self.phases["steps"] = 0
         self.runner.phases = self.sampler.phases = self.phases
 
-    def generate(self, prompts: list, sampling: SamplingParams | list | None = None) -> list[list[int]]:
-        """Runs the prompts (lists of token ids) to the end; returns the generated ids of each."""
+    def generate(self, prompts: list, sampling: SamplingParams | list | None = None, *,
+                 return_logprobs: bool = False):
+        """Runs the prompts (lists of token ids) to the end; returns the generated ids of each. return_logprobs:
+        returns (ids, logprobs) instead, logprobs[i] holding one TokenLogprobs per generated token of a request
+        that asked for them (SamplingParams.logprobs) and None otherwise."""
         params = sampling if isinstance(sampling, list) else [sampling or SamplingParams()] * len(prompts)
         if len(params) != len(prompts):
             raise ValueError("one SamplingParams per prompt, or one for all")
         ids = [self.add_request(p, sp) for p, sp in zip(prompts, params)]
         got = {i: [] for i in ids}
+        about = {i: [] for i in ids}
         idle = 0
         while self.has_unfinished():
             outs = self.step()
@@ -181,4 +196,7 @@ class Engine:
             for o in outs:
                 if o.token is not None and o.request_id in got:
                     got[o.request_id].append(o.token)
+                    about[o.request_id].append(o.logprobs)
+        if return_logprobs:
+            return [got[i] for i in ids], [about[i] if p.logprobs is not None else None for i, p in zip(ids, params)]
         return [got[i] for i in ids]

@@ -492,6 +492,36 @@ def penalties(logits: torch.Tensor, rows: int, ids: torch.Tensor, counts: torch.
              logits.shape[1], _stream())
 
 
+MAX_TOP_LOGPROBS = 32
+
+
+def logit_bias(logits: torch.Tensor, rows: int, entries: torch.Tensor, values: torch.Tensor) -> None:
+    """In place: logits[row, token] += value for entries [n, 2] int32 = (row, token) and values [n] float32.
+    A (row, token) pair occurs once."""
+    _need_gpu(logits, entries, values)
+    assert logits.dtype == torch.float32 and entries.dtype == torch.int32 and values.dtype == torch.float32
+    assert entries.is_contiguous() and entries.dim() == 2 and entries.shape[1] == 2
+    assert values.is_contiguous() and values.numel() == entries.shape[0] and logits.shape[0] >= rows
+    lib.call("dinfer_logit_bias", logits.data_ptr(), _rows(logits), entries.data_ptr(), values.data_ptr(),
+             entries.shape[0], rows, logits.shape[1], _stream())
+
+
+def logprobs(logits: torch.Tensor, chosen: torch.Tensor, top: torch.Tensor, out_ids: torch.Tensor,
+             out_lp: torch.Tensor, rank: torch.Tensor, rows: int) -> None:
+    """Per row r with top[r] >= 0, from the log-softmax of logits[r]: out_ids[r, 0], out_lp[r, 0] = chosen[r] and its
+    log-probability; columns 1..top[r] the most probable tokens, falling (equal values: lower index first);
+    rank[r] = how many tokens have a larger logit than the chosen one. out_ids / out_lp are [>= rows, stride] with
+    stride <= MAX_TOP_LOGPROBS + 1; top[r] is cut to stride - 1."""
+    _need_gpu(logits, chosen, top, out_ids, out_lp, rank)
+    assert logits.dtype == torch.float32 and out_lp.dtype == torch.float32
+    assert chosen.dtype == top.dtype == out_ids.dtype == rank.dtype == torch.int32
+    assert out_ids.is_contiguous() and out_lp.is_contiguous() and out_ids.shape == out_lp.shape and out_ids.dim() == 2
+    assert min(logits.shape[0], chosen.numel(), top.numel(), rank.numel(), out_ids.shape[0]) >= rows
+    lib.call("dinfer_logprobs", logits.data_ptr(), _rows(logits), chosen.data_ptr(), top.data_ptr(),
+             out_ids.shape[1], out_ids.data_ptr(), out_lp.data_ptr(), rank.data_ptr(), rows, logits.shape[1],
+             _stream())
+
+
 # ---- measured ceilings ---------------------------------------------------------------------------
 def measured_hbm_read(device, nbytes: int = 4 << 30, repeats: int = 3) -> float:
     """Bytes per second a kernel that only reads reaches on `nbytes` of device memory (far beyond the caches):

@@ -1,3 +1,3 @@
-from .params import GREEDY_EPS, SamplingParams
+from .params import GREEDY_EPS, SamplingParams, TokenLogprobs
 
-__all__ = ["GREEDY_EPS", "SamplingParams"]
+__all__ = ["GREEDY_EPS", "SamplingParams", "TokenLogprobs"]

@@ -1,12 +1,23 @@
 """Sampling options of a request: names, defaults and ranges of the reference's
 SamplingParams (crates/core/src/sample.rs:81-139, validate :157-205), without the
-text-level and server-level fields (stop strings, logprobs, logit_bias, grammar).
+text-level and server-level fields (stop strings, prompt_logprobs, grammar).
 """
 from __future__ import annotations
 
 from dataclasses import dataclass, field
 
 GREEDY_EPS = 1e-5  # temperature at or below this is greedy (sample.rs:143-145)
+MAX_LOGPROBS = 20      # sample.rs:184-188
+MAX_LOGIT_BIAS = 300   # entries, each in [-100, 100] (sample.rs:198-203)
+
+
+@dataclass
+class TokenLogprobs:
+    """What a request with `logprobs` gets beside every output token (crates/core/src/sampler.rs:156-166)."""
+    token_id: int
+    logprob: float       # log_softmax(the model's logits)[token_id]: before logit_bias, penalties and temperature
+    rank: int            # how many tokens have a larger logit (0: it is the most probable one)
+    top: list            # the k most probable (token id, logprob), falling
 
 
 @dataclass
@@ -23,10 +34,26 @@ class SamplingParams:
     seed: int | None = None        # None: drawn at admission
     stop_token_ids: list = field(default_factory=list)
     ignore_eos: bool = False
+    logprobs: int | None = None    # k: every output token comes with its log-probability, its rank and the k most
+                                   # probable tokens (0: only its own), from the logits the model produced
+    logit_bias: dict = field(default_factory=dict)   # token id -> what is added to its logit before anything else
+                                                     # (pairs (token, bias) are taken too)
+
+    def __post_init__(self):
+        pairs = list(self.logit_bias.items()) if isinstance(self.logit_bias, dict) else list(self.logit_bias)
+        as_dict = {int(t): float(b) for t, b in pairs}       # (keys may come as strings of digits)
+        if len(as_dict) != len(pairs):
+            raise ValueError("logit_bias names a token twice")
+        self.logit_bias = as_dict
 
     @property
     def is_greedy(self) -> bool:
         return self.temperature <= GREEDY_EPS
+
+    @property
+    def picks_largest_logit(self) -> bool:
+        """The token is the largest of the logits the model produced: nothing changes them on the way."""
+        return self.is_greedy and not self.has_penalties and not self.logit_bias
 
     @property
     def has_penalties(self) -> bool:
@@ -51,5 +78,14 @@ class SamplingParams:
             raise ValueError("max_tokens must be at least 1")
         if self.min_tokens > self.max_tokens:
             raise ValueError(f"min_tokens {self.min_tokens} > max_tokens {self.max_tokens}")
+        if self.logprobs is not None and not (0 <= self.logprobs <= MAX_LOGPROBS):
+            raise ValueError(f"logprobs must be in [0, {MAX_LOGPROBS}], got {self.logprobs}")
+        if len(self.logit_bias) > MAX_LOGIT_BIAS:
+            raise ValueError(f"logit_bias has {len(self.logit_bias)} entries, at most {MAX_LOGIT_BIAS}")
+        for t, b in self.logit_bias.items():
+            if not (isinstance(t, int) and t >= 0):
+                raise ValueError(f"logit_bias names {t!r}, which is no token id")
+            if not (-100.0 <= b <= 100.0):
+                raise ValueError(f"logit_bias[{t}] = {b} is outside [-100, 100]")
         if self.seed is not None and not (0 <= self.seed < 1 << 64):
             raise ValueError(f"seed must fit 64 unsigned bits, got {self.seed}")

@@ -14,13 +14,30 @@ import numpy as np
 import torch
 
 from ..kernels import ops
+from .params import MAX_LOGPROBS, TokenLogprobs
 
 
 class Sampled:
     """The tokens of one launch(): on their way to pinned host memory until tokens() has waited for them."""
 
-    def __init__(self, sampler, n: int, host, event):
+    def __init__(self, sampler, n: int, host, event, asked=None, about=None):
         self._sampler, self._n, self._host, self._event = sampler, n, host, event
+        self._asked, self._about = asked, about     # per row k or None; the pinned (ids, logprobs, rank) of the launch
+
+    def logprobs(self) -> list:
+        """Per row None, or the TokenLogprobs of its token (rows whose request asked for them)."""
+        if self._asked is None:
+            return [None] * self._n
+        self._event.synchronize()
+        ids, lps, rank = self._about
+        out: list = []
+        for r, k in enumerate(self._asked):
+            if k is None:
+                out.append(None)
+                continue
+            i, l = ids[r, :k + 1].tolist(), lps[r, :k + 1].tolist()
+            out.append(TokenLogprobs(i[0], l[0], int(rank[r]), list(zip(i[1:], l[1:]))))
+        return out
 
     def tokens(self) -> list[int]:
         if self._n == 0:
@@ -58,6 +75,11 @@ class Sampler:
         self._slots: dict = {}                      # request -> [history slot, outputs already counted]
         self.phases: dict | None = None             # Engine.measure_phases: host time of the last launches and of the wait
         self._free: list = []
+        # made on first use of logprobs: a copy of the logits as the model gave them (where a bias or a penalty
+        # changes them before the token is chosen), the kernel's outputs and their pinned landing places
+        self._raw: torch.Tensor | None = None
+        self._about_dev: tuple | None = None
+        self._about_host: list | None = None
 
     def _buffers(self) -> None:
         if self.work is not None:
@@ -92,11 +114,23 @@ class Sampler:
             self._read = [torch.cuda.Event(), torch.cuda.Event()]
         turn = self._turn
         self._turn ^= 1
-        if all(p.is_greedy and not p.has_penalties for p, *_ in rows):
+        asked = [p.logprobs for p, *_ in rows]
+        if all(k is None for k in asked):
+            asked = None
+        changed = any(p.logit_bias or p.has_penalties for p, *_ in rows)
+        given = logits                      # the logits as the model gave them
+        if asked is not None and changed:
+            if self._raw is None:
+                self._raw = torch.empty((self.max_rows, self.vocab), dtype=torch.float32, device=self.device)
+            given = self._raw
+            given[:R].copy_(logits[:R])
+        if all(p.picks_largest_logit for p, *_ in rows):
             if not done:
                 ops.argmax(logits, self.out, R)
         else:
             assert not done
+            if any(p.logit_bias for p, *_ in rows):         # before the penalties (sampling.cu:286)
+                self._bias(logits, rows)
             if any(p.has_penalties for p, *_ in rows):
                 self._penalties(logits, rows)
             self._buffers()
@@ -111,10 +145,43 @@ class Sampler:
             ops.sample_rows(logits, self.work, self.scratch, self.rows_dev, self.out, R, any_filter=any_filter)
         host = self._tokens_host[turn]
         host[:R].copy_(self.out[:R], non_blocking=True)
+        about = self._logprobs(given, asked, R, turn) if asked is not None else None
         self._read[turn].record()
         if t0 is not None:
             self.phases["sample"] += time.perf_counter() - t0
-        return Sampled(self, R, host, self._read[turn])
+        return Sampled(self, R, host, self._read[turn], asked, about)
+
+    def _bias(self, logits, rows) -> None:
+        entries = [(i, t, b) for i, (p, *_rest) in enumerate(rows) for t, b in p.logit_bias.items() if t < self.vocab]
+        if not entries:
+            return
+        where = torch.tensor([(i, t) for i, t, _ in entries], dtype=torch.int32).to(self.device)
+        what = torch.tensor([b for *_, b in entries], dtype=torch.float32).to(self.device)
+        ops.logit_bias(logits, len(rows), where, what)
+
+    def _logprobs(self, given, asked, R: int, turn: int) -> tuple:
+        """Issues the kernel that reads the tokens just chosen (self.out) and the copies of what it found to this
+        turn's pinned buffers; returns those (valid once the launch's event has passed)."""
+        stride = MAX_LOGPROBS + 1
+        if self._about_dev is None:
+            dev = dict(device=self.device)
+            self._about_dev = (torch.empty(self.max_rows, dtype=torch.int32, **dev),                # k per row
+                               torch.empty((self.max_rows, stride), dtype=torch.int32, **dev),
+                               torch.empty((self.max_rows, stride), dtype=torch.float32, **dev),
+                               torch.empty(self.max_rows, dtype=torch.int32, **dev))
+            self._about_host = [(torch.empty(self.max_rows, dtype=torch.int32, pin_memory=True),
+                                 torch.empty((self.max_rows, stride), dtype=torch.int32, pin_memory=True),
+                                 torch.empty((self.max_rows, stride), dtype=torch.float32, pin_memory=True),
+                                 torch.empty(self.max_rows, dtype=torch.int32, pin_memory=True)) for _ in range(2)]
+        k_dev, ids_dev, lp_dev, rank_dev = self._about_dev
+        k_host, ids_host, lp_host, rank_host = self._about_host[turn]
+        k_host[:R] = torch.tensor([-1 if k is None else k for k in asked], dtype=torch.int32)
+        k_dev[:R].copy_(k_host[:R], non_blocking=True)
+        ops.logprobs(given, self.out, k_dev, ids_dev, lp_dev, rank_dev, R)
+        ids_host[:R].copy_(ids_dev[:R], non_blocking=True)
+        lp_host[:R].copy_(lp_dev[:R], non_blocking=True)
+        rank_host[:R].copy_(rank_dev[:R], non_blocking=True)
+        return ids_host, lp_host, rank_host
 
     def forget(self, key) -> None:
         """The request is over: its history slot is free again."""

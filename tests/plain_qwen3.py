@@ -175,6 +175,24 @@ def apply_penalties(logits, prompt, output, repetition=1.0, frequency=0.0, prese
     return z
 
 
+def apply_logit_bias(logits, bias):
+    """bias: {token: value} added to the logits before the penalties (crates/kernels/cuda/sampling.cu:286-305)."""
+    z = logits.clone()
+    for t, b in bias.items():
+        z[t] = z[t] + b
+    return z
+
+
+def token_logprobs(logits, chosen, k):
+    """(logprob of chosen, rank, [(token, logprob)] of the k most probable) from the log-softmax of the logits as
+    the model gave them; rank counts the tokens with a strictly larger logit; equal values go by lower index
+    (crates/kernels/cuda/sampling.cu:380-430, crates/core/src/sampler.rs:156-166)."""
+    z = logits.double()
+    lp = z - torch.logsumexp(z, -1)
+    order = sorted(range(z.numel()), key=lambda i: (-float(z[i]), i))[:k]
+    return float(lp[chosen]), int((z > z[chosen]).sum()), [(i, float(lp[i])) for i in order]
+
+
 def candidate_mask(z, top_k=-1, top_p=1.0, min_p=0.0):
     """Which tokens survive min_p -> top-k -> top-p, on z = logits / temperature
     (crates/kernels/cuda/sampling.cu:83-129,352-364; order :266-283). top-p keeps the most

@@ -337,3 +337,52 @@ def test_steps_launched_ahead_give_the_same_tokens(model_dirs, name, dtype, grap
     a, ra, _ = run(False, stop=[stop])
     b, rb, _ = run(True, stop=[stop])
     assert a == b and ra == rb and "stop" in ra
+
+
+@pytest.mark.parametrize("ahead", [False, True])
+def test_logprobs_and_logit_bias_through_the_engine(model_dirs, ahead):
+    """A request that asks for log-probabilities gets, for every token, the plain model's log-softmax at that place
+    (of the logits before any bias), also when steps are launched ahead; a bias of +100 makes its token the only
+    one that comes, a bias of -100 on the plain model's choice keeps it away."""
+    from dinfer_amd import SamplingParams
+    name = "B"
+    cfg, w = plain.load(model_dirs[name])
+    V = cfg["vocab_size"]
+    prompts = prompts_for(name, [9, 40, 21, 5], 13)
+    first = [int(plain.forward(cfg, w, p)[-1].argmax()) for p in prompts]
+    sps = [SamplingParams(max_tokens=10, temperature=0.0, ignore_eos=True, logprobs=4),
+           SamplingParams(max_tokens=10, temperature=0.0, ignore_eos=True, logprobs=0, logit_bias={V - 2: 100.0}),
+           SamplingParams(max_tokens=6, temperature=0.0, ignore_eos=True, logit_bias={first[2]: -100.0}, logprobs=1),
+           SamplingParams(max_tokens=10, temperature=0.8, seed=3, ignore_eos=True)]
+    eng = engine(model_dirs[name], name, async_scheduling=ahead, max_num_batched_tokens=32)
+    got, about = eng.generate(prompts, sps, return_logprobs=True)
+    assert about[3] is None and got[1] == [V - 2] * 10 and got[2][0] != first[2]
+    for p, g, a, sp in zip(prompts[:3], got[:3], about[:3], sps[:3]):
+        assert len(a) == len(g)
+        ids = list(p)
+        for i, (tok, lp) in enumerate(zip(g, a)):
+            row = plain.forward(cfg, w, ids)[-1]
+            want, rank, top = plain.token_logprobs(row, tok, sp.logprobs)
+            assert lp.token_id == tok and abs(lp.logprob - want) < 1e-4, (len(p), i, lp, want)
+            gap = float((row.sort(descending=True).values[:-1] - row.sort(descending=True).values[1:])[:sp.logprobs + 1].min())
+            if gap > 1e-4:          # (two logits nearer than rounding may change places)
+                assert lp.rank == rank and [t for t, _ in lp.top] == [t for t, _ in top], (len(p), i)
+            for (_, x), (_, y) in zip(lp.top, top):
+                assert abs(x - y) < 1e-4
+            ids.append(tok)
+    assert all(x.rank == 0 and x.top[0][0] == x.token_id for x in about[0])
+    assert eng.runner.cache.num_free(0) == 128
+
+
+def test_logprobs_in_bfloat16_graphs_equal_step_by_step(model_dirs):
+    """Greedy rows whose token a replayed graph finds itself still get their log-probabilities, the same ones
+    with and without steps launched ahead."""
+    from dinfer_amd import SamplingParams
+    prompts = prompts_for("A", [5, 17, 33], 3)
+    sp = SamplingParams(max_tokens=12, temperature=0.0, ignore_eos=True, logprobs=3)
+    runs = []
+    for ahead in (False, True):
+        eng = engine(model_dirs["A"], "A", dtype="bfloat16", hip_graph=True, async_scheduling=ahead)
+        runs.append(eng.generate(prompts, sp, return_logprobs=True))
+    assert runs[0] == runs[1]
+    assert all(x.rank == 0 and x.top[0] == (x.token_id, x.logprob) for a in runs[0][1] for x in a)

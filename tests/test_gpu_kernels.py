@@ -992,3 +992,94 @@ def test_measured_ceilings_are_plausible():
     assert 1.6e12 < hbm < 8.0e12, hbm
     mfma = ops().measured_mfma_bf16(DEV)
     assert 0.5e15 < mfma < 2.5e15, mfma
+
+
+@pytest.mark.parametrize("V", [331, 4097, 151936])
+def test_logprobs_of_chosen_and_most_probable_tokens(V):
+    """Log-softmax of the row as given: the chosen token's value and rank, the k most probable in falling order.
+    Equal logits (planted at the top and around the chosen token) go by index; a row that asks nothing is left
+    alone; k = 0 gives the chosen token only."""
+    g = torch.Generator().manual_seed(V)
+    logits = torch.randn(6, V, generator=g) * 4
+    ks = [-1, 0, 3, 20, 7, 32]
+    chosen = [5, V - 1, 17, 0, 200, 9]
+    logits[2, [40, 3, 300]] = logits[2].max() + 1.0            # three equal best: 3, 40, 300 in that order
+    logits[4, [100, 200, 250]] = float(logits[4].topk(5).values[-1])   # the chosen one has twins of equal value
+    logits[5, 1:] = logits[5, 0]                                # a flat row: every rank is 0, the top is 0, 1, 2, ...
+    stride = 33
+    ids = torch.full((6, stride), -7, dtype=torch.int32, device=DEV)
+    lps = torch.full((6, stride), 7.0, dtype=torch.float32, device=DEV)
+    rank = torch.full((6,), -7, dtype=torch.int32, device=DEV)
+    i32 = lambda xs: torch.tensor(xs, device=DEV, dtype=torch.int32)
+    ops().logprobs(logits.to(DEV), i32(chosen), i32(ks), ids, lps, rank, 6)
+    ids, lps, rank = ids.cpu(), lps.cpu(), rank.cpu()
+    assert (ids[0] == -7).all() and (lps[0] == 7.0).all() and rank[0] == -7
+    for r in range(1, 6):
+        lp, rk, top = plain.token_logprobs(logits[r], chosen[r], ks[r])
+        assert ids[r, 0] == chosen[r] and rank[r] == rk, (r, int(rank[r]), rk)
+        assert abs(float(lps[r, 0]) - lp) < 2e-5
+        assert ids[r, 1:ks[r] + 1].tolist() == [t for t, _ in top], r
+        torch.testing.assert_close(lps[r, 1:ks[r] + 1].double(), torch.tensor([v for _, v in top], dtype=torch.float64),
+                                   rtol=0, atol=2e-5)
+        assert (ids[r, ks[r] + 1:] == -7).all()
+    assert ids[2, 1:4].tolist() == [3, 40, 300] and rank[5] == 0 and ids[5, 1:5].tolist() == [0, 1, 2, 3]
+
+
+def test_logprobs_of_a_vocabulary_smaller_than_k():
+    logits = torch.tensor([[0.0, 1.0, -1.0]])
+    ids = torch.zeros((1, 6), dtype=torch.int32, device=DEV)
+    lps = torch.zeros((1, 6), dtype=torch.float32, device=DEV)
+    rank = torch.zeros(1, dtype=torch.int32, device=DEV)
+    i32 = lambda xs: torch.tensor(xs, device=DEV, dtype=torch.int32)
+    ops().logprobs(logits.to(DEV), i32([2]), i32([5]), ids, lps, rank, 1)
+    assert ids.cpu()[0].tolist() == [2, 1, 0, 2, -1, -1] and rank.item() == 2
+    assert lps.cpu()[0, 4:].tolist() == [float("-inf")] * 2
+
+
+def test_logit_bias_adds_to_the_named_logits_only():
+    V = 1000
+    logits = torch.randn(3, V)
+    entries = [(0, 5, 2.5), (2, 999, -100.0), (2, 0, 100.0), (1, 17, 0.25), (3, 4, 9.0), (1, 1000, 9.0), (-1, 3, 9.0)]
+    got = logits.to(DEV)
+    ops().logit_bias(got, 3, torch.tensor([(r, t) for r, t, _ in entries], dtype=torch.int32, device=DEV),
+                     torch.tensor([b for *_, b in entries], dtype=torch.float32, device=DEV))
+    want = logits.clone()
+    for r, bias in ((0, {5: 2.5}), (1, {17: 0.25}), (2, {999: -100.0, 0: 100.0})):      # the rest names no cell
+        want[r] = plain.apply_logit_bias(logits[r], bias)
+    torch.testing.assert_close(got.cpu(), want, rtol=0, atol=0)
+
+
+def test_sampler_with_bias_penalties_and_logprobs_in_one_batch():
+    """Rows of every kind side by side: the token comes from the logits after bias and penalties, the
+    log-probabilities from the logits as they were given."""
+    from dinfer_amd.sampling.params import SamplingParams
+    from dinfer_amd.sampling.sampler import Sampler
+    V = 777
+    s = Sampler(DEV, 6, V)
+    g = torch.Generator().manual_seed(9)
+    for turn in range(3):                       # (the pinned buffers alternate: both are used, and one again)
+        logits = torch.randn(5, V, generator=g) * 3
+        best = logits.argmax(-1).tolist()
+        sps = [SamplingParams(temperature=0.0, logprobs=2),
+               SamplingParams(temperature=0.0, logit_bias={best[1]: -100.0}, logprobs=0),
+               SamplingParams(temperature=0.0, logit_bias={3: 100.0}),
+               SamplingParams(temperature=0.0, repetition_penalty=2.0, presence_penalty=2.0, logprobs=20),
+               SamplingParams(temperature=0.9, seed=5, logit_bias=[(7, 1.5), (8, -1.5)], logprobs=1)]
+        prompt, output = [best[3], 4], [best[3], 9]
+        rows = [(p, turn, prompt, output, p.seed or 0) for p in sps]
+        launched = s.launch(logits.to(DEV), rows)
+        toks, about = launched.tokens(), launched.logprobs()
+        z1 = plain.apply_logit_bias(logits[1].double(), sps[1].logit_bias)
+        z3 = plain.apply_penalties(logits[3].double(), prompt, output, 2.0, 0.0, 2.0)
+        z4 = plain.apply_logit_bias(logits[4].double(), sps[4].logit_bias)
+        want4, slack = plain.sample_row(z4, 0.9, 5, turn)
+        assert toks[0] == best[0] and toks[1] == int(z1.argmax()) != best[1] and toks[2] == 3
+        assert toks[3] == int(z3.argmax()) != best[3]
+        assert toks[4] == want4 or slack < 1e-5
+        assert about[2] is None
+        for r in (0, 1, 3, 4):
+            lp, rk, top = plain.token_logprobs(logits[r], toks[r], sps[r].logprobs)
+            a = about[r]
+            assert a.token_id == toks[r] and a.rank == rk and abs(a.logprob - lp) < 2e-5
+            assert [t for t, _ in a.top] == [t for t, _ in top]
+        assert about[0].rank == 0 and about[1].rank == 1 and about[3].rank >= 1

@@ -2,6 +2,8 @@
 besides the reference's text: special cases that reduce to a library routine, invariants, and
 known answers. Each check is chosen so that a plausible mistake fails it (noted per test). No GPU."""
 
+import math
+
 import pytest
 import torch
 import torch.nn.functional as F
@@ -180,3 +182,21 @@ def test_penalties_by_hand():
     z = torch.tensor([2.0, -2.0, 1.0, 1.0, 3.0])
     out = plain.apply_penalties(z, prompt=[0, 1], output=[1, 2, 2], repetition=2.0, frequency=0.5, presence=0.1)
     torch.testing.assert_close(out, torch.tensor([1.0, -4.0 - 0.6, 0.5 - 1.1, 1.0, 3.0]))
+
+
+def test_logit_bias_and_logprobs_by_hand():
+    p = torch.tensor([0.5, 0.25, 0.125, 0.125])
+    z = torch.log(p) + 3.0                                  # any shift of the logits leaves the probabilities
+    lp, rank, top = plain.token_logprobs(z, 2, 3)
+    assert abs(lp - math.log(0.125)) < 1e-6 and rank == 2   # two tokens are more probable; its twin is not
+    assert [t for t, _ in top] == [0, 1, 2]                 # of the equal pair the lower index comes first
+    torch.testing.assert_close(torch.tensor([v for _, v in top], dtype=torch.float64), torch.log(p[:3]).double(), rtol=1e-6, atol=1e-6)
+    assert plain.token_logprobs(z, 0, 0) == (pytest.approx(math.log(0.5), abs=1e-6), 0, [])
+    # against the library's routine
+    g = torch.randn(300, generator=torch.Generator().manual_seed(4)) * 4
+    lp, rank, top = plain.token_logprobs(g, 17, 5)
+    ref = torch.log_softmax(g.double(), -1)
+    assert abs(lp - float(ref[17])) < 1e-12 and [t for t, _ in top] == torch.topk(g, 5).indices.tolist()
+    assert rank == int((ref > ref[17]).sum())
+    b = plain.apply_logit_bias(torch.tensor([1.0, 2.0, 3.0]), {0: 5.0, 2: -100.0})
+    assert b.tolist() == [6.0, 2.0, -97.0]

@@ -1,5 +1,7 @@
 """The scheduler's decisions (no GPU), driven step by step with made-up sampled tokens. The vectors
 are the ones the reference's own tests hold (crates/core/src/sched/mod.rs:830-1442)."""
+import pytest
+
 from dinfer_amd.cache import CacheManager, GroupSpec
 from dinfer_amd.config import EngineOptions
 from dinfer_amd.engine.request import LENGTH, PREEMPTED, STOP, Request
@@ -539,3 +541,32 @@ def test_random_loads_planned_ahead_match_step_by_step():
         assert outs[0] == outs[1], f"seed {seed}"
         looked += res[1]
     assert looked > 50                                  # the loads do spend most decode steps planned ahead
+
+
+@pytest.mark.parametrize("fields,needle", [
+    (dict(temperature=-0.1), "temperature"), (dict(top_p=0.0), "top_p"), (dict(top_k=0), "top_k"),
+    (dict(min_p=1.5), "min_p"), (dict(repetition_penalty=0.0), "repetition_penalty"),
+    (dict(frequency_penalty=2.5), "frequency_penalty"), (dict(presence_penalty=-2.5), "presence_penalty"),
+    (dict(max_tokens=0), "max_tokens"), (dict(max_tokens=3, min_tokens=4), "min_tokens"),
+    (dict(logprobs=21), "logprobs"), (dict(logprobs=-1), "logprobs"),
+    (dict(logit_bias={5: 100.5}), "logit_bias"), (dict(logit_bias={-3: 1.0}), "logit_bias"),
+    (dict(logit_bias={i: 0.5 for i in range(301)}), "at most 300"), (dict(seed=1 << 64), "seed")])
+def test_sampling_options_out_of_range_are_refused_at_admission(fields, needle):
+    """The ranges of crates/core/src/sample.rs:157-205."""
+    s = mk(4, 64, 16)
+    with pytest.raises(ValueError, match=needle):
+        s.add_request(Request(0, [1, 2, 3], SamplingParams(**fields)))
+    assert not s.has_unfinished()
+
+
+def test_logit_bias_takes_a_mapping_or_pairs():
+    a = SamplingParams(logit_bias={"7": 1, 9: -2.5})
+    b = SamplingParams(logit_bias=[(7, 1.0), (9, -2.5)])
+    assert a.logit_bias == b.logit_bias == {7: 1.0, 9: -2.5}
+    a.validate()
+    assert SamplingParams(logprobs=20, logit_bias={i: 100.0 for i in range(300)}).validate() is None
+    with pytest.raises(ValueError, match="twice"):
+        SamplingParams(logit_bias=[(7, 1.0), (7, 2.0)])
+    assert SamplingParams(temperature=0.0).picks_largest_logit
+    assert not SamplingParams(temperature=0.0, logit_bias={1: 1.0}).picks_largest_logit
+    assert not SamplingParams(temperature=0.0, presence_penalty=0.5).picks_largest_logit
