@@ -203,7 +203,8 @@ void* dh_sched_create(const dh_sched_options* opt, void* cache, const int32_t* e
 void dh_sched_destroy(void* sched) { delete S(sched); }
 
 int32_t dh_sched_add(void* sched, int64_t rid, const int32_t* prompt, int32_t n_prompt, int32_t max_tokens,
-                     int32_t min_tokens, int32_t ignore_eos, const int32_t* stop_ids, int32_t n_stop) {
+                     int32_t min_tokens, int32_t ignore_eos, const int32_t* stop_ids, int32_t n_stop,
+                     int32_t every_row) {
     return guarded([&] {
         auto r = std::make_unique<Request>();
         r->id = rid;
@@ -212,6 +213,7 @@ int32_t dh_sched_add(void* sched, int64_t rid, const int32_t* prompt, int32_t n_
         r->min_tokens = min_tokens;
         r->ignore_eos = ignore_eos != 0;
         r->stop_ids.assign(stop_ids, stop_ids + (n_stop > 0 ? n_stop : 0));
+        r->every_row = every_row != 0;
         S(sched)->sched.add(std::move(r));
         return 0;
     });

@@ -79,18 +79,22 @@ int32_t dh_batch_fill(void* cache, const dh_batch_buffers* buf, int32_t n, const
 typedef struct {
     int32_t max_num_batched_tokens, max_num_seqs, max_model_len, prefill_tokens_per_step,
         long_prefill_token_threshold, enable_chunked_prefill, decode_exempt_from_budget, enable_prefix_caching,
-        prefill_chunk_alignment;
+        prefill_chunk_alignment, max_logits_rows;
 } dh_sched_options;
 
-typedef struct { int64_t id; int32_t start, num_new, samples; } dh_scheduled;
+/* rows_from, num_rows: prompt positions at which logits are wanted as well; their rows follow the sampling rows */
+typedef struct { int64_t id; int32_t start, num_new, samples, rows_from, num_rows; } dh_scheduled;
 typedef struct { int64_t id; int32_t token, reason; } dh_update_result;
 /* status: 0 waiting, 1 running, 2 preempted, 3 finished. reason: 0 none, 1 stop, 2 length, 3 abort */
 typedef struct { int32_t num_prompt, num_tokens, num_computed, status, reason, preemptions, num_cached; } dh_request_info;
 
 void* dh_sched_create(const dh_sched_options* opt, void* cache, const int32_t* eos, int32_t n_eos);
 void dh_sched_destroy(void* sched);
+/* every_row: logits are wanted at every prompt position whose next token is in the prompt (needs max_logits_rows >
+ * max_num_seqs) */
 int32_t dh_sched_add(void* sched, int64_t rid, const int32_t* prompt, int32_t n_prompt, int32_t max_tokens,
-                     int32_t min_tokens, int32_t ignore_eos, const int32_t* stop_ids, int32_t n_stop);
+                     int32_t min_tokens, int32_t ignore_eos, const int32_t* stop_ids, int32_t n_stop,
+                     int32_t every_row);
 int32_t dh_sched_abort(void* sched, int64_t rid);
 int32_t dh_sched_forget(void* sched, int64_t rid);
 int32_t dh_sched_has_unfinished(void* sched);

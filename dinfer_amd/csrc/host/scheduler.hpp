@@ -40,6 +40,8 @@ struct SchedOptions {
     int32_t decode_exempt_from_budget;
     int32_t enable_prefix_caching;  // needs a cache manager built with a prefix cache
     int32_t prefill_chunk_alignment;  // a portion that does not end its request's tokens ends at a multiple of this (<= 1: anywhere)
+    int32_t max_logits_rows;  // rows of logits a step can return (0: max_num_seqs); what exceeds max_num_seqs is free
+                              // for the prompt positions of requests that want logits at each of them
 };
 
 enum Status : int32_t { WAITING = 0, RUNNING = 1, PREEMPTED = 2, FINISHED = 3 };
@@ -63,6 +65,12 @@ struct Request {
     // request's last whatever it is (max_tokens or max_model_len), so no further step is planned for it.
     int32_t pending = 0, pending_src = -1;
     bool ending = false;
+    // every_row: logits are wanted at every position of the prompt whose next token is in the prompt too (the
+    // log-probabilities of a prompt, crates/core/src/sample.rs:103-105), beside the row that samples. Such a request
+    // takes nothing from the prefix cache, and its portions are cut to the rows a step has to spare. rows_done:
+    // positions below this have had theirs (a request that is preempted computes them again, silently).
+    bool every_row = false;
+    int32_t rows_done = 0;
 
     int32_t num_tokens() const { return static_cast<int32_t>(tokens.size()); }
     int32_t num_output() const { return num_tokens() - num_prompt; }
@@ -73,6 +81,8 @@ struct Scheduled {
     int32_t start;    // tokens computed before this step
     int32_t num_new;  // tokens this step feeds
     int32_t samples;  // the step reaches the end of the known tokens, so a token is sampled
+    int32_t rows_from, num_rows;  // logits are wanted at the num_rows positions from rows_from on as well (after the
+                                  // rows of all sampling requests, in the order of the plan)
 };
 
 // (feedback: for each scheduled request, the place among the sampled tokens of the step before whose value its last
@@ -108,8 +118,17 @@ public:
             throw Error(ERR_VALUE, "prompt of " + std::to_string(req->num_prompt) +
                                        " tokens leaves no room for output within max_model_len " +
                                        std::to_string(opt_.max_model_len));
+        if (req->every_row) {
+            if (spare_rows() <= 0)
+                throw Error(ERR_VALUE, "logits at every prompt position need rows beyond one per request: "
+                                       "max_logits_rows must exceed max_num_seqs");
+            if (!opt_.enable_chunked_prefill && req->num_prompt - 1 > spare_rows())
+                throw Error(ERR_VALUE, "without chunked prefill a prompt of " + std::to_string(req->num_prompt) +
+                                           " tokens needs " + std::to_string(req->num_prompt - 1) + " spare rows of logits");
+        }
         req->status = WAITING;
         req->num_computed = 0;
+        req->rows_done = 0;
         Request* r = req.get();
         reqs_.emplace(r->id, std::move(req));
         waiting_.push_back(r);
@@ -144,6 +163,22 @@ public:
         if (a <= 1 || n <= 0 || n >= remaining) return n;
         const int64_t end = (computed + n) / a * a;
         return end > computed ? end - computed : 0;
+    }
+
+    // Rows of logits a step has beyond one per request.
+    int64_t spare_rows() const {
+        return opt_.max_logits_rows > opt_.max_num_seqs ? opt_.max_logits_rows - opt_.max_num_seqs : 0;
+    }
+    // The prompt positions of [c, c + n) at which r still wants logits: [first, second).
+    static std::pair<int64_t, int64_t> prompt_rows(const Request& r, int64_t c, int64_t n) {
+        if (!r.every_row) return {0, 0};
+        const int64_t lo = std::max<int64_t>(c, r.rows_done), hi = std::min<int64_t>(c + n, r.num_prompt - 1);
+        return hi > lo ? std::make_pair(lo, hi) : std::make_pair<int64_t, int64_t>(0, 0);
+    }
+    // The most of n tokens from c on whose prompt rows fit into `spare`.
+    static int64_t fit_rows(const Request& r, int64_t c, int64_t n, int64_t spare) {
+        const auto rows = prompt_rows(r, c, n);
+        return rows.second - rows.first <= spare ? n : rows.first + spare - c;
     }
 
     // ---- one step
@@ -199,6 +234,15 @@ private:
         const size_t eligible = running_.size() + waiting_.size();
         const int64_t threshold = eligible > 1 ? opt_.long_prefill_token_threshold : 0;
         bool preempted_any = false;
+        int64_t spare = spare_rows();
+        auto put = [&](Request* r, int64_t n, int32_t feedback) {
+            const auto rows = prompt_rows(*r, r->num_computed, n);
+            plan_.scheduled.push_back({r->id, r->num_computed, static_cast<int32_t>(n),
+                                       r->num_computed + n == r->num_tokens(), static_cast<int32_t>(rows.first),
+                                       static_cast<int32_t>(rows.second - rows.first)});
+            plan_.feedback.push_back(feedback);
+            spare -= rows.second - rows.first;
+        };
 
         size_t i = 0;
         while (i < running_.size()) {
@@ -215,6 +259,7 @@ private:
             if (threshold && n > threshold) n = threshold;
             if (charged) n = std::min(n, budget);
             if (!is_decode) n = std::min(n, quota);
+            n = fit_rows(*r, r->num_computed, n, spare);
             if (n < remaining && !opt_.enable_chunked_prefill) n = 0;
             n = aligned(r->num_computed, n, remaining);
             if (n <= 0) {
@@ -241,9 +286,7 @@ private:
                 preempted_any = true;
             }
             if (!got) break;
-            plan_.scheduled.push_back({r->id, r->num_computed, static_cast<int32_t>(n),
-                                       r->num_computed + n == r->num_tokens()});
-            plan_.feedback.push_back(r->pending && r->num_computed + n == r->num_tokens() ? r->pending_src : -1);
+            put(r, n, r->pending && r->num_computed + n == r->num_tokens() ? r->pending_src : -1);
             if (charged) budget -= n;
             if (!is_decode) quota -= n;
             ++i;
@@ -256,7 +299,8 @@ private:
                 cache_->admit(r->id);
                 // a prefix of the prompt (or, after a preemption, of prompt and outputs) may be in the cache
                 // still: those tokens are not computed again (:564-570)
-                if (opt_.enable_prefix_caching && r->num_computed == 0) {
+                const bool rows_open = r->every_row && r->rows_done < r->num_prompt - 1;  // every position is computed
+                if (opt_.enable_prefix_caching && r->num_computed == 0 && !rows_open) {
                     r->num_cached = static_cast<int32_t>(cache_->lookup(r->id, r->tokens.data(), r->num_tokens()));
                     r->num_computed = r->num_cached;
                 }
@@ -264,6 +308,7 @@ private:
                 int64_t n = remaining;
                 if (threshold && n > threshold) n = threshold;
                 n = std::min(n, std::min(budget, quota));
+                n = fit_rows(*r, r->num_computed, n, spare);
                 if (n < remaining && !opt_.enable_chunked_prefill) n = 0;
                 n = aligned(r->num_computed, n, remaining);
                 if (n <= 0 || !cache_->allocate(r->id, r->num_computed, n)) {
@@ -274,9 +319,7 @@ private:
                 waiting_.pop_front();
                 r->status = RUNNING;
                 running_.push_back(r);
-                plan_.scheduled.push_back({r->id, r->num_computed, static_cast<int32_t>(n),
-                                           r->num_computed + n == r->num_tokens()});
-                plan_.feedback.push_back(-1);
+                put(r, n, -1);
                 budget -= n;
                 quota -= n;
             }
@@ -285,6 +328,7 @@ private:
         for (const Scheduled& s : plan_.scheduled) {
             Request* r = reqs_.at(s.id).get();
             if (r->status == RUNNING) r->num_computed = s.start + s.num_new;
+            if (s.num_rows > 0) r->rows_done = s.rows_from + s.num_rows;
         }
         plan_.open = !plan_.scheduled.empty();
         return plan_;
@@ -331,13 +375,17 @@ public:
     // The plan's entries over the requests' own token storage (valid until the next update).
     void plan_entries(std::vector<EntryView>& entries, std::vector<int32_t>& want_store) const {
         entries.clear();
-        want_store.assign(plan_.scheduled.size(), 0);
-        size_t i = 0;
+        size_t rows = 0;
+        for (const Scheduled& s : plan_.scheduled) rows += s.num_rows;
+        want_store.assign(plan_.scheduled.size() + rows, 0);  // (sized once: the entries point into it)
+        size_t i = 0, at = plan_.scheduled.size();
         for (const Scheduled& s : plan_.scheduled) {
             const Request* r = reqs_.at(s.id).get();
             want_store[i] = s.num_new - 1;
+            for (int32_t j = 0; j < s.num_rows; ++j) want_store[at + j] = s.rows_from - s.start + j;
             entries.push_back({s.id, s.start, s.num_new, r->tokens.data() + s.start, &want_store[i], s.samples ? 1 : 0,
-                               plan_.feedback[i]});
+                               plan_.feedback[i], &want_store[at], s.num_rows});
+            at += s.num_rows;
             ++i;
         }
     }

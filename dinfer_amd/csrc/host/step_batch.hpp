@@ -10,7 +10,7 @@
 //   seq_lens     [B]     request length after this step (start + n)
 //   block_table  [B, MB] per cache group, -1 where no page is held
 //   state_slots  [B]     the request's fixed-size state slot
-//   logits_rows  [R]     rows of the flat batch whose logits are wanted
+//   logits_rows  [R]     rows of the flat batch whose logits are wanted: every entry's `want`, then every entry's `more`
 //   feedback_src [T]     -1, or: the token's id is the feedback_src-th token the last step sampled (still on the device)
 //
 // Padding (pad_to > B): a step of single rows that replays a captured graph of pad_to requests
@@ -57,6 +57,8 @@ struct EntryView {
     int32_t n_want;
     int32_t feedback_src = -1;  // >= 0: the entry's last token is not known on the host yet; it is this one of the
                                 // tokens the last step samples (its id in `tokens` is a placeholder)
+    const int32_t* more = nullptr;  // n_more further wanted places, whose rows come after the `want` rows of
+    int32_t n_more = 0;             // all entries
 };
 
 inline void fill_batch(const CacheManager& cache, const BatchBuffers& buf, const EntryView* entries, int n_entries,
@@ -67,7 +69,7 @@ inline void fill_batch(const CacheManager& cache, const BatchBuffers& buf, const
     for (int b = 0; b < n_entries; ++b) {
         if (entries[b].count <= 0) throw Error(ERR_VALUE, "entry " + std::to_string(b) + " brings no token to this step");
         T += entries[b].count;
-        R += entries[b].n_want;
+        R += entries[b].n_want + entries[b].n_more;
     }
     const int B = n_entries;
     if (B == 0) throw Error(ERR_VALUE, "a step needs at least one request with at least one token");
@@ -117,6 +119,16 @@ inline void fill_batch(const CacheManager& cache, const BatchBuffers& buf, const
         max_len = e.start + n > max_len ? e.start + n : max_len;
         singles += n == 1;
         t += n;
+    }
+    for (int b = 0; b < B; ++b) {
+        const EntryView& e = entries[b];
+        for (int i = 0; i < e.n_more; ++i) {
+            const int w = e.more[i];
+            if (w < 0 || w >= e.count)
+                throw Error(ERR_VALUE, "entry " + std::to_string(b) + ": wanted place " + std::to_string(w) +
+                                           " is outside its " + std::to_string(e.count) + " tokens");
+            buf.logits_rows[r++] = buf.cu_seqlens[b] + w;
+        }
     }
     int Bp = B;
     if (pad_to > B) {

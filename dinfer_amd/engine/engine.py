@@ -30,6 +30,16 @@ class StepOutput:
     finished: bool
     finish_reason: str | None
     logprobs: object = None    # TokenLogprobs of the token, for a request that asked for them
+    prompt_logprobs: list | None = None   # [(position, TokenLogprobs)] of the prompt tokens this step judged
+
+
+@dataclass
+class Generation:
+    """What generate(..., details=True) returns for a prompt."""
+    token_ids: list
+    finish_reason: str | None
+    logprobs: list | None          # one TokenLogprobs per generated token (SamplingParams.logprobs)
+    prompt_logprobs: list | None   # one per prompt token, None for the first (SamplingParams.prompt_logprobs)
 
 
 class _Ready:
@@ -67,7 +77,8 @@ class Engine:
         # the host has read them
         last = getattr(getattr(self.runner, "batch", None), "last_tokens", None)
         self.sampler = Sampler(self.runner.device, self.runner.max_rows, spec.vocab_size, out=last)
-        # the step in flight: (plan, tokens on their way, device events, the sampled rows' requests if any wants logprobs)
+        # the step in flight: (plan, tokens on their way, device events, the sampled rows' requests if any wants
+        # logprobs, the prompt rows and what is found at them)
         self._running = None
         self._ids = itertools.count()
         self._seeds = random.Random()
@@ -110,14 +121,18 @@ class Engine:
                 outs += self._launch(ahead=True)        # (a plan ahead ends nobody: nothing is added)
             finally:                                    # whatever happened, the running step is still the running step
                 self._running, nxt = held, self._running
-        so, sampled, events, asking = self._running
+        so, sampled, events, asking, prompt = self._running
         tokens = sampled.tokens()
         t0 = time.perf_counter() if ph is not None else 0.0
-        about = {}
+        about, about_prompt = {}, {}
         if asking is not None:      # the requests of the sampled rows, where one of them wants log-probabilities
             about = {r.id: lp for r, lp in zip(asking, sampled.logprobs()) if lp is not None}
+        if prompt is not None:      # ((request, position) of the prompt rows, what was found there)
+            for (r, pos), lp in zip(prompt[0], prompt[1].logprobs()):
+                about_prompt.setdefault(r.id, []).append((pos + 1, lp))       # the token judged is the next one
         for r, tok, reason in self.scheduler.update(so, tokens):
-            outs.append(StepOutput(r.id, tok, reason is not None, reason, about.get(r.id) if tok is not None else None))
+            outs.append(StepOutput(r.id, tok, reason is not None, reason, about.get(r.id) if tok is not None else None,
+                                   about_prompt.get(r.id)))
         for o in outs:
             if o.finished:
                 self.sampler.forget(o.request_id)
@@ -157,12 +172,19 @@ class Engine:
         rows = [(r.sampling, len(r.output_ids) + (1 if ahead else 0), r.prompt_ids, r.output_ids, r.seed, r.id)
                 for r in sampling]
         launch = getattr(self.sampler, "launch", None)                 # (a stand-in may only know how to sample())
+        ours = logits[:len(rows)]       # (rows of prompt positions may follow)
         if launch:      # adds to sample (and, later, to wait); a replayed graph may have found the best tokens already
-            sampled = launch(logits, rows, done=getattr(self.runner, "argmax_done", False))
+            sampled = launch(ours, rows, done=getattr(self.runner, "argmax_done", False))
         else:
-            sampled = _Ready(self.sampler.sample(logits, rows))
+            sampled = _Ready(self.sampler.sample(ours, rows))
         asking = sampling if any(r.sampling.logprobs is not None for r in sampling) else None
-        self._running = (so, sampled, self.runner.take_gpu_events() if ph is not None else None, asking)
+        prompt = so.prompt_rows()
+        if prompt:      # their logits follow the sampling rows
+            found = self.sampler.about_rows(logits[len(rows):len(rows) + len(prompt)],
+                                            [r.prompt_ids[p + 1] for r, p in prompt],
+                                            [r.sampling.prompt_logprobs for r, _ in prompt])
+            prompt = (prompt, found)
+        self._running = (so, sampled, self.runner.take_gpu_events() if ph is not None else None, asking, prompt or None)
         return outs
 
     def measure_phases(self, on: bool = True) -> None:
@@ -176,17 +198,17 @@ class Engine:
             self.phases["steps"] = 0
         self.runner.phases = self.sampler.phases = self.phases
 
-    def generate(self, prompts: list, sampling: SamplingParams | list | None = None, *,
-                 return_logprobs: bool = False):
-        """Runs the prompts (lists of token ids) to the end; returns the generated ids of each. return_logprobs:
-        returns (ids, logprobs) instead, logprobs[i] holding one TokenLogprobs per generated token of a request
-        that asked for them (SamplingParams.logprobs) and None otherwise."""
+    def generate(self, prompts: list, sampling: SamplingParams | list | None = None, *, details: bool = False):
+        """Runs the prompts (lists of token ids) to the end; returns the generated ids of each, or with `details`
+        a Generation for each (ids, finish reason, and the log-probabilities its SamplingParams asked for)."""
         params = sampling if isinstance(sampling, list) else [sampling or SamplingParams()] * len(prompts)
         if len(params) != len(prompts):
             raise ValueError("one SamplingParams per prompt, or one for all")
         ids = [self.add_request(p, sp) for p, sp in zip(prompts, params)]
         got = {i: [] for i in ids}
         about = {i: [] for i in ids}
+        about_prompt = {i: [None] for i in ids}
+        why = {i: None for i in ids}
         idle = 0
         while self.has_unfinished():
             outs = self.step()
@@ -194,9 +216,18 @@ class Engine:
             if idle > 2:
                 raise RuntimeError("the scheduler made no progress: a request fits neither the budget nor the pool")
             for o in outs:
-                if o.token is not None and o.request_id in got:
+                if o.request_id not in got:
+                    continue
+                if o.token is not None:
                     got[o.request_id].append(o.token)
                     about[o.request_id].append(o.logprobs)
-        if return_logprobs:
-            return [got[i] for i in ids], [about[i] if p.logprobs is not None else None for i, p in zip(ids, params)]
+                for pos, lp in o.prompt_logprobs or ():
+                    assert pos == len(about_prompt[o.request_id]), "prompt positions come in order, each once"
+                    about_prompt[o.request_id].append(lp)
+                if o.finished:
+                    why[o.request_id] = o.finish_reason
+        if details:
+            return [Generation(got[i], why[i], about[i] if p.logprobs is not None else None,
+                               about_prompt[i] if p.prompt_logprobs is not None else None)
+                    for i, p in zip(ids, params)]
         return [got[i] for i in ids]

@@ -31,7 +31,8 @@ from ..cache import CacheManager
 from ..config import EngineOptions
 from .request import REASON_NAMES, Request
 
-_SCHEDULED = np.dtype([("id", "<i8"), ("start", "<i4"), ("num_new", "<i4"), ("samples", "<i4")], align=True)
+_SCHEDULED = np.dtype([("id", "<i8"), ("start", "<i4"), ("num_new", "<i4"), ("samples", "<i4"), ("rows_from", "<i4"),
+                       ("num_rows", "<i4")], align=True)
 _RESULT = np.dtype([("id", "<i8"), ("token", "<i4"), ("reason", "<i4")], align=True)
 assert _SCHEDULED.itemsize == ctypes.sizeof(native.Scheduled) and _RESULT.itemsize == ctypes.sizeof(native.UpdateResult)
 _INT32_MAX = 2**31 - 1
@@ -77,6 +78,15 @@ class SchedulerOutput:
     def sampling_requests(self) -> list:
         return [r for r, s in zip(self.requests, self.rows["samples"].tolist()) if s]
 
+    def prompt_rows(self) -> list:
+        """[(request, position)]: the prompt positions at which this step returns logits beside the sampling rows
+        (for requests that want the log-probabilities of their prompt), in the order of the logits rows that
+        follow the sampling rows."""
+        if not self.rows["num_rows"].any():
+            return []
+        return [(r, p) for r, lo, n in zip(self.requests, self.rows["rows_from"].tolist(), self.rows["num_rows"].tolist())
+                for p in range(lo, lo + n)]
+
 
 class Scheduler:
     def __init__(self, options: EngineOptions, cache: CacheManager, eos_token_ids=()):
@@ -86,7 +96,8 @@ class Scheduler:
                                 options.prefill_tokens_per_step or 0, options.long_prefill_token_threshold or 0,
                                 int(options.enable_chunked_prefill), int(options.decode_exempt_from_budget),
                                 int(cache.prefix_caching if options.enable_prefix_caching is None
-                                    else options.enable_prefix_caching), int(options.prefill_chunk_alignment or 1))
+                                    else options.enable_prefix_caching), int(options.prefill_chunk_alignment or 1),
+                                int(options.max_logits_rows or 0))
         eos = np.array(sorted(self.eos) or [0], dtype=np.int32)
         self._h = native.created("dh_sched_create", o, cache._h, eos.ctypes.data, len(self.eos))
         self.requests: dict = {}        # id -> Request, for every request that is not finished
@@ -119,7 +130,7 @@ class Scheduler:
         try:
             native.checked("dh_sched_add", self._h, number, prompt.ctypes.data, len(prompt),
                            min(sp.max_tokens, _INT32_MAX), sp.min_tokens, int(sp.ignore_eos), stop.ctypes.data,
-                           len(sp.stop_token_ids))
+                           len(sp.stop_token_ids), int(sp.prompt_logprobs is not None))
         except Exception:
             self.cache.forget(req.id)
             raise

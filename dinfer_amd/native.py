@@ -29,11 +29,12 @@ class BatchFacts(Structure):
 class SchedOptions(Structure):
     _fields_ = [(n, _I) for n in ("max_num_batched_tokens", "max_num_seqs", "max_model_len", "prefill_tokens_per_step",
                                   "long_prefill_token_threshold", "enable_chunked_prefill",
-                                  "decode_exempt_from_budget", "enable_prefix_caching", "prefill_chunk_alignment")]
+                                  "decode_exempt_from_budget", "enable_prefix_caching", "prefill_chunk_alignment",
+                                  "max_logits_rows")]
 
 
 class Scheduled(Structure):
-    _fields_ = [("id", _L), ("start", _I), ("num_new", _I), ("samples", _I)]
+    _fields_ = [("id", _L), ("start", _I), ("num_new", _I), ("samples", _I), ("rows_from", _I), ("num_rows", _I)]
 
 
 class UpdateResult(Structure):
@@ -76,7 +77,7 @@ _SIGNATURES = {
     "dh_batch_fill": (_I, [_P, POINTER(BatchBuffers), _I, _P, _P, _P, _P, _P, _P, _I, POINTER(BatchFacts)]),
     "dh_sched_create": (_P, [POINTER(SchedOptions), _P, _P, _I]),
     "dh_sched_destroy": (None, [_P]),
-    "dh_sched_add": (_I, [_P, _L, _P, _I, _I, _I, _I, _P, _I]),
+    "dh_sched_add": (_I, [_P, _L, _P, _I, _I, _I, _I, _P, _I, _I]),
     "dh_sched_abort": (_I, [_P, _L]),
     "dh_sched_forget": (_I, [_P, _L]),
     "dh_sched_has_unfinished": (_I, [_P]),

@@ -1,6 +1,6 @@
 """Sampling options of a request: names, defaults and ranges of the reference's
 SamplingParams (crates/core/src/sample.rs:81-139, validate :157-205), without the
-text-level and server-level fields (stop strings, prompt_logprobs, grammar).
+text-level and server-level fields (stop strings, grammar).
 """
 from __future__ import annotations
 
@@ -38,6 +38,8 @@ class SamplingParams:
                                    # probable tokens (0: only its own), from the logits the model produced
     logit_bias: dict = field(default_factory=dict)   # token id -> what is added to its logit before anything else
                                                      # (pairs (token, bias) are taken too)
+    prompt_logprobs: int | None = None   # k: the same for every token of the prompt but the first, given the
+                                         # tokens before it (the engine needs max_logits_rows > max_num_seqs)
 
     def __post_init__(self):
         pairs = list(self.logit_bias.items()) if isinstance(self.logit_bias, dict) else list(self.logit_bias)
@@ -80,6 +82,8 @@ class SamplingParams:
             raise ValueError(f"min_tokens {self.min_tokens} > max_tokens {self.max_tokens}")
         if self.logprobs is not None and not (0 <= self.logprobs <= MAX_LOGPROBS):
             raise ValueError(f"logprobs must be in [0, {MAX_LOGPROBS}], got {self.logprobs}")
+        if self.prompt_logprobs is not None and not (0 <= self.prompt_logprobs <= MAX_LOGPROBS):
+            raise ValueError(f"prompt_logprobs must be in [0, {MAX_LOGPROBS}], got {self.prompt_logprobs}")
         if len(self.logit_bias) > MAX_LOGIT_BIAS:
             raise ValueError(f"logit_bias has {len(self.logit_bias)} entries, at most {MAX_LOGIT_BIAS}")
         for t, b in self.logit_bias.items():

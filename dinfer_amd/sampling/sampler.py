@@ -80,6 +80,10 @@ class Sampler:
         self._raw: torch.Tensor | None = None
         self._about_dev: tuple | None = None
         self._about_host: list | None = None
+        self._given: list | None = None             # about_rows(): the tokens to judge, pinned, two turns
+        self._given_dev: torch.Tensor | None = None
+        self._given_read: list | None = None
+        self._given_turn = 0
 
     def _buffers(self) -> None:
         if self.work is not None:
@@ -151,6 +155,28 @@ class Sampler:
             self.phases["sample"] += time.perf_counter() - t0
         return Sampled(self, R, host, self._read[turn], asked, about)
 
+    def about_rows(self, logits: torch.Tensor, targets: list, asked: list) -> Sampled:
+        """The log-probabilities of given tokens: row r of logits is judged as if targets[r] had been chosen there,
+        with its asked[r] most probable tokens beside it (the prompt's own tokens, each given the tokens before it:
+        SamplingParams.prompt_logprobs). Returns at once; logprobs() of what comes back waits. At most two of these
+        may be waiting at a time."""
+        R = len(targets)
+        assert logits.shape[0] == R == len(asked) and R <= self.max_rows and all(k is not None for k in asked)
+        if R == 0:
+            return Sampled(self, 0, None, None)
+        if self._given is None:
+            self._given = [torch.empty(self.max_rows, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+            self._given_dev = torch.empty(self.max_rows, dtype=torch.int32, device=self.device)
+            self._given_read = [torch.cuda.Event(), torch.cuda.Event()]
+        turn = self._given_turn
+        self._given_turn ^= 1
+        host = self._given[turn]
+        host[:R] = torch.tensor(targets, dtype=torch.int32)
+        self._given_dev[:R].copy_(host[:R], non_blocking=True)
+        about = self._logprobs(logits, asked, R, 2 + turn, chosen=self._given_dev)
+        self._given_read[turn].record()
+        return Sampled(self, R, host, self._given_read[turn], asked, about)
+
     def _bias(self, logits, rows) -> None:
         entries = [(i, t, b) for i, (p, *_rest) in enumerate(rows) for t, b in p.logit_bias.items() if t < self.vocab]
         if not entries:
@@ -159,9 +185,10 @@ class Sampler:
         what = torch.tensor([b for *_, b in entries], dtype=torch.float32).to(self.device)
         ops.logit_bias(logits, len(rows), where, what)
 
-    def _logprobs(self, given, asked, R: int, turn: int) -> tuple:
-        """Issues the kernel that reads the tokens just chosen (self.out) and the copies of what it found to this
-        turn's pinned buffers; returns those (valid once the launch's event has passed)."""
+    def _logprobs(self, given, asked, R: int, turn: int, chosen=None) -> tuple:
+        """Issues the kernel that reads the tokens just chosen (self.out, or `chosen`) and the copies of what it
+        found to pinned buffers (turn 0 and 1: launch()'s, 2 and 3: about_rows()'s); returns those (valid once the
+        caller's event has passed)."""
         stride = MAX_LOGPROBS + 1
         if self._about_dev is None:
             dev = dict(device=self.device)
@@ -172,12 +199,12 @@ class Sampler:
             self._about_host = [(torch.empty(self.max_rows, dtype=torch.int32, pin_memory=True),
                                  torch.empty((self.max_rows, stride), dtype=torch.int32, pin_memory=True),
                                  torch.empty((self.max_rows, stride), dtype=torch.float32, pin_memory=True),
-                                 torch.empty(self.max_rows, dtype=torch.int32, pin_memory=True)) for _ in range(2)]
+                                 torch.empty(self.max_rows, dtype=torch.int32, pin_memory=True)) for _ in range(4)]
         k_dev, ids_dev, lp_dev, rank_dev = self._about_dev
         k_host, ids_host, lp_host, rank_host = self._about_host[turn]
         k_host[:R] = torch.tensor([-1 if k is None else k for k in asked], dtype=torch.int32)
         k_dev[:R].copy_(k_host[:R], non_blocking=True)
-        ops.logprobs(given, self.out, k_dev, ids_dev, lp_dev, rank_dev, R)
+        ops.logprobs(given, self.out if chosen is None else chosen, k_dev, ids_dev, lp_dev, rank_dev, R)
         ids_host[:R].copy_(ids_dev[:R], non_blocking=True)
         lp_host[:R].copy_(lp_dev[:R], non_blocking=True)
         rank_host[:R].copy_(rank_dev[:R], non_blocking=True)

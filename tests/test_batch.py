@@ -176,3 +176,27 @@ def test_planned_fill_writes_what_the_entries_would():
         s.update(out, [7000 + step] * len(out.sampling_requests()))
         cache.check()
     assert step >= 5
+
+
+def test_rows_of_prompt_positions_follow_the_sampling_rows():
+    """A request that wants logits at every prompt position: those rows come after the rows of all requests that
+    sample, so the sampler's rows stay the first ones."""
+    opt = EngineOptions(max_num_seqs=4, max_num_batched_tokens=64, block_size=16, max_model_len=4096, num_blocks=64,
+                        max_logits_rows=10, decode_exempt_from_budget=False)
+    cache = CacheManager([GroupSpec(16, 64)], 4)
+    s, b = Scheduler(opt, cache, eos_token_ids=[]), StepBatch(torch.device("cpu"), 256, 4, 10, [8])
+    s.add_request(Request(1, list(range(100, 104)), SamplingParams(max_tokens=4, prompt_logprobs=0)))
+    s.add_request(Request(2, list(range(200, 207)), SamplingParams(max_tokens=4)))
+    s.add_request(Request(3, list(range(300, 320)), SamplingParams(max_tokens=4, prompt_logprobs=3)))
+    out = s.schedule()
+    b.fill_planned(s)
+    # request 1: rows at 0..2 and the sampling row 3; request 2 samples at its 7th token; request 3 gets the three
+    # rows that are left and is cut there
+    assert [(x.request.id, x.num_new, x.samples) for x in out.scheduled] == [(1, 4, True), (2, 7, True), (3, 3, False)]
+    assert b.num_rows == 8 and b.h["logits_rows"][:8].tolist() == [3, 10, 0, 1, 2, 11, 12, 13]
+    assert [(r.id, p) for r, p in out.prompt_rows()] == [(1, 0), (1, 1), (1, 2), (3, 0), (3, 1), (3, 2)]
+    s.update(out, {1: 5, 2: 5})
+    out = s.schedule()
+    b.fill_planned(s)
+    assert [(x.request.id, x.start, x.num_new) for x in out.scheduled] == [(1, 4, 1), (2, 7, 1), (3, 3, 6)]
+    assert b.h["logits_rows"][:8].tolist() == [0, 1, 2, 3, 4, 5, 6, 7]

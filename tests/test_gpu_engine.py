@@ -355,7 +355,9 @@ def test_logprobs_and_logit_bias_through_the_engine(model_dirs, ahead):
            SamplingParams(max_tokens=6, temperature=0.0, ignore_eos=True, logit_bias={first[2]: -100.0}, logprobs=1),
            SamplingParams(max_tokens=10, temperature=0.8, seed=3, ignore_eos=True)]
     eng = engine(model_dirs[name], name, async_scheduling=ahead, max_num_batched_tokens=32)
-    got, about = eng.generate(prompts, sps, return_logprobs=True)
+    res = eng.generate(prompts, sps, details=True)
+    got, about = [g.token_ids for g in res], [g.logprobs for g in res]
+    assert [g.finish_reason for g in res] == ["length"] * 4 and all(g.prompt_logprobs is None for g in res)
     assert about[3] is None and got[1] == [V - 2] * 10 and got[2][0] != first[2]
     for p, g, a, sp in zip(prompts[:3], got[:3], about[:3], sps[:3]):
         assert len(a) == len(g)
@@ -383,6 +385,44 @@ def test_logprobs_in_bfloat16_graphs_equal_step_by_step(model_dirs):
     runs = []
     for ahead in (False, True):
         eng = engine(model_dirs["A"], "A", dtype="bfloat16", hip_graph=True, async_scheduling=ahead)
-        runs.append(eng.generate(prompts, sp, return_logprobs=True))
+        runs.append(eng.generate(prompts, sp, details=True))
     assert runs[0] == runs[1]
-    assert all(x.rank == 0 and x.top[0] == (x.token_id, x.logprob) for a in runs[0][1] for x in a)
+    assert all(x.rank == 0 and x.top[0] == (x.token_id, x.logprob) for g in runs[0] for x in g.logprobs)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_log_probabilities_of_the_prompt(model_dirs, dtype):
+    """prompt_logprobs: every token of the prompt but the first, given the tokens before it, against the plain
+    model's log-softmax at the position before; prompts longer than the spare rows come in several portions, beside
+    requests that decode, and a prompt that is in the prefix cache already is still computed."""
+    from dinfer_amd import SamplingParams
+    name = "B"
+    cfg, w = plain.load(model_dirs[name])
+    prompts = prompts_for(name, [40, 9, 70, 2], 17)
+    prompts.append(list(prompts[0]))                          # the same prompt again
+    sps = [SamplingParams(max_tokens=12, temperature=0.0, ignore_eos=True),
+           SamplingParams(max_tokens=5, temperature=0.0, ignore_eos=True, prompt_logprobs=0),
+           SamplingParams(max_tokens=3, temperature=0.0, ignore_eos=True, prompt_logprobs=3, logprobs=1),
+           SamplingParams(max_tokens=3, temperature=0.0, ignore_eos=True, prompt_logprobs=1),
+           SamplingParams(max_tokens=3, temperature=0.0, ignore_eos=True, prompt_logprobs=2)]
+    eng = engine(model_dirs[name], name, dtype=dtype, max_num_batched_tokens=48, max_logits_rows=4 + 20)
+    first = eng.generate(prompts[:4], sps[:4], details=True)
+    res = first + eng.generate(prompts[4:], sps[4:], details=True)
+    assert res[0].prompt_logprobs is None and res[0].logprobs is None and len(res[2].logprobs) == 3
+    for p, sp, g in zip(prompts[1:], sps[1:], res[1:]):
+        got = g.prompt_logprobs
+        assert len(got) == len(p) and got[0] is None
+        rows = plain.forward(cfg, w, p)
+        for i in range(1, len(p)):
+            want, rank, top = plain.token_logprobs(rows[i - 1], p[i], sp.prompt_logprobs)
+            # (bfloat16 logits are off by up to 0.05 of the row's spread each, as everywhere in these tests)
+            tol = 1e-4 if dtype == "float32" else 0.08 * float(rows[i - 1].std())
+            assert got[i].token_id == p[i] and abs(got[i].logprob - want) < tol, (len(p), i, got[i], want)
+            assert len(got[i].top) == sp.prompt_logprobs
+            if dtype == "float32":
+                for (_, x), (_, y) in zip(got[i].top, top):
+                    assert abs(x - y) < tol
+    assert res[4].token_ids == res[0].token_ids[:3] or dtype != "float32"
+    assert eng.runner.cache.num_free(0) == 128
+    with pytest.raises(ValueError, match="max_logits_rows"):
+        engine(model_dirs[name], name).generate([[1, 2, 3]], SamplingParams(prompt_logprobs=0, max_tokens=1))

@@ -570,3 +570,87 @@ def test_logit_bias_takes_a_mapping_or_pairs():
     assert SamplingParams(temperature=0.0).picks_largest_logit
     assert not SamplingParams(temperature=0.0, logit_bias={1: 1.0}).picks_largest_logit
     assert not SamplingParams(temperature=0.0, presence_penalty=0.5).picks_largest_logit
+
+
+def rows_of(out):
+    return [(x.request.id, x.start, x.num_new, bool(x.samples)) for x in out.scheduled], \
+        [(r.id, p) for r, p in out.prompt_rows()]
+
+
+def test_a_prompt_whose_every_position_is_wanted_is_cut_to_the_spare_rows():
+    """prompt_logprobs: logits at every prompt position whose next token is in the prompt, at most as many a step
+    as the engine has rows beyond one per request; the last prompt token's row is the sampling row."""
+    s = mk(4, 64, 32, max_logits_rows=9)                       # 5 to spare
+    s.add_request(req(1, 23, 3, prompt_logprobs=2))
+    seen, cuts = [], []
+    for _ in range(5):
+        out = s.schedule()
+        plan, rows = rows_of(out)
+        cuts.append(plan[0][1:])
+        seen += [p for _, p in rows]
+        s.update(out, {1: 7} if plan[0][3] else {})
+    assert cuts == [(0, 5, False), (5, 5, False), (10, 5, False), (15, 5, False), (20, 3, True)]
+    assert seen == list(range(22))                           # each once, in order; position 22 samples
+    out = s.schedule()
+    assert rows_of(out) == ([(1, 23, 1, True)], [])          # decoding: nothing more
+
+
+def test_two_such_prompts_share_the_spare_rows_and_others_are_not_held_up():
+    s = mk(4, 64, 32, max_logits_rows=10)                      # 6 to spare
+    s.add_request(req(1, 10, 2, prompt_logprobs=0))
+    s.add_request(req(2, 30, 2))
+    s.add_request(req(3, 10, 2, prompt_logprobs=0))
+    # the first takes the six rows; the plain prompt between them goes in whole; the third finds no row left
+    # and waits (and so does whoever comes after it)
+    out = s.schedule()
+    plan, rows = rows_of(out)
+    assert plan == [(1, 0, 6, False), (2, 0, 30, True)] and rows == [(1, p) for p in range(6)]
+    s.update(out, {2: 5})
+    out = s.schedule()
+    plan, rows = rows_of(out)
+    assert plan == [(1, 6, 4, True), (2, 30, 1, True), (3, 0, 3, False)]
+    assert rows == [(1, 6), (1, 7), (1, 8), (3, 0), (3, 1), (3, 2)]
+
+
+def test_every_position_is_computed_whatever_the_prefix_cache_holds_and_once_whatever_is_preempted():
+    cache = CacheManager([GroupSpec(16, 8)], 4, prefix_caching=True)
+    opt = EngineOptions(max_num_seqs=4, max_num_batched_tokens=64, block_size=16, num_blocks=8, max_model_len=4096,
+                        max_logits_rows=40, decode_exempt_from_budget=False)
+    s = Scheduler(opt, cache, eos_token_ids=[2])
+    first = Request(1, list(range(500, 540)), SamplingParams(max_tokens=1))
+    s.add_request(first)
+    s.update(s.schedule(), {1: 9})                           # ends; its two full pages stay in the prefix cache
+    other = Request(3, list(range(900, 950)), SamplingParams(max_tokens=40))
+    s.add_request(other)
+    s.update(s.schedule(), {3: 7})
+    same = Request(2, list(range(500, 540)), SamplingParams(max_tokens=30, prompt_logprobs=0))
+    s.add_request(same)
+    out = s.schedule()
+    assert rows_of(out) == ([(3, 50, 1, True), (2, 0, 36, False)], [(2, p) for p in range(36)])
+    assert same.num_cached_tokens == 0                       # (the same prompt without the option takes 32 from there)
+    s.update(out, {3: 7})
+    out = s.schedule()
+    assert rows_of(out) == ([(3, 51, 1, True), (2, 36, 4, True)], [(2, 36), (2, 37), (2, 38)])
+    s.update(out, {2: 7, 3: 7})
+    # 4 + 3 pages of 8 are held; both decode until the first needs a page that is not there and the one admitted
+    # last is preempted: when it comes back it computes its prompt again, and no position is reported twice
+    seen = []
+    for _ in range(200):
+        out = s.schedule()
+        seen += out.prompt_rows()
+        s.update(out, {r.id: 7 for r in out.sampling_requests()})
+        if not s.has_unfinished():
+            break
+    assert same.num_preemptions > 0 and seen == []
+    assert same.finish_reason == other.finish_reason == "length" and same.num_output == 30
+
+
+def test_every_position_needs_rows_to_spare():
+    s = mk(4, 64, 32)
+    with pytest.raises(ValueError, match="max_logits_rows"):
+        s.add_request(req(1, 10, 2, prompt_logprobs=1))
+    s = mk(4, 64, 32, max_logits_rows=8, enable_chunked_prefill=False)
+    with pytest.raises(ValueError, match="spare rows"):
+        s.add_request(req(1, 10, 2, prompt_logprobs=1))     # 9 rows, 4 to spare, and no cutting
+    s.add_request(req(2, 5, 2, prompt_logprobs=1))          # 4 rows fit
+    assert rows_of(s.schedule()) == ([(2, 0, 5, True)], [(2, 0), (2, 1), (2, 2), (2, 3)])
