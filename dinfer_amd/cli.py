@@ -37,6 +37,9 @@ def _engine_flags(p: argparse.ArgumentParser) -> None:
     p.add_argument("--gemm-tuning", choices=["measured", "heuristic"], default="measured",
                    help="library products: time the library's candidates once per shape at start-up and keep the "
                         "choices in a file (measured), or take its first suggestion (heuristic)")
+    p.add_argument("--max-logits-rows", type=int, default=None,
+                   help="rows of logits a step can return (default: one per live request); --prompt-logprobs needs "
+                        "more than --max-num-seqs")
     p.add_argument("--device", type=int, default=0)
 
 
@@ -49,7 +52,7 @@ def _options(a):
         enable_prefix_caching=a.prefix_caching,
         long_prefill_token_threshold=a.long_prefill_token_threshold,
         prefill_tokens_per_step=a.prefill_tokens_per_step, hip_graph=not a.no_graph, async_scheduling=not a.no_async,
-        device=a.device,
+        device=a.device, max_logits_rows=a.max_logits_rows,
         gemm_tuning=a.gemm_tuning)
 
 
@@ -73,6 +76,10 @@ def main(argv=None) -> int:
     g.add_argument("--seed", type=int, default=None)
     g.add_argument("--stop-token-ids", default="", help="comma-separated extra stop ids")
     g.add_argument("--ignore-eos", action="store_true")
+    g.add_argument("--logprobs", type=int, default=None,
+                   help="with every output token: its log-probability, rank and this many most probable tokens")
+    g.add_argument("--prompt-logprobs", type=int, default=None, help="the same for every prompt token but the first")
+    g.add_argument("--logit-bias", default="", help="token:bias pairs, comma-separated, added to those logits")
 
     r = sub.add_parser("random-weights", help="write a model folder with random weights from a config.json")
     r.add_argument("--config", required=True, help="a config.json of a registered architecture")
@@ -114,10 +121,19 @@ def main(argv=None) -> int:
                         top_k=a.top_k, min_p=a.min_p, repetition_penalty=a.repetition_penalty,
                         frequency_penalty=a.frequency_penalty, presence_penalty=a.presence_penalty, seed=a.seed,
                         stop_token_ids=[int(t) for t in a.stop_token_ids.split(",") if t.strip()],
-                        ignore_eos=a.ignore_eos)
+                        ignore_eos=a.ignore_eos, logprobs=a.logprobs, prompt_logprobs=a.prompt_logprobs,
+                        logit_bias=[(int(t), float(b)) for t, b in (x.split(":") for x in a.logit_bias.split(",") if x.strip())])
+    if a.prompt_logprobs is not None and a.max_logits_rows is None:
+        a.max_logits_rows = a.max_num_seqs + 256
     eng = Engine(a.model, options=_options(a))
-    for p, out in zip(prompts, eng.generate(prompts, sp)):
-        print(json.dumps({"prompt_ids": p, "output_ids": out}))
+    shown = lambda x: None if x is None else {"token_id": x.token_id, "logprob": x.logprob, "rank": x.rank, "top": x.top}
+    for p, g in zip(prompts, eng.generate(prompts, sp, details=True)):
+        rec = {"prompt_ids": p, "output_ids": g.token_ids, "finish_reason": g.finish_reason}
+        if g.logprobs is not None:
+            rec["logprobs"] = [shown(x) for x in g.logprobs]
+        if g.prompt_logprobs is not None:
+            rec["prompt_logprobs"] = [shown(x) for x in g.prompt_logprobs]
+        print(json.dumps(rec))
     return 0
 
 

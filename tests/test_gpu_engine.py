@@ -188,6 +188,18 @@ def test_command_line_generate(model_dirs, tmp_path):
     got = [json.loads(l) for l in p.stdout.splitlines() if l.startswith("{")]
     want = engine(model_dirs[name], name).generate(prompts, SamplingParams(max_tokens=5, temperature=0.0, ignore_eos=True))
     assert [g["prompt_ids"] for g in got] == prompts and [g["output_ids"] for g in got] == want
+    assert all(g["finish_reason"] == "length" and "logprobs" not in g for g in got)
+    forced = want[0][0] + 1
+    p = subprocess.run([sys.executable, str(root / "bin" / "dinfer"), "generate", "--model", str(model_dirs[name]),
+                        "--dtype", "float32", "--max-model-len", "128", "--max-num-seqs", "4", "--block-size", "4",
+                        "--num-blocks", "64", "--prompt-ids", ",".join(map(str, prompts[0])), "--max-tokens", "2",
+                        "--temperature", "0", "--ignore-eos", "--logprobs", "2", "--prompt-logprobs", "0", "--logit-bias",
+                        f"{forced}:100"], capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    g = [json.loads(l) for l in p.stdout.splitlines() if l.startswith("{")][0]
+    assert g["output_ids"] == [forced] * 2 and [x["token_id"] for x in g["logprobs"]] == [forced] * 2
+    assert g["logprobs"][0]["top"][0][0] == want[0][0] and g["logprobs"][0]["rank"] >= 1
+    assert g["prompt_logprobs"][0] is None and [x["token_id"] for x in g["prompt_logprobs"][1:]] == prompts[0][1:]
     p = subprocess.run([sys.executable, str(root / "bin" / "dinfer"), "device-info"], capture_output=True, text=True, timeout=120)
     assert p.returncode == 0 and "gfx950" in json.loads(p.stdout)["arch"]
 
