@@ -876,12 +876,37 @@ constexpr int MAX_TOP = 32;
 // (value, index) pairs in falling order of value, rising index among equals: is (v, i) behind (pv, pi)?
 __device__ __forceinline__ bool behind(float v, int i, float pv, int pi) { return v < pv || (v == pv && i > pi); }
 
+// A row cut into pieces that threads own in turn: where the row is 16-byte aligned the first vocab / 4 pieces are
+// four entries each (one load), the rest (and every entry of an unaligned row) single entries. Piece p belongs to
+// thread p % BLOCK.
+struct Pieces {
+  const float* row;
+  int n4, total;  // pieces of four; all pieces
+  __device__ Pieces(const float* r, int vocab) : row(r) {
+    n4 = ((uintptr_t)r & 15) == 0 ? vocab >> 2 : 0;
+    total = n4 + (vocab - 4 * n4);
+  }
+  __device__ int piece_of(int i) const { return i < 4 * n4 ? i >> 2 : n4 + (i - 4 * n4); }
+  template <class F>
+  __device__ void visit(int p, F&& f) const {  // f(value, index), indices rising
+    if (p < n4) {
+      const f32x4 v = ((const f32x4*)row)[p];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) f(v[e], 4 * p + e);
+    } else {
+      const int i = 4 * n4 + (p - n4);
+      f(row[i], i);
+    }
+  }
+};
+
 // One workgroup a row; k_of[row] < 0: nothing is asked about the row. log-softmax of the row as it is given:
 // column 0 of out_ids / out_lp [rows][stride] takes the chosen token and its log-probability, columns 1..k the k
 // most probable tokens in falling order (equal values: lower index first), rank[row] the number of tokens
-// whose logit is larger than the chosen one's. The k best come from a tournament: every thread names the
-// best of its own entries, the workgroup picks among 1024 names, and only the thread whose entry won
-// looks for its next.
+// whose logit is larger than the chosen one's. One pass over the row gives every thread the best of its own
+// entries, its count of entries larger than the chosen one and its share of the sum (kept relative to its own
+// running maximum). The k best then come from a tournament: the workgroup picks among the 1024 names, and the
+// wave of the thread whose entry won looks through that thread's entries for its next one, a piece a lane.
 __global__ void __launch_bounds__(BLOCK) logprobs_kernel(const float* __restrict__ logits, int64_t ld,
                                                          const int32_t* __restrict__ chosen,
                                                          const int32_t* __restrict__ k_of, int stride,
@@ -892,22 +917,43 @@ __global__ void __launch_bounds__(BLOCK) logprobs_kernel(const float* __restrict
   const int b = blockIdx.x;
   const int k = k_of[b] < stride - 1 ? k_of[b] : stride - 1;
   if (k < 0) return;
-  const float* row = logits + (int64_t)b * ld;
+  const Pieces pc(logits + (int64_t)b * ld, vocab);
   int c = chosen[b];
   c = c < 0 ? 0 : (c >= vocab ? vocab - 1 : c);
-  const float cv = row[c];
-  float best = -INFINITY;
+  const float cv = pc.row[c];
+  float best = -INFINITY, sum = 0.f;  // (best is also the maximum that sum is relative to)
   int besti = 0x7fffffff, larger = 0;
-  for (int i = threadIdx.x; i < vocab; i += BLOCK) {
-    const float v = row[i];
-    better(best, besti, v, i);
-    larger += v > cv;
+  auto take = [&](f32x4 v, int p) {
+    const float pm = fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]));
+    if (pm > best) sum = best == -INFINITY ? 0.f : sum * expf(best - pm);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      better(best, besti, v[e], 4 * p + e);
+      larger += v[e] > cv;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) sum += expf(v[e] - best);
+  };
+  int p = threadIdx.x;
+  for (; p + 3 * BLOCK < pc.n4; p += 4 * BLOCK) {  // four loads in flight
+    const f32x4* r4 = (const f32x4*)pc.row;
+    const f32x4 v0 = r4[p], v1 = r4[p + BLOCK], v2 = r4[p + 2 * BLOCK], v3 = r4[p + 3 * BLOCK];
+    take(v0, p);
+    take(v1, p + BLOCK);
+    take(v2, p + 2 * BLOCK);
+    take(v3, p + 3 * BLOCK);
   }
+  for (; p < pc.total; p += BLOCK)
+    pc.visit(p, [&](float v, int i) {
+      if (v > best) sum = best == -INFINITY ? 0.f : sum * expf(best - v);
+      better(best, besti, v, i);
+      larger += v > cv;
+      sum += expf(v - best);
+    });
+  const float own_top = best;
   float top = 0.f;
   int wi = block_argmax(best, besti, red, &top);
-  float sum = 0.f;
-  for (int i = threadIdx.x; i < vocab; i += BLOCK) sum += expf(row[i] - top);
-  sum = block_sum(sum, fred);
+  sum = block_sum(own_top == -INFINITY ? 0.f : sum * expf(own_top - top), fred);
   const float lse = top + logf(sum);
   const float n_larger = block_sum((float)larger, fred);  // (a count below 2^24 is exact in a float)
   int32_t* ids = out_ids + (int64_t)b * stride;
@@ -917,21 +963,33 @@ __global__ void __launch_bounds__(BLOCK) logprobs_kernel(const float* __restrict
     lps[0] = cv - lse;
     rank[b] = (int)n_larger;
   }
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   float wv = top;
   for (int j = 0; j < k; ++j) {
     if (j > 0) wi = block_argmax(best, besti, red, &wv);
+    const bool none = wi == 0x7fffffff;  // fewer tokens than k
     if (threadIdx.x == 0) {
-      const bool none = wi == 0x7fffffff;  // fewer tokens than k
       ids[1 + j] = none ? -1 : wi;
       lps[1 + j] = none ? -INFINITY : wv - lse;
     }
-    if (wi != 0x7fffffff && wi % BLOCK == (int)threadIdx.x) {  // the winner was this thread's: its next one
-      best = -INFINITY;
-      besti = 0x7fffffff;
-      for (int i = threadIdx.x; i < vocab; i += BLOCK) {
-        const float v = row[i];
-        if (behind(v, i, wv, wi)) better(best, besti, v, i);
-      }
+    if (none) continue;
+    const int owner = pc.piece_of(wi) % BLOCK;
+    if ((owner >> 6) != wave) continue;  // (the same for the whole wave)
+    float nv = -INFINITY;
+    int ni = 0x7fffffff;
+    for (int q = owner + BLOCK * lane; q < pc.total; q += BLOCK * 64)
+      pc.visit(q, [&](float v, int i) {
+        if (behind(v, i, wv, wi)) better(nv, ni, v, i);
+      });
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(nv, o, 64);
+      const int oi = __shfl_xor(ni, o, 64);
+      better(nv, ni, ov, oi);
+    }
+    if (lane == (owner & 63)) {
+      best = nv;
+      besti = ni;
     }
   }
 }
