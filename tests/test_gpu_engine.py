@@ -259,20 +259,23 @@ def test_random_workloads_equal_the_plain_continuations(seed, tmp_path):
     """Requests that arrive over time, share prompt stems (the prefix cache is on where the model allows), are cut
     by small budgets, meet a pool so small that some are preempted, and are aborted now and then; graphs on or off.
     In 32-bit, every request that finishes has generated exactly the plain implementation's greedy continuation,
-    and every page is back at the end."""
+    and every page is back at the end. Some requests ask for the log-probabilities of their outputs or of their
+    prompts (with few rows to spare, so those prompts come in small portions): each value against the plain
+    log-softmax, every prompt position once and in order, and nobody's tokens change."""
     from dinfer_amd import Engine, SamplingParams
     from dinfer_amd.config.qwen3 import Qwen3Config
     from dinfer_amd.weights import write_random_model
-    rng = random.Random(500 + seed)
+    rng, rng2 = random.Random(500 + seed), random.Random(900 + seed)
     name = "ABC"[seed % 3]
     cfgd, page = CONFIGS[name][0], PAGE[name]
     write_random_model(Qwen3Config.from_dict(cfgd), tmp_path, seed=seed, dtype="float32")
     cfg, w = plain.load(tmp_path)
     nblocks = rng.choice([12, 20, 40])
     maxlen = min(cfgd["max_position_embeddings"], nblocks * page)
-    eng = Engine(str(tmp_path), dtype="float32", max_model_len=maxlen, max_num_seqs=rng.choice([2, 4]),
+    seqs = rng.choice([2, 4])
+    eng = Engine(str(tmp_path), dtype="float32", max_model_len=maxlen, max_num_seqs=seqs,
                  max_num_batched_tokens=rng.choice([8, 16, 64]), block_size=page, num_blocks=nblocks,
-                 hip_graph=seed % 2 == 0)
+                 hip_graph=seed % 2 == 0, max_logits_rows=seqs + rng2.choice([1, 3, 8]))
     V = cfgd["vocab_size"]
     stems = [[rng.randrange(V) for _ in range(rng.randint(1, 3 * page))] for _ in range(2)]
     arrivals = []
@@ -282,11 +285,14 @@ def test_random_workloads_equal_the_plain_continuations(seed, tmp_path):
         arrivals.append((rng.randint(0, 12), p[:maxlen - n], n))
     arrivals.sort(key=lambda x: x[0])
     asked, got, aborted, step = {}, {}, set(), 0
+    about, about_prompt, options = {}, {}, {}
     while arrivals or eng.has_unfinished():
         while arrivals and arrivals[0][0] <= step:
             _, p, n = arrivals.pop(0)
-            rid = eng.add_request(p, SamplingParams(max_tokens=n, temperature=0.0, ignore_eos=True))
-            asked[rid], got[rid] = (p, n), []
+            sp = SamplingParams(max_tokens=n, temperature=0.0, ignore_eos=True,
+                                logprobs=rng2.choice([None, None, 0, 2]), prompt_logprobs=rng2.choice([None, None, 0, 1]))
+            rid = eng.add_request(p, sp)
+            asked[rid], got[rid], about[rid], about_prompt[rid], options[rid] = (p, n), [], [], [], sp
         if rng.random() < 0.04 and got:
             victim = rng.choice(list(got))
             if len(got[victim]) < asked[victim][1]:
@@ -295,6 +301,8 @@ def test_random_workloads_equal_the_plain_continuations(seed, tmp_path):
         for o in eng.step():
             if o.token is not None:
                 got[o.request_id].append(o.token)
+                about[o.request_id].append(o.logprobs)
+            about_prompt[o.request_id] += o.prompt_logprobs or []
         step += 1
         assert step < 2000, "the engine makes no progress"
     eng.runner.cache.check()
@@ -302,10 +310,25 @@ def test_random_workloads_equal_the_plain_continuations(seed, tmp_path):
     for rid, (p, n) in asked.items():
         if rid in aborted:
             continue
-        ids = list(p)
-        for _ in range(n):
-            ids.append(int(plain.forward(cfg, w, ids)[-1].argmax()))
+        ids, sp = list(p), options[rid]
+        for i in range(n):
+            row = plain.forward(cfg, w, ids)[-1]
+            ids.append(int(row.argmax()))
+            if sp.logprobs is not None and len(got[rid]) > i and got[rid][i] == ids[-1]:
+                lp = about[rid][i]
+                want = plain.token_logprobs(row, ids[-1], 0)[0]
+                assert lp.token_id == ids[-1] and abs(lp.logprob - want) < 1e-4 and len(lp.top) == sp.logprobs
         assert got[rid] == ids[len(p):], f"request {rid} (prompt of {len(p)}): {got[rid]} != {ids[len(p):]}"
+        if sp.logprobs is None:
+            assert about[rid] == [None] * n
+        if sp.prompt_logprobs is None:
+            assert about_prompt[rid] == []
+        else:
+            assert [pos for pos, _ in about_prompt[rid]] == list(range(1, len(p)))
+            rows = plain.forward(cfg, w, p)
+            for pos, lp in about_prompt[rid]:
+                want = plain.token_logprobs(rows[pos - 1], p[pos], 0)[0]
+                assert lp.token_id == p[pos] and abs(lp.logprob - want) < 1e-4 and len(lp.top) == sp.prompt_logprobs
 
 
 @pytest.mark.parametrize("dtype,graph", [("float32", False), ("bfloat16", True), ("bfloat16", False)])
