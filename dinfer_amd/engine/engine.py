@@ -42,6 +42,9 @@ class Generation:
     prompt_logprobs: list | None   # one per prompt token, None for the first (SamplingParams.prompt_logprobs)
 
 
+_ENDED = {"stop": "request_success_stop", "length": "request_success_length", "abort": "request_abort"}
+
+
 class _Ready:
     """Tokens that are on the host already, in the shape of what Sampler.launch returns."""
 
@@ -82,6 +85,11 @@ class Engine:
         self._running = None
         self._ids = itertools.count()
         self._seeds = random.Random()
+        # counters under the names of the reference's engine metrics (crates/core/src/metrics.rs:63-89)
+        self.counters = {k: 0 for k in ("engine_steps_total", "prompt_tokens_total", "generation_tokens_total",
+                                        "num_preemptions_total", "prefix_cache_hit_tokens_total", "request_success_stop",
+                                        "request_success_length", "request_abort")}
+        self._in_prompt: set = set()        # requests with prompt tokens still to compute (what the counters look at)
         self.phases: dict | None = None     # see measure_phases
 
     # ---- requests ------------------------------------------------------------------------------
@@ -94,11 +102,23 @@ class Engine:
         rid = next(self._ids) if request_id is None else request_id
         seed = sampling.seed if sampling.seed is not None else self._seeds.getrandbits(64)
         self.scheduler.add_request(Request(rid, list(prompt_ids), sampling, seed=seed))
+        self._in_prompt.add(rid)
         return rid
 
     def abort(self, request_id) -> None:
+        if request_id in self.scheduler.requests:
+            self.counters["request_abort"] += 1
         self.scheduler.abort(request_id)
         self.sampler.forget(request_id)
+        self._in_prompt.discard(request_id)
+
+    def stats(self) -> dict:
+        """The counters since the engine was made, and what is true now: requests running and waiting, and the
+        share of the cache's pages in use (of the fullest group)."""
+        cache = self.runner.cache
+        used = [1.0 - cache.num_free(g) / max(spec.num_blocks, 1) for g, spec in enumerate(cache.groups)]
+        return dict(self.counters, num_requests_running=len(self.scheduler.running),
+                    num_requests_waiting=len(self.scheduler.waiting), kv_cache_usage=max(used, default=0.0))
 
     def has_unfinished(self) -> bool:
         return self.scheduler.has_unfinished() or self._running is not None
@@ -130,9 +150,13 @@ class Engine:
         if prompt is not None:      # ((request, position) of the prompt rows, what was found there)
             for (r, pos), lp in zip(prompt[0], prompt[1].logprobs()):
                 about_prompt.setdefault(r.id, []).append((pos + 1, lp))       # the token judged is the next one
+        count = self.counters
         for r, tok, reason in self.scheduler.update(so, tokens):
             outs.append(StepOutput(r.id, tok, reason is not None, reason, about.get(r.id) if tok is not None else None,
                                    about_prompt.get(r.id)))
+            count["generation_tokens_total"] += tok is not None
+            if reason is not None:
+                count[_ENDED[reason]] += 1
         for o in outs:
             if o.finished:
                 self.sampler.forget(o.request_id)
@@ -162,9 +186,26 @@ class Engine:
         if ph is not None:
             ph["schedule"] += time.perf_counter() - t0
         outs = [StepOutput(rid, None, True, reason) for rid, reason in so.force_finished]
+        count = self.counters
+        count["num_preemptions_total"] += len(so.preempted)
+        self._in_prompt.update(so.preempted)        # (they compute their prompts again)
+        for rid, reason in so.force_finished:
+            count[_ENDED[reason]] += 1
+            self._in_prompt.discard(rid)
         if not len(so):
             self._running = None
             return outs
+        count["engine_steps_total"] += 1
+        if self._in_prompt:
+            for x in so.scheduled:
+                r = x.request
+                if r.id not in self._in_prompt:
+                    continue
+                count["prompt_tokens_total"] += max(0, min(x.start + x.num_new, r.num_prompt) - x.start)
+                if x.start and x.start == r.num_cached_tokens:      # admitted in this step with that many found
+                    count["prefix_cache_hit_tokens_total"] += x.start
+                if x.start + x.num_new >= r.num_prompt:
+                    self._in_prompt.discard(r.id)
         sampling = so.sampling_requests()
         greedy = all(r.sampling.picks_largest_logit for r in sampling)
         logits = self.runner.step_planned(self.scheduler, so, greedy=greedy)      # adds to fill and launch itself

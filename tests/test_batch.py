@@ -146,6 +146,18 @@ def test_engine_loop_with_a_stand_in_runner():
     assert eng.runner.cache.num_free() == 32 and not eng.has_unfinished()
     outs = eng.generate([[5] * 47], SamplingParams(max_tokens=10, temperature=0.0))
     assert outs == [[47, 48, 49]]                                           # 49 is eos
+    st = eng.stats()                                                        # the counters of both runs
+    assert (st["prompt_tokens_total"], st["generation_tokens_total"]) == (42 + 47, 9 + 3)
+    assert (st["request_success_length"], st["request_success_stop"], st["request_abort"]) == (3, 1, 0)
+    assert st["engine_steps_total"] == len(eng.runner.steps) and st["num_preemptions_total"] == 0
+    assert (st["num_requests_running"], st["num_requests_waiting"], st["kv_cache_usage"]) == (0, 0, 0.0)
+    eng.add_request([1, 2, 3], SamplingParams(max_tokens=5))
+    eng.add_request(list(range(20)), SamplingParams(max_tokens=5), request_id="b")
+    eng.step()
+    st = eng.stats()
+    assert st["num_requests_running"] + st["num_requests_waiting"] == 2 and st["kv_cache_usage"] > 0
+    eng.abort("b")
+    assert eng.stats()["request_abort"] == 1
 
 
 def test_planned_fill_writes_what_the_entries_would():

@@ -136,6 +136,9 @@ def test_preemption_recomputes_and_gives_the_same_tokens(model_dirs):
     got = tight.generate(prompts, sp)
     assert got == roomy
     assert tight.runner.cache.num_free(0) == 15
+    st = tight.stats()
+    assert st["num_preemptions_total"] >= 1 and st["prompt_tokens_total"] > 90 and st["generation_tokens_total"] == 60
+    assert st["request_success_length"] == 3
     tight.runner.cache.check()
 
 
@@ -231,6 +234,8 @@ def test_prefix_caching_changes_nothing_but_the_work(model_dirs, dtype):
         cached.append(req.num_cached_tokens)
     page = PAGE[name]
     assert cached[0] == 0 and all(c == 40 // page * page for c in cached[1:]), cached
+    assert eng.stats()["prefix_cache_hit_tokens_total"] == sum(cached)
+    assert eng.stats()["prompt_tokens_total"] == sum(len(p) for p in prompts) - sum(cached)
     got += eng.generate(prompts, sp)        # all together: pages shared between live requests
     if dtype == "float32":
         assert got == want
