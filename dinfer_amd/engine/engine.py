@@ -42,6 +42,17 @@ class Generation:
     prompt_logprobs: list | None   # one per prompt token, None for the first (SamplingParams.prompt_logprobs)
 
 
+@dataclass
+class _InFlight:
+    """A step that has been launched and whose tokens have not been read yet."""
+    plan: object                    # the scheduler's plan of the step
+    sampled: object                 # Sampler.launch's handle: the tokens on their way
+    events: tuple | None            # device events around the model's kernels (while phases are measured)
+    asking: list | None             # the sampled rows' requests, if one of them wants log-probabilities
+    prompt_rows: list | None        # [(request, position)] of the prompt positions judged in this step
+    prompt_found: object = None     # Sampler.about_rows' handle for them
+
+
 _ENDED = {"stop": "request_success_stop", "length": "request_success_length", "abort": "request_abort"}
 
 
@@ -80,9 +91,7 @@ class Engine:
         # the host has read them
         last = getattr(getattr(self.runner, "batch", None), "last_tokens", None)
         self.sampler = Sampler(self.runner.device, self.runner.max_rows, spec.vocab_size, out=last)
-        # the step in flight: (plan, tokens on their way, device events, the sampled rows' requests if any wants
-        # logprobs, the prompt rows and what is found at them)
-        self._running = None
+        self._running: _InFlight | None = None      # the step whose tokens are read next
         self._ids = itertools.count()
         self._seeds = random.Random()
         # counters under the names of the reference's engine metrics (crates/core/src/metrics.rs:63-89)
@@ -141,17 +150,18 @@ class Engine:
                 outs += self._launch(ahead=True)        # (a plan ahead ends nobody: nothing is added)
             finally:                                    # whatever happened, the running step is still the running step
                 self._running, nxt = held, self._running
-        so, sampled, events, asking, prompt = self._running
-        tokens = sampled.tokens()
+        run = self._running
+        events = run.events
+        tokens = run.sampled.tokens()
         t0 = time.perf_counter() if ph is not None else 0.0
         about, about_prompt = {}, {}
-        if asking is not None:      # the requests of the sampled rows, where one of them wants log-probabilities
-            about = {r.id: lp for r, lp in zip(asking, sampled.logprobs()) if lp is not None}
-        if prompt is not None:      # ((request, position) of the prompt rows, what was found there)
-            for (r, pos), lp in zip(prompt[0], prompt[1].logprobs()):
+        if run.asking is not None:
+            about = {r.id: lp for r, lp in zip(run.asking, run.sampled.logprobs()) if lp is not None}
+        if run.prompt_rows:
+            for (r, pos), lp in zip(run.prompt_rows, run.prompt_found.logprobs()):
                 about_prompt.setdefault(r.id, []).append((pos + 1, lp))       # the token judged is the next one
         count = self.counters
-        for r, tok, reason in self.scheduler.update(so, tokens):
+        for r, tok, reason in self.scheduler.update(run.plan, tokens):
             outs.append(StepOutput(r.id, tok, reason is not None, reason, about.get(r.id) if tok is not None else None,
                                    about_prompt.get(r.id)))
             count["generation_tokens_total"] += tok is not None
@@ -175,7 +185,7 @@ class Engine:
         penalty counts the tokens seen so far)."""
         if not self.options.async_scheduling or not self.scheduler.can_look_ahead():
             return False
-        return not any(r.sampling.has_penalties for r in self._running[0].requests)
+        return not any(r.sampling.has_penalties for r in self._running.plan.requests)
 
     def _launch(self, ahead: bool) -> list[StepOutput]:
         """Plans a step and issues it and its sampling; what is in flight afterwards is in _running (None: nothing
@@ -219,13 +229,13 @@ class Engine:
         else:
             sampled = _Ready(self.sampler.sample(ours, rows))
         asking = sampling if any(r.sampling.logprobs is not None for r in sampling) else None
-        prompt = so.prompt_rows()
+        prompt, found = so.prompt_rows(), None
         if prompt:      # their logits follow the sampling rows
             found = self.sampler.about_rows(logits[len(rows):len(rows) + len(prompt)],
                                             [r.prompt_ids[p + 1] for r, p in prompt],
                                             [r.sampling.prompt_logprobs for r, _ in prompt])
-            prompt = (prompt, found)
-        self._running = (so, sampled, self.runner.take_gpu_events() if ph is not None else None, asking, prompt or None)
+        self._running = _InFlight(so, sampled, self.runner.take_gpu_events() if ph is not None else None, asking,
+                                  prompt, found)
         return outs
 
     def measure_phases(self, on: bool = True) -> None:
