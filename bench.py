@@ -3,6 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L] [--shape 8b|14b|32b|0.6b]
                     [--prompt P] [--context C] [--workload decode|serving [--sampled]]
+    python bench.py --workload closed --shape 0.6b --concurrency 8 --prompt 128 --max-tokens 128 [--num-requests N]
 
 Prints ONE JSON line. `value` is decoded tokens per second at the default batch (8), each
 request with a 2,048-token prompt in a 4,096-token context; a "step" is one decode step
@@ -136,6 +137,66 @@ def serving(a, torch, Engine, SamplingParams, Qwen3Config) -> int:
     return 0
 
 
+def closed(a, torch, Engine, SamplingParams, Qwen3Config) -> int:
+    """The load of the reference's own serving bench without the server (bins/bench/src/main.rs:1-16,
+    scripts/verify/bench_compare.sh:36-66): `concurrency` requests are live at any time, each with a fresh prompt of
+    `prompt` random tokens and `max_tokens` greedy outputs (eos ignored); when one ends the next is added, until
+    `num_requests` (default: four per worker, at least 16) are done. The first two requests of every worker's
+    worth are not special here: the whole workload runs once untimed first (kernel loads, product shapes, graphs).
+    TTFT = first token on the host - arrival; TPOT = (latency - TTFT) / (outputs - 1)."""
+    sizes = {**SIZES, **SHAPES[a.shape]}
+    if a.layers:
+        sizes["num_hidden_layers"] = a.layers
+    cfg = Qwen3Config.from_dict(sizes)
+    c, P, O = a.concurrency, a.prompt, a.max_tokens
+    n_req = a.num_requests or max(16, 4 * c)
+    ctx = -(-(P + O + 1) // 16) * 16
+    eng = Engine(config=cfg, seed=0, dtype=a.dtype, max_model_len=ctx, max_num_seqs=c, max_num_batched_tokens=max(2048, P),
+                 block_size=16, num_blocks=c * ctx // 16 + 64, hip_graph=not a.no_hip_graph)
+    rng = random.Random(0)
+    sp = SamplingParams(max_tokens=O, temperature=0.0, ignore_eos=True)
+
+    def run():
+        arrived, first, ended, outs = {}, {}, {}, {}
+        added = 0
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        while added < n_req or eng.has_unfinished():
+            while added < n_req and len(arrived) - len(ended) < c:
+                rid = eng.add_request([rng.randrange(cfg.vocab_size) for _ in range(P)], sp)
+                arrived[rid], outs[rid] = time.perf_counter(), 0
+                added += 1
+            got = eng.step()
+            now = time.perf_counter()
+            for o in got:
+                if o.token is not None:
+                    outs[o.request_id] += 1
+                    first.setdefault(o.request_id, now)
+                if o.finished:
+                    ended[o.request_id] = now
+        dt = time.perf_counter() - t0
+        ttft = sorted((first[r] - arrived[r]) * 1e3 for r in arrived)
+        tpot = sorted((ended[r] - first[r]) / (outs[r] - 1) * 1e3 for r in arrived if outs[r] > 1)
+        lat = sorted((ended[r] - arrived[r]) * 1e3 for r in arrived)
+        return dt, sum(outs.values()), ttft, tpot, lat
+
+    run()
+    dt, n_out, ttft, tpot, lat = run()
+    pct = lambda xs, q: round(xs[min(len(xs) - 1, int(q * len(xs)))], 3) if xs else None
+    print(json.dumps({
+        "metric": f"output tokens/s, closed loop (Qwen3-{a.shape.upper()} shape, {c} live requests, prompts of {P}, {O} outputs each)",
+        "value": round(n_out / dt, 1), "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True, "vs_baseline": None,
+        "dtype": "bf16" if a.dtype == "bfloat16" else "fp32", "data": "synthetic", "seconds": round(dt, 3),
+        "requests": n_req, "requests_per_s": round(n_req / dt, 2), "output_tokens": n_out,
+        "total_tokens_per_s": round((n_out + n_req * P) / dt, 1),
+        "ttft_ms": {"p50": pct(ttft, 0.5), "p99": pct(ttft, 0.99)}, "tpot_ms": {"p50": pct(tpot, 0.5), "p99": pct(tpot, 0.99)},
+        "latency_ms": {"p50": pct(lat, 0.5)}, "counters": eng.stats(),
+        "config": {"model": f"Qwen3-{a.shape.upper()} shape, random weights", "layers": sizes["num_hidden_layers"],
+                   "concurrency": c, "prompt_len": P, "max_tokens": O, "context": ctx, "parallelism": "single GPU",
+                   "in_process": True}}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -150,9 +211,14 @@ def main() -> int:
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="layer sizes (default: Qwen3-8B)")
     ap.add_argument("--prompt", type=int, default=DEFAULT_PROMPT, help="prompt tokens per request (and of the timed prefill)")
     ap.add_argument("--context", type=int, default=DEFAULT_CONTEXT, help="max_model_len the engine is built for")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serving"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "closed"],
                     help="serving: 32 requests with prompts of 512 to 3,072 tokens fed in portions of 512 beside the "
-                         "requests that decode, 256 outputs each (meant for the 14B shape); its own JSON line")
+                         "requests that decode, 256 outputs each (meant for the 14B shape); closed: --concurrency "
+                         "requests live at any time, --prompt tokens in and --max-tokens out each, the load of the "
+                         "reference's own serving bench without the server; each its own JSON line")
+    ap.add_argument("--concurrency", type=int, default=8, help="closed: live requests")
+    ap.add_argument("--max-tokens", type=int, default=128, help="closed: outputs per request")
+    ap.add_argument("--num-requests", type=int, default=0, help="closed: requests in all (0: four per live request, at least 16)")
     ap.add_argument("--runs", type=int, default=2,
                     help="serving: the workload runs this many times on one engine and the last run is reported")
     ap.add_argument("--sampled", action="store_true",
@@ -167,6 +233,8 @@ def main() -> int:
     from dinfer_amd.config.qwen3 import Qwen3Config
     if a.workload == "serving":
         return serving(a, torch, Engine, SamplingParams, Qwen3Config)
+    if a.workload == "closed":
+        return closed(a, torch, Engine, SamplingParams, Qwen3Config)
 
     sizes = {**SIZES, **SHAPES[a.shape]}
     PROMPT, CONTEXT = a.prompt, a.context
