@@ -314,6 +314,68 @@ __global__ void __launch_bounds__(BLOCK) argmax_kernel(const float* __restrict__
   if (threadIdx.x == 0) out[blockIdx.x] = c;
 }
 
+// The same argmax with a row spread over many workgroups (a row of 152k entries is 600 KB: one workgroup needs
+// 16 us for it, whatever the batch): every workgroup names the best of ARG_SEG entries, a second launch picks among
+// the names. Both compare like row_argmax, so the result is the same index.
+constexpr int ARG_SEG = 4096;
+constexpr int ARG_THREADS = 256;
+
+__global__ void __launch_bounds__(ARG_THREADS) argmax_parts_kernel(const float* __restrict__ logits, int64_t ld,
+                                                                   float* __restrict__ part_val,
+                                                                   int32_t* __restrict__ part_idx, int vocab, int segs) {
+  __shared__ float sv[ARG_THREADS / 64];
+  __shared__ int si[ARG_THREADS / 64];
+  const int r = blockIdx.y, s = blockIdx.x;
+  const float* row = logits + (int64_t)r * ld;
+  const int lo = s * ARG_SEG, hi = min(vocab, lo + ARG_SEG);
+  float best = -INFINITY;
+  int besti = 0x7fffffff;
+  if (((uintptr_t)(row + lo) & 15) == 0) {
+    const f32x4* r4 = (const f32x4*)(row + lo);
+    const int n4 = (hi - lo) >> 2;
+    for (int j = threadIdx.x; j < n4; j += ARG_THREADS) {  // (ARG_SEG / 4 / ARG_THREADS = 4 loads a thread, unrolled)
+      const f32x4 v = r4[j];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) better(best, besti, v[e], lo + 4 * j + e);
+    }
+    for (int i = lo + 4 * n4 + threadIdx.x; i < hi; i += ARG_THREADS) better(best, besti, row[i], i);
+  } else {
+    for (int i = lo + threadIdx.x; i < hi; i += ARG_THREADS) better(best, besti, row[i], i);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(best, o, 64);
+    const int oi = __shfl_xor(besti, o, 64);
+    better(best, besti, ov, oi);
+  }
+  if ((threadIdx.x & 63) == 0) {
+    sv[threadIdx.x >> 6] = best;
+    si[threadIdx.x >> 6] = besti;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < ARG_THREADS / 64; ++w) better(best, besti, sv[w], si[w]);
+    part_val[(int64_t)r * segs + s] = best;
+    part_idx[(int64_t)r * segs + s] = besti;
+  }
+}
+
+__global__ void __launch_bounds__(64) argmax_join_kernel(const float* __restrict__ part_val,
+                                                         const int32_t* __restrict__ part_idx,
+                                                         int32_t* __restrict__ out, int segs) {
+  const int r = blockIdx.x;
+  float best = -INFINITY;
+  int besti = 0x7fffffff;
+  for (int s = threadIdx.x; s < segs; s += 64) better(best, besti, part_val[(int64_t)r * segs + s], part_idx[(int64_t)r * segs + s]);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(best, o, 64);
+    const int oi = __shfl_xor(besti, o, 64);
+    better(best, besti, ov, oi);
+  }
+  if (threadIdx.x == 0) out[r] = besti == 0x7fffffff ? 0 : besti;
+}
+
 // One entry per distinct token of a row's history: ids[e], count among the
 // outputs cnt[e] (0 if it occurs in the prompt only). Row b owns the entries
 // offsets[b] .. offsets[b+1].
@@ -996,10 +1058,29 @@ __global__ void __launch_bounds__(BLOCK) logprobs_kernel(const float* __restrict
 
 }  // namespace
 
+// Bytes of scratch with which dinfer_argmax spreads a row over many workgroups.
+extern "C" int dinfer_argmax_scratch_bytes(int64_t rows, int64_t vocab, int64_t* bytes) {
+  if (rows <= 0 || vocab <= 0 || !bytes) return ERR_BAD_SHAPE;
+  *bytes = rows * ((vocab + ARG_SEG - 1) / ARG_SEG) * 8;
+  return OK;
+}
+
+// out[r] = index of the largest entry of row r (the lowest such index). scratch (device memory, 4-byte aligned, may
+// be null): with dinfer_argmax_scratch_bytes of it a long row is spread over many workgroups in two launches;
+// without it, or for short rows, one workgroup takes a row.
 extern "C" int dinfer_argmax(const float* logits, int64_t ld, int32_t* out, int64_t rows, int64_t vocab,
-                             hipStream_t stream) {
+                             void* scratch, int64_t scratch_bytes, hipStream_t stream) {
   if (rows <= 0) return OK;
   if (vocab <= 0 || vocab > (1 << 24) || ld < vocab || rows > 0x7fffffff) return ERR_BAD_SHAPE;
+  const int64_t segs = (vocab + ARG_SEG - 1) / ARG_SEG;
+  if (scratch && segs >= 4 && rows <= 65535 && scratch_bytes >= rows * segs * 8 && ((uintptr_t)scratch & 3) == 0) {
+    float* val = (float*)scratch;
+    int32_t* idx = (int32_t*)(val + rows * segs);
+    argmax_parts_kernel<<<dim3((unsigned)segs, (unsigned)rows), ARG_THREADS, 0, stream>>>(logits, ld, val, idx, (int)vocab,
+                                                                                         (int)segs);
+    argmax_join_kernel<<<(unsigned)rows, 64, 0, stream>>>(val, idx, out, (int)segs);
+    return launch_status();
+  }
   argmax_kernel<<<(unsigned)rows, BLOCK, 0, stream>>>(logits, ld, out, (int)vocab);
   return launch_status();
 }

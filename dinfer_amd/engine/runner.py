@@ -90,6 +90,7 @@ class ModelRunner:
         sizes = {1 << i for i in range(top.bit_length() + 1)} | {24, 40, 48, 56} | {3 << i for i in range(5, top.bit_length())}
         self._buckets = sorted({min(x, top) for x in sizes})
         self._graphs: dict[tuple, torch.cuda.CUDAGraph] = {}   # (bucket, finds the best tokens itself) -> graph
+        self._argmax_scratch: torch.Tensor | None = None       # made in the eager step before the first such capture
         self.phases: dict | None = None     # Engine.measure_phases
         self._events = None
         self._graph_pool = None
@@ -322,7 +323,9 @@ class ModelRunner:
         def forward():
             logits = self.model.forward(b, self.cache_views)
             if greedy:      # (padded rows find a token as well; nobody reads it)
-                ops.argmax(logits, b.last_tokens, bucket)
+                if self._argmax_scratch is None:
+                    self._argmax_scratch = ops.argmax_scratch(self.max_rows, logits.shape[1], self.device)
+                ops.argmax(logits, b.last_tokens, bucket, self._argmax_scratch)
 
         forward()
         torch.cuda.synchronize()

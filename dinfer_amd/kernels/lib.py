@@ -58,7 +58,8 @@ SIGNATURES = {
     "dinfer_gemm_mid_m_static_init": ("gemm_mid", []),
     "dinfer_stream_read": ("ceilings", [_P, _L, _I, _P, _P]),
     "dinfer_mfma_loop": ("ceilings", [_I, _I, _P, _P, _P]),
-    "dinfer_argmax": ("sampling", [_P, _L, _P, _L, _L, _P]),
+    "dinfer_argmax": ("sampling", [_P, _L, _P, _L, _L, _P, _L, _P]),
+    "dinfer_argmax_scratch_bytes": ("sampling", [_L, _L, _P]),
     "dinfer_sample": ("sampling", [_P, _L, _P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _P]),
     "dinfer_sample_rows": ("sampling", [_P, _L, _P, _P, _L, _P, _P, _L, _L, _I, _I, _P]),
     "dinfer_sample_scratch_bytes": ("sampling", [_L, _L, _P]),

@@ -398,10 +398,21 @@ def gemm_mid_m(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, work
     return out
 
 
-def argmax(logits: torch.Tensor, out: torch.Tensor, rows: int) -> torch.Tensor:
-    _need_gpu(logits, out)
+def argmax_scratch(rows: int, vocab: int, device) -> torch.Tensor:
+    """The scratch with which argmax spreads each of up to `rows` rows over many workgroups."""
+    n = ctypes.c_int64(0)
+    lib.call("dinfer_argmax_scratch_bytes", rows, vocab, ctypes.addressof(n))
+    return torch.empty(n.value, dtype=torch.uint8, device=device)
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor, rows: int, scratch: torch.Tensor | None = None) -> torch.Tensor:
+    """out[r] = the index of the largest of logits[r] (the lowest such index). scratch (argmax_scratch): a long row
+    is spread over many workgroups instead of taken by one."""
+    _need_gpu(logits, out, scratch)
     assert logits.dtype == torch.float32 and out.dtype == torch.int32 and out.numel() >= rows
-    lib.call("dinfer_argmax", logits.data_ptr(), _rows(logits), out.data_ptr(), rows, logits.shape[1], _stream())
+    assert scratch is None or (scratch.dtype == torch.uint8 and scratch.is_contiguous())
+    lib.call("dinfer_argmax", logits.data_ptr(), _rows(logits), out.data_ptr(), rows, logits.shape[1], _ptr(scratch),
+             0 if scratch is None else scratch.numel(), _stream())
     return out
 
 

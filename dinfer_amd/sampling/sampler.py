@@ -63,6 +63,7 @@ class Sampler:
         # two launches may be in flight (a step planned ahead of the one that runs): what the host fills or reads
         # alternates between two pinned buffers (made at the first launch)
         self._tokens_host: list | None = None
+        self._arg_scratch: torch.Tensor | None = None    # the argmax kernels' own memory between their two launches
         self._read: list | None = None
         self._turn = 0
         # made on first non-greedy use: [max_rows, vocab] float32 for rows that take the one-workgroup path,
@@ -130,7 +131,9 @@ class Sampler:
             given[:R].copy_(logits[:R])
         if all(p.picks_largest_logit for p, *_ in rows):
             if not done:
-                ops.argmax(logits, self.out, R)
+                if self._arg_scratch is None:
+                    self._arg_scratch = ops.argmax_scratch(self.max_rows, self.vocab, self.device)
+                ops.argmax(logits, self.out, R, self._arg_scratch)
         else:
             assert not done
             if any(p.logit_bias for p, *_ in rows):         # before the penalties (sampling.cu:286)

@@ -419,16 +419,30 @@ def test_attention_window_edge(kernel, inside):
 
 
 # ---- sampling -------------------------------------------------------------------------------------
-def test_argmax_ties_to_lowest_index():
-    V = 163841
-    logits = torch.randn(6, V, device=DEV) * 3
-    logits[2, 100] = logits[2, 90000] = 50.0
+@pytest.mark.parametrize("V", [163841, 16385, 4096 * 4, 1000])
+@pytest.mark.parametrize("spread", [False, True])
+def test_argmax_ties_to_lowest_index(V, spread):
+    """One workgroup a row, and a row spread over many workgroups in two launches (long rows, with scratch): equal
+    entries go to the lowest index, also across the pieces; a row of -inf gives 0; rows that start at any alignment."""
+    logits = torch.randn(7, V, device=DEV) * 3
+    logits[2, 100] = logits[2, V - 7] = 50.0
     logits[3, :] = 1.0
-    out = torch.empty(6, device=DEV, dtype=torch.int32)
-    ops().argmax(logits, out, 6)
+    logits[4, :] = float("-inf")
+    logits[5, V - 1] = 60.0                     # in the last, short piece
+    logits[6, 4095:4097] = 70.0 if V > 4097 else logits[6, 4095:4097]     # across a piece's edge
+    out = torch.full((7,), -1, device=DEV, dtype=torch.int32)
+    scratch = ops().argmax_scratch(7, V, DEV) if spread else None
+    ops().argmax(logits, out, 7, scratch)
     want = logits.argmax(-1).tolist()
-    want[2], want[3] = 100, 0
+    want[2], want[3], want[4], want[5] = 100, 0, 0, V - 1
+    if V > 4097:
+        want[6] = 4095
     assert out.tolist() == want
+    if spread:      # fewer rows than the scratch was made for, and a view with a row stride of its own
+        wide = torch.randn(3, V + 13, device=DEV)
+        view = wide[:, 5:5 + V]
+        ops().argmax(view, out, 3, scratch)
+        assert out[:3].tolist() == view.argmax(-1).tolist()
 
 
 PATHS = ["one_workgroup", "spread", "spread_forced_generic"]
