@@ -90,7 +90,10 @@ class Engine:
         # the sampled tokens land where the next step can take them from as its input, if it is launched before
         # the host has read them
         last = getattr(getattr(self.runner, "batch", None), "last_tokens", None)
-        self.sampler = Sampler(self.runner.device, self.runner.max_rows, spec.vocab_size, out=last)
+        # a step samples one row per request at most; the rows beyond that are prompt positions to be judged
+        rows = self.runner.max_rows
+        self.sampler = Sampler(self.runner.device, min(rows, self.options.max_num_seqs), spec.vocab_size, out=last,
+                               max_judged=rows)
         self._running: _InFlight | None = None      # the step whose tokens are read next
         self._ids = itertools.count()
         self._seeds = random.Random()

@@ -54,10 +54,12 @@ class Sampled:
 
 
 class Sampler:
-    def __init__(self, device, max_rows: int, vocab: int, out: torch.Tensor | None = None):
-        """out: int32 [>= max_rows] on the device where the sampled tokens are to land (the engine names the buffer
-        that the next step may take its input tokens from); made here if absent."""
+    def __init__(self, device, max_rows: int, vocab: int, out: torch.Tensor | None = None, max_judged: int | None = None):
+        """max_rows: the most rows a launch samples. out: int32 [>= max_rows] on the device where the sampled tokens
+        are to land (the engine names the buffer that the next step may take its input tokens from); made here if
+        absent. max_judged: the most rows about_rows() is asked about at once (default: max_rows)."""
         self.device, self.max_rows, self.vocab = device, max_rows, vocab
+        self.max_judged = max(max_rows, max_judged or 0)
         self.out = out if out is not None else torch.empty(max_rows, dtype=torch.int32, device=device)
         assert self.out.dtype == torch.int32 and self.out.numel() >= max_rows
         # two launches may be in flight (a step planned ahead of the one that runs): what the host fills or reads
@@ -164,12 +166,12 @@ class Sampler:
         SamplingParams.prompt_logprobs). Returns at once; logprobs() of what comes back waits. At most two of these
         may be waiting at a time."""
         R = len(targets)
-        assert logits.shape[0] == R == len(asked) and R <= self.max_rows and all(k is not None for k in asked)
+        assert logits.shape[0] == R == len(asked) and R <= self.max_judged and all(k is not None for k in asked)
         if R == 0:
             return Sampled(self, 0, None, None)
         if self._given is None:
-            self._given = [torch.empty(self.max_rows, dtype=torch.int32, pin_memory=True) for _ in range(2)]
-            self._given_dev = torch.empty(self.max_rows, dtype=torch.int32, device=self.device)
+            self._given = [torch.empty(self.max_judged, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+            self._given_dev = torch.empty(self.max_judged, dtype=torch.int32, device=self.device)
             self._given_read = [torch.cuda.Event(), torch.cuda.Event()]
         turn = self._given_turn
         self._given_turn ^= 1
@@ -194,15 +196,15 @@ class Sampler:
         caller's event has passed)."""
         stride = MAX_LOGPROBS + 1
         if self._about_dev is None:
-            dev = dict(device=self.device)
-            self._about_dev = (torch.empty(self.max_rows, dtype=torch.int32, **dev),                # k per row
-                               torch.empty((self.max_rows, stride), dtype=torch.int32, **dev),
-                               torch.empty((self.max_rows, stride), dtype=torch.float32, **dev),
-                               torch.empty(self.max_rows, dtype=torch.int32, **dev))
-            self._about_host = [(torch.empty(self.max_rows, dtype=torch.int32, pin_memory=True),
-                                 torch.empty((self.max_rows, stride), dtype=torch.int32, pin_memory=True),
-                                 torch.empty((self.max_rows, stride), dtype=torch.float32, pin_memory=True),
-                                 torch.empty(self.max_rows, dtype=torch.int32, pin_memory=True)) for _ in range(4)]
+            dev, n = dict(device=self.device), self.max_judged
+            self._about_dev = (torch.empty(n, dtype=torch.int32, **dev),                # k per row
+                               torch.empty((n, stride), dtype=torch.int32, **dev),
+                               torch.empty((n, stride), dtype=torch.float32, **dev),
+                               torch.empty(n, dtype=torch.int32, **dev))
+            self._about_host = [(torch.empty(n, dtype=torch.int32, pin_memory=True),
+                                 torch.empty((n, stride), dtype=torch.int32, pin_memory=True),
+                                 torch.empty((n, stride), dtype=torch.float32, pin_memory=True),
+                                 torch.empty(n, dtype=torch.int32, pin_memory=True)) for _ in range(4)]
         k_dev, ids_dev, lp_dev, rank_dev = self._about_dev
         k_host, ids_host, lp_host, rank_host = self._about_host[turn]
         k_host[:R] = torch.tensor([-1 if k is None else k for k in asked], dtype=torch.int32)
