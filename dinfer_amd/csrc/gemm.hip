@@ -100,12 +100,16 @@ struct NormLink {
 // GATED (RT == 2): W is [2N, K], rows [0, N) the gate and [N, 2N) the up projection; the workgroup's
 // two row tiles are gate rows n0.. and up rows N + n0.., and the epilogue stores
 // silu(gate) * up into C [M, N]: the activation costs no pass of its own.
-template <int MT, int RT, class O, bool GATED, bool STREAM, int MODE = PLAIN>
+// CUT (not GATED, not SINK): the last 8 rows of the workgroup's last tile are left out, so a workgroup takes
+// 16 RT - 8 weight rows: with two tiles 24 rows, which makes 256 workgroups of N = 6,144 where 32 rows make 192.
+template <int MT, int RT, class O, bool GATED, bool STREAM, int MODE = PLAIN, bool CUT = false>
 __global__ void __launch_bounds__(1024) gemm_small_m_kernel(const bf16* __restrict__ A, int64_t lda,
                                                             const bf16* __restrict__ W, int64_t ldw,
                                                             O* __restrict__ C, int64_t ldc, int M, int N, int K,
                                                             NormLink link = NormLink{}) {
   static_assert(!GATED || RT == 2, "the gated form pairs one gate tile with one up tile");
+  static_assert(!CUT || (!GATED && MODE != SINK), "the cut form is for the plain and the scaled product");
+  constexpr int ROWS = 16 * RT - (CUT ? 8 : 0);  // weight rows of a workgroup (not GATED)
   // 64-wide k steps in flight per wave: as many as the register file takes at 16 waves a workgroup
   constexpr int UNROLL = MT <= 2 ? (4 / RT > 0 ? 4 / RT : 1) : (2 / RT > 0 ? 2 / RT : 1);
   constexpr int ROW_BYTES = 144;              // 64 k of a row and 16 bytes of padding
@@ -115,7 +119,8 @@ __global__ void __launch_bounds__(1024) gemm_small_m_kernel(const bf16* __restri
   const int nw = blockDim.x >> 6;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, i16 = lane & 15, g4 = lane >> 4;
   const int lrow = lane >> 3, lpiece = lane & 7;  // what this lane loads: piece lpiece of rows lrow and lrow + 8
-  const int n0 = GATED ? blockIdx.x * 16 : blockIdx.x * 16 * RT;
+  const int n0 = GATED ? blockIdx.x * 16 : blockIdx.x * ROWS;
+  const int n_end = GATED ? N : (n0 + ROWS < N ? n0 + ROWS : N);  // rows from here on are not this workgroup's
   char* strip = smem + wave * STRIP_BYTES;
   char* put = strip + lrow * ROW_BYTES + lpiece * 16;  // where this lane's loads go (rows lrow, + 8)
   const char* get = strip + i16 * ROW_BYTES + g4 * 16;  // its MFMA operands: row i16, pieces g4 and 4 + g4
@@ -180,7 +185,8 @@ __global__ void __launch_bounds__(1024) gemm_small_m_kernel(const bf16* __restri
 #pragma unroll
       for (int r = 0; r < RT; ++r)
 #pragma unroll
-        for (int h = 0; h < 2; ++h) wraw[u][r][h] = ok ? ld_weight<STREAM>(wp[r][h] + kk) : zero8();
+        for (int h = 0; h < 2; ++h)
+          wraw[u][r][h] = (CUT && r == RT - 1 && h == 1) ? zero8() : (ok ? ld_weight<STREAM>(wp[r][h] + kk) : zero8());
 #pragma unroll
       for (int t = 0; t < MT; ++t)
 #pragma unroll
@@ -296,10 +302,10 @@ __global__ void __launch_bounds__(1024) gemm_small_m_kernel(const bf16* __restri
       if ((ln >> 4) == 0 && m < M) link.stats_out[(int64_t)m * link.ld_stats + (n0 >> 4) + r] = ss;
     } else if (m < M) {
       O* cp = C + (int64_t)m * ldc + n;
-      if (n + 3 < N) {
+      if (n + 3 < n_end) {
         store4<O>(cp, s);
       } else {
-        for (int e = 0; e < 4 && n + e < N; ++e) cp[e] = from_f32<O>(s[e]);
+        for (int e = 0; e < 4 && n + e < n_end; ++e) cp[e] = from_f32<O>(s[e]);
       }
     }
   }
@@ -348,11 +354,26 @@ int dispatch(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, O* C, int64
 }
 
 // The SCALED and SINK forms: up to 32 rows, bf16 out, one or two row tiles.
+// Two row tiles a workgroup leave CUs without work (fewer than 256 workgroups) where 24 rows a workgroup would not
+// (measured on weights taken in turn, K = 4,096: N = 6,144 in 256 workgroups 12.4 us at 8 tokens, N = 6,176 in 193
+// workgroups of 32 rows 13.2; 11.5 against 12.2 at one token, 13.7 against 15.0 at 16).
+inline bool cut_pays(int N) { return N / 32 < 256 && (N + 23) / 24 <= 256; }
+
 template <int MT, int RT, int MODE>
 int launch_linked(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, bf16* C, int64_t ldc, int M, int N, int K,
                   int waves, const NormLink& link, hipStream_t stream) {
   const int row_tiles = (N + 16 * RT - 1) / (16 * RT);
   const size_t lds = lds_bytes(waves, RT, MT) + RS_BYTES;
+  if constexpr (MODE == SCALED && RT == 2 && MT == 1) {
+    if (cut_pays(N)) {
+      const unsigned blocks = (unsigned)((N + 23) / 24);
+      if (streams_weight(N, K))
+        gemm_small_m_kernel<MT, RT, bf16, false, true, MODE, true><<<blocks, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, link);
+      else
+        gemm_small_m_kernel<MT, RT, bf16, false, false, MODE, true><<<blocks, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, link);
+      return launch_status();
+    }
+  }
   if (streams_weight(N, K))
     gemm_small_m_kernel<MT, RT, bf16, false, true, MODE><<<(unsigned)row_tiles, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, link);
   else

@@ -818,9 +818,11 @@ def test_gemm_small_m_gated(M):
 def test_gemm_small_m_carries_the_norm(M):
     """A product that adds into the residual stream and leaves what the next RMSNorm needs (the stream times the gain,
     sums of squares per 16 columns), and the product that takes those: together they equal add, norm and product, to
-    rounding, at widths that are no multiples of the tiles, with the gain in either dtype and an offset."""
+    rounding, at widths that are no multiples of the tiles, with the gain in either dtype and an offset. (Consumers of
+    4,097 to 6,144 outputs take 24 weight rows a workgroup at up to 16 tokens: 6,144, 5,000 and 4,120 end their last
+    workgroup at 24, 8 and 16 rows.)"""
     eps = 1e-5
-    for N, K, N2 in ((96, 512, 136), (328, 80, 1000), (4096, 4096, 6144), (1000, 1096, 50)):
+    for N, K, N2 in ((96, 512, 136), (328, 80, 1000), (4096, 4096, 6144), (1000, 1096, 50), (200, 64, 5000), (72, 128, 4120)):
         for gain_dtype, offset in ((torch.float32, 0.0), (torch.bfloat16, 1.0)):
             a = torch.randn(M, K, device=DEV).to(torch.bfloat16)
             w = (torch.randn(N, K, device=DEV) * 0.05).to(torch.bfloat16)
