@@ -316,11 +316,26 @@ inline bool streams_weight(int64_t rows, int64_t K) { return rows * K * (int64_t
 inline size_t lds_bytes(int waves, int rt, int mt) { return lds_core_bytes(waves, rt, mt); }
 constexpr size_t RS_BYTES = 64 * sizeof(float);  // SCALED: a token's 1 / rms, behind the rest
 
+// Two row tiles a workgroup leave CUs without work (fewer than 256 workgroups) where 24 rows a workgroup would not
+// (measured on weights taken in turn, K = 4,096: N = 6,144 in 256 workgroups 12.4 us at 8 tokens, N = 6,176 in 193
+// workgroups of 32 rows 13.2; 11.5 against 12.2 at one token, 13.7 against 15.0 at 16).
+inline bool cut_pays(int N) { return N / 32 < 256 && (N + 23) / 24 <= 256; }
+
 template <int MT, int RT, class O>
 int launch(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, O* C, int64_t ldc, int M, int N, int K, int waves,
            hipStream_t stream) {
   const int row_tiles = (N + 16 * RT - 1) / (16 * RT);
   const size_t lds = lds_bytes(waves, RT, MT);
+  if constexpr (RT == 2 && MT <= 2 && sizeof(O) == sizeof(bf16)) {
+    if (cut_pays(N)) {
+      const unsigned blocks = (unsigned)((N + 23) / 24);
+      if (streams_weight(N, K))
+        gemm_small_m_kernel<MT, RT, O, false, true, PLAIN, true><<<blocks, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
+      else
+        gemm_small_m_kernel<MT, RT, O, false, false, PLAIN, true><<<blocks, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
+      return launch_status();
+    }
+  }
   if (streams_weight(N, K))
     gemm_small_m_kernel<MT, RT, O, false, true><<<(unsigned)row_tiles, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
   else
@@ -354,11 +369,6 @@ int dispatch(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, O* C, int64
 }
 
 // The SCALED and SINK forms: up to 32 rows, bf16 out, one or two row tiles.
-// Two row tiles a workgroup leave CUs without work (fewer than 256 workgroups) where 24 rows a workgroup would not
-// (measured on weights taken in turn, K = 4,096: N = 6,144 in 256 workgroups 12.4 us at 8 tokens, N = 6,176 in 193
-// workgroups of 32 rows 13.2; 11.5 against 12.2 at one token, 13.7 against 15.0 at 16).
-inline bool cut_pays(int N) { return N / 32 < 256 && (N + 23) / 24 <= 256; }
-
 template <int MT, int RT, int MODE>
 int launch_linked(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, bf16* C, int64_t ldc, int M, int N, int K,
                   int waves, const NormLink& link, hipStream_t stream) {

@@ -701,7 +701,7 @@ def test_penalties_from_a_history_on_the_device():
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 33, 64])
 def test_gemm_small_m(M, out_dtype):
     """Weight-streaming MFMA product against float64, at sizes that are no multiples of its tiles."""
-    for N, K in ((96, 512), (331, 80), (4096, 4096), (1000, 1096), (50, 8)):
+    for N, K in ((96, 512), (331, 80), (4096, 4096), (1000, 1096), (50, 8), (6144, 64), (5000, 128)):
         a = torch.randn(M, K, device=DEV).to(torch.bfloat16)
         w = (torch.randn(N, K, device=DEV) * 0.05).to(torch.bfloat16)
         want = a.double() @ w.double().T
