@@ -25,8 +25,8 @@
 //
 // Two more forms take the norm kernels out of a decode layer (a kernel costs 3 to 5 us however small):
 //   SINK    the product is added to the residual stream in place (one rounding), and what the next RMSNorm
-//           needs leaves with it: the new stream times that norm's gain (XG), and per token and tile of 16
-//           columns the sum of squares of the new stream (rounded as stored), in float;
+//           needs leaves with it: the new stream times that norm's gain (XG), and per token and 16 columns (8 in
+//           the form whose workgroups take 24 rows) the sum of squares of the new stream (rounded as stored), in float;
 //   SCALED  the consumer of those: A is XG, and every token's result is multiplied by
 //           rsqrt(sum of its partial sums of squares / width + eps) before it is stored (or gated).
 // Together: y = (x g) W^T / rms(x) instead of ((x / rms(x)) g) W^T, the same value rounded at other places.
@@ -86,7 +86,7 @@ __host__ __device__ inline size_t lds_core_bytes(int waves, int rt, int mt) {
 // What the SCALED and SINK forms need beside the product's own operands.
 struct NormLink {
   const float* stats;  // SCALED: [M][ld_stats] partial sums of squares, `cols` of them a token
-  float* stats_out;    // SINK: where this product's partial sums go, one a token and tile of 16 columns
+  float* stats_out;    // SINK: where this product's partial sums go, one a token and 16 columns (CUT: 8)
   int64_t ld_stats;
   int cols;
   float eps, inv_width;
@@ -100,7 +100,7 @@ struct NormLink {
 // GATED (RT == 2): W is [2N, K], rows [0, N) the gate and [N, 2N) the up projection; the workgroup's
 // two row tiles are gate rows n0.. and up rows N + n0.., and the epilogue stores
 // silu(gate) * up into C [M, N]: the activation costs no pass of its own.
-// CUT (not GATED, not SINK): the last 8 rows of the workgroup's last tile are left out, so a workgroup takes
+// CUT (not GATED): the last 8 rows of the workgroup's last tile are left out, so a workgroup takes
 // 16 RT - 8 weight rows: with two tiles 24 rows, which makes 256 workgroups of N = 6,144 where 32 rows make 192.
 template <int MT, int RT, class O, bool GATED, bool STREAM, int MODE = PLAIN, bool CUT = false>
 __global__ void __launch_bounds__(1024) gemm_small_m_kernel(const bf16* __restrict__ A, int64_t lda,
@@ -108,7 +108,7 @@ __global__ void __launch_bounds__(1024) gemm_small_m_kernel(const bf16* __restri
                                                             O* __restrict__ C, int64_t ldc, int M, int N, int K,
                                                             NormLink link = NormLink{}) {
   static_assert(!GATED || RT == 2, "the gated form pairs one gate tile with one up tile");
-  static_assert(!CUT || (!GATED && MODE != SINK), "the cut form is for the plain and the scaled product");
+  static_assert(!CUT || !GATED, "the gated form pairs whole tiles");
   constexpr int ROWS = 16 * RT - (CUT ? 8 : 0);  // weight rows of a workgroup (not GATED)
   // 64-wide k steps in flight per wave: as many as the register file takes at 16 waves a workgroup
   constexpr int UNROLL = MT <= 2 ? (4 / RT > 0 ? 4 / RT : 1) : (2 / RT > 0 ? 2 / RT : 1);
@@ -162,7 +162,7 @@ __global__ void __launch_bounds__(1024) gemm_small_m_kernel(const bf16* __restri
       const int m = (tile % MT) * 16 + (ln & 15), n = n0 + (tile / MT) * 16 + 4 * (ln >> 4);
       if (m < M) {
         const bf16* hp = (const bf16*)C + (int64_t)m * ldc + n;
-        for (int e = 0; e < 4 && n + e < N; ++e) {
+        for (int e = 0; e < 4 && n + e < n_end; ++e) {
           res0[e] = (float)hp[e];
           gain0[e] = (link.gain_f32 ? ((const float*)link.gain)[n + e] : (float)((const bf16*)link.gain)[n + e]) +
                      link.gain_offset;
@@ -279,27 +279,33 @@ __global__ void __launch_bounds__(1024) gemm_small_m_kernel(const bf16* __restri
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           float res = res0[e], g = gain0[e];
-          if (!first && n + e < N) {
+          if (!first && n + e < n_end) {
             res = (float)hp[e];
             g = (link.gain_f32 ? ((const float*)link.gain)[n + e] : (float)((const bf16*)link.gain)[n + e]) + link.gain_offset;
           }
           const bf16 h = (bf16)(res + s[e]);
-          const float hf = n + e < N ? (float)h : 0.f;
+          const float hf = n + e < n_end ? (float)h : 0.f;
           hv[e] = h;
           ss += hf * hf;
           xv[e] = (bf16)(hf * g);
         }
-        if (n + 3 < N && ((ldc | link.ld_xg) & 3) == 0 && (((uintptr_t)C | (uintptr_t)link.xg) & 7) == 0) {
+        if (n + 3 < n_end && ((ldc | link.ld_xg) & 3) == 0 && (((uintptr_t)C | (uintptr_t)link.xg) & 7) == 0) {
           *(bf16x4*)hp = hv;  // four columns as one 8-byte store
           *(bf16x4*)xp = xv;
         } else {
-          for (int e = 0; e < 4 && n + e < N; ++e) hp[e] = hv[e], xp[e] = xv[e];
+          for (int e = 0; e < 4 && n + e < n_end; ++e) hp[e] = hv[e], xp[e] = xv[e];
         }
       }
-      // the tile's 16 columns of a token lie in the four lanes ln, ln + 16, + 32, + 48
-      ss += __shfl_xor(ss, 16, 64);
-      ss += __shfl_xor(ss, 32, 64);
-      if ((ln >> 4) == 0 && m < M) link.stats_out[(int64_t)m * link.ld_stats + (n0 >> 4) + r] = ss;
+      if constexpr (CUT) {
+        // 8 columns of a token lie in the two lanes ln and ln + 16 (n0 is a multiple of 8, so they share n / 8)
+        ss += __shfl_xor(ss, 16, 64);
+        if (((ln >> 4) & 1) == 0 && m < M && n < n_end) link.stats_out[(int64_t)m * link.ld_stats + (n >> 3)] = ss;
+      } else {
+        // the tile's 16 columns of a token lie in the four lanes ln, ln + 16, + 32, + 48
+        ss += __shfl_xor(ss, 16, 64);
+        ss += __shfl_xor(ss, 32, 64);
+        if ((ln >> 4) == 0 && m < M) link.stats_out[(int64_t)m * link.ld_stats + (n0 >> 4) + r] = ss;
+      }
     } else if (m < M) {
       O* cp = C + (int64_t)m * ldc + n;
       if (n + 3 < n_end) {
@@ -374,7 +380,7 @@ int launch_linked(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, bf16* 
                   int waves, const NormLink& link, hipStream_t stream) {
   const int row_tiles = (N + 16 * RT - 1) / (16 * RT);
   const size_t lds = lds_bytes(waves, RT, MT) + RS_BYTES;
-  if constexpr (MODE == SCALED && RT == 2 && MT == 1) {
+  if constexpr (RT == 2 && MT == 1) {
     if (cut_pays(N)) {
       const unsigned blocks = (unsigned)((N + 23) / 24);
       if (streams_weight(N, K))
@@ -543,16 +549,23 @@ extern "C" int dinfer_gemm_small_m_scaled(const void* A, int64_t lda, const void
 }
 
 // H[:M] += A . W^T in place (H bf16, the residual stream; summed in float, rounded once), and for the RMSNorm that
-// reads H next: XG[:M] = H * (gain + gain_offset), and stats[m][j] = sum of squares of H[m] over columns 16 j .. 16 j + 15
-// (ceil(N / 16) of them a token). M <= 32.
+// reads H next: XG[:M] = H * (gain + gain_offset), and stats[m][j] = sum of squares of H[m] over columns g j .. g j + g - 1
+// with g = 16, or 8 for the sizes dinfer_gemm_small_m_sink_stats_columns says so; ceil(N / g) of them a token. M <= 32.
+extern "C" int dinfer_gemm_small_m_sink_stats_columns(int64_t M, int64_t N, int64_t K) {
+  int rt, nw;
+  shape_for(M, N, K, &rt, &nw);
+  return M <= 16 && rt == 2 && cut_pays((int)N) ? 8 : 16;
+}
+
 extern "C" int dinfer_gemm_small_m_sink(const void* A, int64_t lda, const void* W, int64_t ldw, void* H, int64_t ldh, void* XG,
                                         int64_t ld_xg, const void* gain, int gain_f32, float gain_offset, float* stats,
                                         int64_t ld_stats, int64_t M, int64_t N, int64_t K, hipStream_t stream) {
   if (M <= 0 || N <= 0) return OK;
   if (M > 32) return ERR_UNSUPPORTED;
-  if (!linked_operands_ok(A, lda, W, ldw, ldh, M, N, K) || !H || !XG || !gain || !stats || ld_xg < N ||
-      ld_stats < (N + 15) / 16)
+  if (!linked_operands_ok(A, lda, W, ldw, ldh, M, N, K) || !H || !XG || !gain || !stats || ld_xg < N)
     return ERR_BAD_SHAPE;
+  const int64_t g = dinfer_gemm_small_m_sink_stats_columns(M, N, K);
+  if (ld_stats < (N + g - 1) / g) return ERR_BAD_SHAPE;
   NormLink link{};
   link.stats_out = stats, link.ld_stats = ld_stats, link.xg = (bf16*)XG, link.ld_xg = ld_xg, link.gain = gain;
   link.gain_f32 = gain_f32, link.gain_offset = gain_offset;

@@ -123,18 +123,19 @@ def gated_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, scratch: torch
     return out
 
 
+STATS_COLUMNS = 8   # a product that carries a norm leaves one sum of squares per token and this many columns, or twice as many
 CARRY_M = 32   # the products that carry a norm take up to this many rows (the block arrangement asks for fewer)
 
 
 def sink_nt(a: torch.Tensor, w: torch.Tensor, stream: torch.Tensor, xg: torch.Tensor, gain: torch.Tensor, offset: float,
-            stats: torch.Tensor, m: int) -> bool:
+            stats: torch.Tensor, m: int) -> int:
     """stream[:m] += a[:m] @ w.T in place, leaving xg = stream * (gain + offset) and per-row partial sums of squares in
-    stats for the RMSNorm that reads the stream next. False (nothing done) where no kernel does this for the sizes."""
+    stats for the RMSNorm that reads the stream next: returns how many of them a row has. 0 (nothing done) where no
+    kernel does this for the sizes."""
     n, k = w.shape
     if not (a.is_cuda and a.dtype == torch.bfloat16 and 0 < m <= CARRY_M and k % 8 == 0 and not _tall(m, n, k)):
-        return False
-    ops.gemm_small_m_sink(a, w, stream, xg, gain, stats, m, gain_offset=offset)
-    return True
+        return 0
+    return ops.gemm_small_m_sink(a, w, stream, xg, gain, stats, m, gain_offset=offset)
 
 
 def add_nt(a: torch.Tensor, w: torch.Tensor, stream: torch.Tensor, m: int) -> bool:

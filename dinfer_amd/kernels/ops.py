@@ -344,18 +344,21 @@ def gemm_small_m_gated(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: i
 
 
 def gemm_small_m_sink(a: torch.Tensor, w: torch.Tensor, stream_: torch.Tensor, xg: torch.Tensor, gain: torch.Tensor,
-                      stats: torch.Tensor, m: int, *, gain_offset: float = 0.0) -> None:
+                      stats: torch.Tensor, m: int, *, gain_offset: float = 0.0) -> int:
     """stream_[:m] += a[:m] @ w.T in place (the residual stream: summed in float, rounded once), and what the RMSNorm
     that reads it next needs: xg[:m] = stream_ * (gain + gain_offset), stats[r, j] = sum of squares of stream_[r] over
-    columns 16 j .. 16 j + 15. m <= 32, bf16."""
+    columns g j .. g j + g - 1, g being 16 or 8 as the kernel for these sizes has it. Returns how many of them a token
+    has (ceil(n / g)). m <= 32, bf16."""
     _need_gpu(a, w, stream_, xg, gain, stats)
     n, k = w.shape
     assert a.dtype == w.dtype == stream_.dtype == xg.dtype == torch.bfloat16 and stats.dtype == torch.float32
     assert a.shape[1] == k and stream_.shape[1] == n and xg.shape[1] == n and gain.numel() == n and gain.is_contiguous()
-    assert min(a.shape[0], stream_.shape[0], xg.shape[0], stats.shape[0]) >= m and stats.shape[1] >= -(-n // 16)
+    cols = -(-n // lib.get("dinfer_gemm_small_m_sink_stats_columns")(m, n, k))
+    assert min(a.shape[0], stream_.shape[0], xg.shape[0], stats.shape[0]) >= m and stats.shape[1] >= cols
     lib.call("dinfer_gemm_small_m_sink", a.data_ptr(), _rows(a), w.data_ptr(), _rows(w), stream_.data_ptr(), _rows(stream_),
              xg.data_ptr(), _rows(xg), gain.data_ptr(), _is_param_f32(gain, torch.bfloat16), float(gain_offset),
              stats.data_ptr(), _rows(stats), m, n, k, _stream())
+    return cols
 
 
 def gemm_small_m_scaled(xg: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, stats: torch.Tensor, cols: int,

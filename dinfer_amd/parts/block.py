@@ -13,6 +13,7 @@ from __future__ import annotations
 
 import torch
 
+from ..kernels import gemm
 from .base import Block, CacheView, Carried, Into
 from .registry import BLOCKS, FEED_FORWARDS, MIXERS, NORMS
 from .spec import LayerSpec
@@ -62,7 +63,8 @@ class PreNormBlock(Block):
         self.normed = ws.buffer("normed", self.hidden)
         # for norms carried by the products around them (steps of up to CARRY_ROWS tokens)
         self.xg = ws.buffer("carried_xg", self.hidden, rows=CARRY_ROWS)
-        self.stats = ws.buffer("carried_stats", -(-self.hidden // 16), dtype=torch.float32, rows=CARRY_ROWS)
+        self.stats = ws.buffer("carried_stats", -(-self.hidden // gemm.STATS_COLUMNS), dtype=torch.float32,
+                               rows=CARRY_ROWS)
 
     def input_norm(self):
         return self.norm_in if self.mixer.carries_norms else None

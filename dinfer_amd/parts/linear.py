@@ -36,8 +36,9 @@ class Linear:
         params = into.norm.carried()
         if params is not None and params[0] is not None and m <= into.xg.shape[0]:
             gain, offset, eps = params
-            if gemm.sink_nt(x, self.weight, into.stream, into.xg, gain, offset, into.stats, m):
-                return Carried(into.xg, into.stats, -(-width // 16), eps, width, into.norm, into.stream, into.buf, m)
+            cols = gemm.sink_nt(x, self.weight, into.stream, into.xg, gain, offset, into.stats, m)
+            if cols:
+                return Carried(into.xg, into.stats, cols, eps, width, into.norm, into.stream, into.buf, m)
         if gemm.add_nt(x, self.weight, into.stream, m):
             return Carried(None, None, 0, 0.0, width, into.norm, into.stream, into.buf, m)
         return None

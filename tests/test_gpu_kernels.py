@@ -817,12 +817,13 @@ def test_gemm_small_m_gated(M):
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 32])
 def test_gemm_small_m_carries_the_norm(M):
     """A product that adds into the residual stream and leaves what the next RMSNorm needs (the stream times the gain,
-    sums of squares per 16 columns), and the product that takes those: together they equal add, norm and product, to
+    sums of squares per 16 or 8 columns), and the product that takes those: together they equal add, norm and product, to
     rounding, at widths that are no multiples of the tiles, with the gain in either dtype and an offset. (Consumers of
     4,097 to 6,144 outputs take 24 weight rows a workgroup at up to 16 tokens: 6,144, 5,000 and 4,120 end their last
-    workgroup at 24, 8 and 16 rows.)"""
+    workgroup at 24, 8 and 16 rows; so do producers of that width: 5,120 and 4,108, whose last workgroup has 4 rows.)"""
     eps = 1e-5
-    for N, K, N2 in ((96, 512, 136), (328, 80, 1000), (4096, 4096, 6144), (1000, 1096, 50), (200, 64, 5000), (72, 128, 4120)):
+    for N, K, N2 in ((96, 512, 136), (328, 80, 1000), (4096, 4096, 6144), (1000, 1096, 50), (200, 64, 5000), (72, 128, 4120),
+                     (5120, 256, 64), (4108, 64, 32)):
         for gain_dtype, offset in ((torch.float32, 0.0), (torch.bfloat16, 1.0)):
             a = torch.randn(M, K, device=DEV).to(torch.bfloat16)
             w = (torch.randn(N, K, device=DEV) * 0.05).to(torch.bfloat16)
@@ -830,9 +831,10 @@ def test_gemm_small_m_carries_the_norm(M):
             gain = (torch.randn(N, device=DEV) * 0.1 + (1.0 - offset)).to(gain_dtype)
             h = h0.clone()
             xg = torch.full((M + 1, N), 7.0, device=DEV, dtype=torch.bfloat16)
-            cols = -(-N // 16)
-            stats = torch.full((M + 1, cols + 3), 7.0, device=DEV)
-            ops().gemm_small_m_sink(a, w, h, xg, gain, stats, M, gain_offset=offset)
+            stats = torch.full((M + 1, -(-N // 8) + 3), 7.0, device=DEV)
+            cols = ops().gemm_small_m_sink(a, w, h, xg, gain, stats, M, gain_offset=offset)
+            per = 8 if cols == -(-N // 8) else 16         # the 24-row form counts per 8 columns
+            assert cols == -(-N // per) and (per == 8) == (M <= 16 and 4096 < N <= 6144)
             want_h = (h0[:M].double() + a.double() @ w.double().T)
             err = (h[:M].double() - want_h).abs()
             # one rounding of a float sum of K products
@@ -840,8 +842,8 @@ def test_gemm_small_m_carries_the_norm(M):
             assert torch.equal(h[M:], h0[M:]) and bool((xg[M:] == 7.0).all()) and bool((stats[M:] == 7.0).all())
             assert bool((stats[:M, cols:] == 7.0).all())
             hs = h[:M].double()                                       # from here on the stream as it was stored
-            pad = torch.zeros(M, cols * 16 - N, device=DEV, dtype=torch.float64)
-            want_stats = torch.cat([hs, pad], dim=1).reshape(M, cols, 16).pow(2).sum(-1)
+            pad = torch.zeros(M, cols * per - N, device=DEV, dtype=torch.float64)
+            want_stats = torch.cat([hs, pad], dim=1).reshape(M, cols, per).pow(2).sum(-1)
             torch.testing.assert_close(stats[:M, :cols].double(), want_stats, rtol=1e-5, atol=1e-6)
             want_xg = hs * (gain.double() + offset)
             assert bool(((xg[:M].double() - want_xg).abs() <= 2 ** -8 * want_xg.abs() + 1e-6).all())
