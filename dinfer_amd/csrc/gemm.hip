@@ -304,7 +304,7 @@ __global__ void __launch_bounds__(1024) gemm_small_m_kernel(const bf16* __restri
         // the tile's 16 columns of a token lie in the four lanes ln, ln + 16, + 32, + 48
         ss += __shfl_xor(ss, 16, 64);
         ss += __shfl_xor(ss, 32, 64);
-        if ((ln >> 4) == 0 && m < M) link.stats_out[(int64_t)m * link.ld_stats + (n0 >> 4) + r] = ss;
+        if ((ln >> 4) == 0 && m < M && n0 + r * 16 < N) link.stats_out[(int64_t)m * link.ld_stats + (n0 >> 4) + r] = ss;
       }
     } else if (m < M) {
       O* cp = C + (int64_t)m * ldc + n;
@@ -326,6 +326,8 @@ constexpr size_t RS_BYTES = 64 * sizeof(float);  // SCALED: a token's 1 / rms, b
 // (measured on weights taken in turn, K = 4,096: N = 6,144 in 256 workgroups 12.4 us at 8 tokens, N = 6,176 in 193
 // workgroups of 32 rows 13.2; 11.5 against 12.2 at one token, 13.7 against 15.0 at 16).
 inline bool cut_pays(int N) { return N / 32 < 256 && (N + 23) / 24 <= 256; }
+// (40 rows a workgroup where 32 give 257 to 511 workgroups, N = 10,240 in 256 workgroups instead of 320: slower,
+// 26.6 -> 31.1 us at 8 tokens; three tiles leave a wave one k step of loads in flight.)
 
 template <int MT, int RT, class O>
 int launch(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, O* C, int64_t ldc, int M, int N, int K, int waves,

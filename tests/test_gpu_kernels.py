@@ -701,7 +701,7 @@ def test_penalties_from_a_history_on_the_device():
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 33, 64])
 def test_gemm_small_m(M, out_dtype):
     """Weight-streaming MFMA product against float64, at sizes that are no multiples of its tiles."""
-    for N, K in ((96, 512), (331, 80), (4096, 4096), (1000, 1096), (50, 8), (6144, 64), (5000, 128)):
+    for N, K in ((96, 512), (331, 80), (4096, 4096), (1000, 1096), (50, 8), (6144, 64), (5000, 128), (10240, 64), (9001, 72)):
         a = torch.randn(M, K, device=DEV).to(torch.bfloat16)
         w = (torch.randn(N, K, device=DEV) * 0.05).to(torch.bfloat16)
         want = a.double() @ w.double().T
@@ -820,10 +820,11 @@ def test_gemm_small_m_carries_the_norm(M):
     sums of squares per 16 or 8 columns), and the product that takes those: together they equal add, norm and product, to
     rounding, at widths that are no multiples of the tiles, with the gain in either dtype and an offset. (Consumers of
     4,097 to 6,144 outputs take 24 weight rows a workgroup at up to 16 tokens: 6,144, 5,000 and 4,120 end their last
-    workgroup at 24, 8 and 16 rows; so do producers of that width: 5,120 and 4,108, whose last workgroup has 4 rows.)"""
+    workgroup at 24, 8 and 16 rows; so do producers of that width: 5,120 and 4,108, whose last workgroup has 4 rows.
+    A producer of 9,000 columns in two tiles a workgroup ends with a tile that has no column: it leaves no sum.)"""
     eps = 1e-5
     for N, K, N2 in ((96, 512, 136), (328, 80, 1000), (4096, 4096, 6144), (1000, 1096, 50), (200, 64, 5000), (72, 128, 4120),
-                     (5120, 256, 64), (4108, 64, 32)):
+                     (5120, 256, 64), (4108, 64, 32), (64, 72, 10240), (9000, 64, 9000)):
         for gain_dtype, offset in ((torch.float32, 0.0), (torch.bfloat16, 1.0)):
             a = torch.randn(M, K, device=DEV).to(torch.bfloat16)
             w = (torch.randn(N, K, device=DEV) * 0.05).to(torch.bfloat16)
