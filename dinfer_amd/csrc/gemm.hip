@@ -111,7 +111,7 @@ __global__ void __launch_bounds__(1024) gemm_small_m_kernel(const bf16* __restri
   static_assert(!CUT || !GATED, "the gated form pairs whole tiles");
   constexpr int ROWS = 16 * RT - (CUT ? 8 : 0);  // weight rows of a workgroup (not GATED)
   // 64-wide k steps in flight per wave: as many as the register file takes at 16 waves a workgroup
-  constexpr int UNROLL = MT <= 2 ? (4 / RT > 0 ? 4 / RT : 1) : (2 / RT > 0 ? 2 / RT : 1);
+  constexpr int UNROLL = RT == 3 ? (MT == 1 ? 2 : 1) : MT <= 2 ? (4 / RT > 0 ? 4 / RT : 1) : (2 / RT > 0 ? 2 / RT : 1);
   constexpr int ROW_BYTES = 144;              // 64 k of a row and 16 bytes of padding
   constexpr int STRIP_BYTES = 16 * ROW_BYTES;  // one tile of 16 rows
   extern __shared__ __attribute__((aligned(16))) char smem[];  // a strip per wave; afterwards [waves][RT * MT][64 lanes][4] sums
@@ -326,8 +326,10 @@ constexpr size_t RS_BYTES = 64 * sizeof(float);  // SCALED: a token's 1 / rms, b
 // (measured on weights taken in turn, K = 4,096: N = 6,144 in 256 workgroups 12.4 us at 8 tokens, N = 6,176 in 193
 // workgroups of 32 rows 13.2; 11.5 against 12.2 at one token, 13.7 against 15.0 at 16).
 inline bool cut_pays(int N) { return N / 32 < 256 && (N + 23) / 24 <= 256; }
-// (40 rows a workgroup where 32 give 257 to 511 workgroups, N = 10,240 in 256 workgroups instead of 320: slower,
-// 26.6 -> 31.1 us at 8 tokens; three tiles leave a wave one k step of loads in flight.)
+// Likewise 40 rows a workgroup (three tiles, the last 8 rows left out; 8 waves with two k steps of loads in flight
+// each) where 32 rows give 257 to 511 workgroups, some CUs two and most one, and 40 give 256 or fewer: N = 10,240,
+// K = 5,120 at 8 tokens 26.6 -> 21.2 us (with one k step in flight and 4 waves: 31.1).
+inline bool wide_cut_pays(int N) { return (N + 31) / 32 > 256 && (N + 39) / 40 <= 256; }
 
 template <int MT, int RT, class O>
 int launch(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, O* C, int64_t ldc, int M, int N, int K, int waves,
@@ -382,6 +384,18 @@ int launch_linked(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, bf16* 
                   int waves, const NormLink& link, hipStream_t stream) {
   const int row_tiles = (N + 16 * RT - 1) / (16 * RT);
   const size_t lds = lds_bytes(waves, RT, MT) + RS_BYTES;
+  if constexpr (RT == 2 && MT == 1 && MODE == SCALED) {
+    if (wide_cut_pays(N)) {
+      const unsigned blocks = (unsigned)((N + 39) / 40);
+      const int w3 = 8;
+      const size_t lds3 = lds_bytes(w3, 3, MT) + RS_BYTES;
+      if (streams_weight(N, K))
+        gemm_small_m_kernel<MT, 3, bf16, false, true, MODE, true><<<blocks, w3 * 64, lds3, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, link);
+      else
+        gemm_small_m_kernel<MT, 3, bf16, false, false, MODE, true><<<blocks, w3 * 64, lds3, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, link);
+      return launch_status();
+    }
+  }
   if constexpr (RT == 2 && MT == 1) {
     if (cut_pays(N)) {
       const unsigned blocks = (unsigned)((N + 23) / 24);
@@ -445,9 +459,12 @@ inline int few_rows_waves(int mt, int rt, int64_t N, int64_t K) {
 }
 
 // Row tiles and waves of a launch, as dinfer_gemm_small_m chooses them (at most two row tiles here).
-inline void shape_for(int64_t M, int64_t N, int64_t K, int* rt_out, int* nw_out) {
+// scaled: the launch is the consumer of a carried norm, which has a form of 40 rows a workgroup (launched from the
+// two-tile case).
+inline void shape_for(int64_t M, int64_t N, int64_t K, int* rt_out, int* nw_out, bool scaled = false) {
   const int mt = (int)(M + 15) / 16;
   int rt = mt >= 2 ? ((N >= 6144 || streams_weight(N, K)) ? 2 : 1) : few_rows_row_tiles(M, N);
+  if (scaled && mt == 1 && wide_cut_pays((int)N)) rt = 2;
   int nw = few_rows_waves(mt, rt, N, K);
   while (nw > 1 && lds_bytes(nw, rt, mt) + RS_BYTES > 64 * 1024) nw /= 2;
   *rt_out = rt, *nw_out = nw;
@@ -545,7 +562,7 @@ extern "C" int dinfer_gemm_small_m_scaled(const void* A, int64_t lda, const void
     return launch_gated_scaled<2>((const bf16*)A, lda, (const bf16*)W, ldw, (bf16*)C, ldc, (int)M, (int)N, (int)K, nw, link, stream);
   }
   int rt, nw;
-  shape_for(M, N, K, &rt, &nw);
+  shape_for(M, N, K, &rt, &nw, true);
   return dispatch_linked<SCALED>((const bf16*)A, lda, (const bf16*)W, ldw, (bf16*)C, ldc, (int)M, (int)N, (int)K, rt, nw, link,
                                  stream);
 }

@@ -821,7 +821,8 @@ def test_gemm_small_m_carries_the_norm(M):
     rounding, at widths that are no multiples of the tiles, with the gain in either dtype and an offset. (Consumers of
     4,097 to 6,144 outputs take 24 weight rows a workgroup at up to 16 tokens: 6,144, 5,000 and 4,120 end their last
     workgroup at 24, 8 and 16 rows; so do producers of that width: 5,120 and 4,108, whose last workgroup has 4 rows.
-    A producer of 9,000 columns in two tiles a workgroup ends with a tile that has no column: it leaves no sum.)"""
+    A producer of 9,000 columns in two tiles a workgroup ends with a tile that has no column: it leaves no sum. A
+    consumer of 8,193 to 10,240 outputs takes 40 rows a workgroup: 10,240 and 9,000.)"""
     eps = 1e-5
     for N, K, N2 in ((96, 512, 136), (328, 80, 1000), (4096, 4096, 6144), (1000, 1096, 50), (200, 64, 5000), (72, 128, 4120),
                      (5120, 256, 64), (4108, 64, 32), (64, 72, 10240), (9000, 64, 9000)):
