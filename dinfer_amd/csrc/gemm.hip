@@ -331,11 +331,25 @@ inline bool cut_pays(int N) { return N / 32 < 256 && (N + 23) / 24 <= 256; }
 // K = 5,120 at 8 tokens 26.6 -> 21.2 us (with one k step in flight and 4 waves: 31.1).
 inline bool wide_cut_pays(int N) { return (N + 31) / 32 > 256 && (N + 39) / 40 <= 256; }
 
+// And 8 rows a workgroup (one tile less 8 rows) for a weight of so few rows that 16 a workgroup leave half the CUs
+// and more without work (1,024 rows: 64 workgroups).
+inline bool narrow_cut_pays(int N) { return (N + 15) / 16 <= 128; }
+
 template <int MT, int RT, class O>
 int launch(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, O* C, int64_t ldc, int M, int N, int K, int waves,
            hipStream_t stream) {
   const int row_tiles = (N + 16 * RT - 1) / (16 * RT);
   const size_t lds = lds_bytes(waves, RT, MT);
+  if constexpr (RT == 1 && MT <= 2 && sizeof(O) == sizeof(bf16)) {
+    if (narrow_cut_pays(N)) {
+      const unsigned blocks = (unsigned)((N + 7) / 8);
+      if (streams_weight(N, K))
+        gemm_small_m_kernel<MT, RT, O, false, true, PLAIN, true><<<blocks, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
+      else
+        gemm_small_m_kernel<MT, RT, O, false, false, PLAIN, true><<<blocks, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
+      return launch_status();
+    }
+  }
   if constexpr (RT == 2 && MT <= 2 && sizeof(O) == sizeof(bf16)) {
     if (cut_pays(N)) {
       const unsigned blocks = (unsigned)((N + 23) / 24);
@@ -393,6 +407,16 @@ int launch_linked(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, bf16* 
         gemm_small_m_kernel<MT, 3, bf16, false, true, MODE, true><<<blocks, w3 * 64, lds3, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, link);
       else
         gemm_small_m_kernel<MT, 3, bf16, false, false, MODE, true><<<blocks, w3 * 64, lds3, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, link);
+      return launch_status();
+    }
+  }
+  if constexpr (RT == 1 && MT == 1) {
+    if (narrow_cut_pays(N)) {
+      const unsigned blocks = (unsigned)((N + 7) / 8);
+      if (streams_weight(N, K))
+        gemm_small_m_kernel<MT, RT, bf16, false, true, MODE, true><<<blocks, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, link);
+      else
+        gemm_small_m_kernel<MT, RT, bf16, false, false, MODE, true><<<blocks, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, link);
       return launch_status();
     }
   }
@@ -573,7 +597,7 @@ extern "C" int dinfer_gemm_small_m_scaled(const void* A, int64_t lda, const void
 extern "C" int dinfer_gemm_small_m_sink_stats_columns(int64_t M, int64_t N, int64_t K) {
   int rt, nw;
   shape_for(M, N, K, &rt, &nw);
-  return M <= 16 && rt == 2 && cut_pays((int)N) ? 8 : 16;
+  return M <= 16 && ((rt == 2 && cut_pays((int)N)) || (rt == 1 && narrow_cut_pays((int)N))) ? 8 : 16;
 }
 
 extern "C" int dinfer_gemm_small_m_sink(const void* A, int64_t lda, const void* W, int64_t ldw, void* H, int64_t ldh, void* XG,

@@ -822,7 +822,8 @@ def test_gemm_small_m_carries_the_norm(M):
     4,097 to 6,144 outputs take 24 weight rows a workgroup at up to 16 tokens: 6,144, 5,000 and 4,120 end their last
     workgroup at 24, 8 and 16 rows; so do producers of that width: 5,120 and 4,108, whose last workgroup has 4 rows.
     A producer of 9,000 columns in two tiles a workgroup ends with a tile that has no column: it leaves no sum. A
-    consumer of 8,193 to 10,240 outputs takes 40 rows a workgroup: 10,240 and 9,000.)"""
+    consumer of 8,193 to 10,240 outputs takes 40 rows a workgroup: 10,240 and 9,000. Up to 2,048 rows a workgroup
+    takes 8, producer or consumer.)"""
     eps = 1e-5
     for N, K, N2 in ((96, 512, 136), (328, 80, 1000), (4096, 4096, 6144), (1000, 1096, 50), (200, 64, 5000), (72, 128, 4120),
                      (5120, 256, 64), (4108, 64, 32), (64, 72, 10240), (9000, 64, 9000)):
@@ -836,7 +837,7 @@ def test_gemm_small_m_carries_the_norm(M):
             stats = torch.full((M + 1, -(-N // 8) + 3), 7.0, device=DEV)
             cols = ops().gemm_small_m_sink(a, w, h, xg, gain, stats, M, gain_offset=offset)
             per = 8 if cols == -(-N // 8) else 16         # the 24-row form counts per 8 columns
-            assert cols == -(-N // per) and (per == 8) == (M <= 16 and 4096 < N <= 6144)
+            assert cols == -(-N // per) and (per == 8) == (M <= 16 and (N <= 2048 or 4096 < N <= 6144))
             want_h = (h0[:M].double() + a.double() @ w.double().T)
             err = (h[:M].double() - want_h).abs()
             # one rounding of a float sum of K products
