@@ -335,48 +335,39 @@ inline bool wide_cut_pays(int N) { return (N + 31) / 32 > 256 && (N + 39) / 40 <
 // and more without work (1,024 rows: 64 workgroups).
 inline bool narrow_cut_pays(int N) { return (N + 15) / 16 <= 128; }
 
+// One launch of the kernel in the form <MT, RT, O, GATED, ., MODE, CUT>, reading the weight past the caches where
+// it is large.
+template <int MT, int RT, class O, bool GATED, int MODE, bool CUT>
+int go(unsigned blocks, int waves, size_t lds, hipStream_t stream, const bf16* A, int64_t lda, const bf16* W, int64_t ldw,
+       O* C, int64_t ldc, int M, int N, int K, const NormLink& link = NormLink{}) {
+  if (streams_weight(GATED ? 2 * (int64_t)N : N, K))
+    gemm_small_m_kernel<MT, RT, O, GATED, true, MODE, CUT><<<blocks, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, link);
+  else
+    gemm_small_m_kernel<MT, RT, O, GATED, false, MODE, CUT><<<blocks, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, link);
+  return launch_status();
+}
+
 template <int MT, int RT, class O>
 int launch(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, O* C, int64_t ldc, int M, int N, int K, int waves,
            hipStream_t stream) {
-  const int row_tiles = (N + 16 * RT - 1) / (16 * RT);
   const size_t lds = lds_bytes(waves, RT, MT);
   if constexpr (RT == 1 && MT <= 2 && sizeof(O) == sizeof(bf16)) {
-    if (narrow_cut_pays(N)) {
-      const unsigned blocks = (unsigned)((N + 7) / 8);
-      if (streams_weight(N, K))
-        gemm_small_m_kernel<MT, RT, O, false, true, PLAIN, true><<<blocks, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
-      else
-        gemm_small_m_kernel<MT, RT, O, false, false, PLAIN, true><<<blocks, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
-      return launch_status();
-    }
+    if (narrow_cut_pays(N))
+      return go<MT, RT, O, false, PLAIN, true>((unsigned)((N + 7) / 8), waves, lds, stream, A, lda, W, ldw, C, ldc, M, N, K);
   }
   if constexpr (RT == 2 && MT <= 2 && sizeof(O) == sizeof(bf16)) {
-    if (cut_pays(N)) {
-      const unsigned blocks = (unsigned)((N + 23) / 24);
-      if (streams_weight(N, K))
-        gemm_small_m_kernel<MT, RT, O, false, true, PLAIN, true><<<blocks, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
-      else
-        gemm_small_m_kernel<MT, RT, O, false, false, PLAIN, true><<<blocks, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
-      return launch_status();
-    }
+    if (cut_pays(N))
+      return go<MT, RT, O, false, PLAIN, true>((unsigned)((N + 23) / 24), waves, lds, stream, A, lda, W, ldw, C, ldc, M, N, K);
   }
-  if (streams_weight(N, K))
-    gemm_small_m_kernel<MT, RT, O, false, true><<<(unsigned)row_tiles, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
-  else
-    gemm_small_m_kernel<MT, RT, O, false, false><<<(unsigned)row_tiles, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
-  return launch_status();
+  return go<MT, RT, O, false, PLAIN, false>((unsigned)((N + 16 * RT - 1) / (16 * RT)), waves, lds, stream, A, lda, W, ldw, C,
+                                            ldc, M, N, K);
 }
 
 template <int MT>
 int launch_gated(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, bf16* C, int64_t ldc, int M, int N, int K,
                  int waves, hipStream_t stream) {
-  const int col_tiles = (N + 15) / 16;
-  const size_t lds = lds_bytes(waves, 2, MT);
-  if (streams_weight(2 * (int64_t)N, K))
-    gemm_small_m_kernel<MT, 2, bf16, true, true><<<(unsigned)col_tiles, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
-  else
-    gemm_small_m_kernel<MT, 2, bf16, true, false><<<(unsigned)col_tiles, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
-  return launch_status();
+  return go<MT, 2, bf16, true, PLAIN, false>((unsigned)((N + 15) / 16), waves, lds_bytes(waves, 2, MT), stream, A, lda, W, ldw,
+                                             C, ldc, M, N, K);
 }
 
 template <class O>
@@ -396,45 +387,22 @@ int dispatch(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, O* C, int64
 template <int MT, int RT, int MODE>
 int launch_linked(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, bf16* C, int64_t ldc, int M, int N, int K,
                   int waves, const NormLink& link, hipStream_t stream) {
-  const int row_tiles = (N + 16 * RT - 1) / (16 * RT);
   const size_t lds = lds_bytes(waves, RT, MT) + RS_BYTES;
   if constexpr (RT == 2 && MT == 1 && MODE == SCALED) {
-    if (wide_cut_pays(N)) {
-      const unsigned blocks = (unsigned)((N + 39) / 40);
-      const int w3 = 8;
-      const size_t lds3 = lds_bytes(w3, 3, MT) + RS_BYTES;
-      if (streams_weight(N, K))
-        gemm_small_m_kernel<MT, 3, bf16, false, true, MODE, true><<<blocks, w3 * 64, lds3, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, link);
-      else
-        gemm_small_m_kernel<MT, 3, bf16, false, false, MODE, true><<<blocks, w3 * 64, lds3, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, link);
-      return launch_status();
-    }
+    if (wide_cut_pays(N))  // three tiles less 8 rows, 8 waves
+      return go<MT, 3, bf16, false, MODE, true>((unsigned)((N + 39) / 40), 8, lds_bytes(8, 3, MT) + RS_BYTES, stream, A, lda, W,
+                                                ldw, C, ldc, M, N, K, link);
   }
   if constexpr (RT == 1 && MT == 1) {
-    if (narrow_cut_pays(N)) {
-      const unsigned blocks = (unsigned)((N + 7) / 8);
-      if (streams_weight(N, K))
-        gemm_small_m_kernel<MT, RT, bf16, false, true, MODE, true><<<blocks, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, link);
-      else
-        gemm_small_m_kernel<MT, RT, bf16, false, false, MODE, true><<<blocks, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, link);
-      return launch_status();
-    }
+    if (narrow_cut_pays(N))
+      return go<MT, RT, bf16, false, MODE, true>((unsigned)((N + 7) / 8), waves, lds, stream, A, lda, W, ldw, C, ldc, M, N, K, link);
   }
   if constexpr (RT == 2 && MT == 1) {
-    if (cut_pays(N)) {
-      const unsigned blocks = (unsigned)((N + 23) / 24);
-      if (streams_weight(N, K))
-        gemm_small_m_kernel<MT, RT, bf16, false, true, MODE, true><<<blocks, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, link);
-      else
-        gemm_small_m_kernel<MT, RT, bf16, false, false, MODE, true><<<blocks, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, link);
-      return launch_status();
-    }
+    if (cut_pays(N))
+      return go<MT, RT, bf16, false, MODE, true>((unsigned)((N + 23) / 24), waves, lds, stream, A, lda, W, ldw, C, ldc, M, N, K, link);
   }
-  if (streams_weight(N, K))
-    gemm_small_m_kernel<MT, RT, bf16, false, true, MODE><<<(unsigned)row_tiles, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, link);
-  else
-    gemm_small_m_kernel<MT, RT, bf16, false, false, MODE><<<(unsigned)row_tiles, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, link);
-  return launch_status();
+  return go<MT, RT, bf16, false, MODE, false>((unsigned)((N + 16 * RT - 1) / (16 * RT)), waves, lds, stream, A, lda, W, ldw, C,
+                                              ldc, M, N, K, link);
 }
 
 template <int MODE>
@@ -451,13 +419,8 @@ int dispatch_linked(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, bf16
 template <int MT>
 int launch_gated_scaled(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, bf16* C, int64_t ldc, int M, int N, int K,
                         int waves, const NormLink& link, hipStream_t stream) {
-  const int col_tiles = (N + 15) / 16;
-  const size_t lds = lds_bytes(waves, 2, MT) + RS_BYTES;
-  if (streams_weight(2 * (int64_t)N, K))
-    gemm_small_m_kernel<MT, 2, bf16, true, true, SCALED><<<(unsigned)col_tiles, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, link);
-  else
-    gemm_small_m_kernel<MT, 2, bf16, true, false, SCALED><<<(unsigned)col_tiles, waves * 64, lds, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, link);
-  return launch_status();
+  return go<MT, 2, bf16, true, SCALED, false>((unsigned)((N + 15) / 16), waves, lds_bytes(waves, 2, MT) + RS_BYTES, stream, A,
+                                              lda, W, ldw, C, ldc, M, N, K, link);
 }
 
 // Row tiles a workgroup (16 weight rows each) for up to 16 tokens. Measured inside whole decode steps on MI355X (256
