@@ -148,9 +148,11 @@ def test_qkv_post_partial_and_interleaved_rotation():
 
 
 # ---- attention ------------------------------------------------------------------------------------
-def paged_case(dtype, H, Hkv, D, page, hist, new, seed=0, spike=None):
+def paged_case(dtype, H, Hkv, D, page, hist, new, seed=0, spike=None, sharp=1.0):
     """Requests with `hist` cached tokens and `new` rows each; pages in shuffled order.
-    Returns q [T, H*D], caches, metadata tensors and the expected output [T, H, D] in float64."""
+    Returns q [T, H*D], caches, metadata tensors and the expected output [T, H, D] in float64.
+    sharp: the queries are that much larger, so that among thousands of keys a few, anywhere, carry a row's softmax
+    (the mean of thousands of random values is as small as the tolerance, whatever keys went into it)."""
     g = torch.Generator().manual_seed(seed)
     B = len(hist)
     total = [h + n for h, n in zip(hist, new)]
@@ -165,10 +167,11 @@ def paged_case(dtype, H, Hkv, D, page, hist, new, seed=0, spike=None):
     for b in range(B):
         k = torch.randn(total[b], Hkv, D, generator=g).to(dtype)
         v = torch.randn(total[b], Hkv, D, generator=g).to(dtype)
-        q = torch.randn(new[b], H, D, generator=g).to(dtype)
-        if spike is not None and total[b] > spike[0] and new[b] > 0:
+        q = (torch.randn(new[b], H, D, generator=g) * sharp).to(dtype)
+        sp = spike.get(b) if isinstance(spike, dict) else spike   # one for all requests, or {request: (key, amp)}
+        if sp is not None and total[b] > sp[0] and new[b] > 0:
             # one far key that must win: scale a query and that key so that one score stands out
-            key, amp = spike
+            key, amp = sp
             k[key] = k[key] * 0 + q[-1, ::H // Hkv][:, :].float().to(dtype) * amp
         for i in range(-(-total[b] // page)):
             blk = order.pop()
@@ -184,14 +187,17 @@ def paged_case(dtype, H, Hkv, D, page, hist, new, seed=0, spike=None):
     return q_all, ops().k_cache_pack(kc).to(DEV), vc.to(DEV), meta, outs
 
 
-def expected_attention(outs, hist, scale, window):
+def expected_attention(outs, hist, scale, window, device="cpu"):
+    """float64 softmax attention of every request, rows [sum of new, H, D] on the CPU (device: where it is computed;
+    thousands of rows against thousands of keys take the CPU minutes)."""
     res = []
     for (q, k, v), h in zip(outs, hist):
+        q, k, v = q.to(device), k.to(device), v.to(device)
         Tq, H, D = q.shape
         G = H // k.shape[1]
         o = torch.zeros_like(q)
-        pos = h + torch.arange(Tq)[:, None]
-        j = torch.arange(k.shape[0])[None, :]
+        pos = h + torch.arange(Tq, device=device)[:, None]
+        j = torch.arange(k.shape[0], device=device)[None, :]
         hidden = j > pos
         if window:
             hidden = hidden | (j <= pos - window)
@@ -199,7 +205,7 @@ def expected_attention(outs, hist, scale, window):
             s = (q[:, hh] @ k[:, hh // G].T) * scale
             s = s.masked_fill(hidden, float("-inf"))
             o[:, hh] = torch.softmax(s, -1) @ v[:, hh // G]
-        res.append(o)
+        res.append(o.cpu())
     return torch.cat(res)
 
 
@@ -259,63 +265,77 @@ def test_attention_decode_takes_norm_rotation_and_cache_write_along(H, Hkv, D, p
     key and value into their pages and attends. Against the plain functions, and against the two kernels it stands for
     (whose page contents it must reproduce bit for bit). The slot of the new key holds stale content beforehand; one
     request writes nothing (slot -1: its pages hold the key already)."""
-    theta, eps, scale = 1e4, 1e-5, D ** -0.5
     # parts of several blocks, a part of one block (the store is waited for at once), a single key, many short ones
     rng = random.Random(3)
     for hist, splits in (([299, 69, 0, 1000], 7), ([rng.randrange(64) for _ in range(32)], 2),
                          ([0, 45, 1000, 130], 4), ([100, 31, 32, 33], 1)):
-        B = len(hist)
-        _, kc, vc, m, outs = paged_case(torch.bfloat16, H, Hkv, D, page, hist, [1] * B, seed=11)
-        g = torch.Generator().manual_seed(B)
-        raw = torch.randn(B, (H + 2 * Hkv) * D, generator=g).to(torch.bfloat16)
-        wq = wk = None
-        if gains != "none":
-            wq = (torch.rand(D, generator=g) + 0.5).to(torch.bfloat16)
-            wk = (torch.rand(D, generator=g) + 0.5).to(torch.bfloat16)
-        pos = [h for h in hist]
-        table = rope_table(1024, D, theta).to(DEV)
-        slots = []
-        for b in range(B):
-            blk = int(m["bt"][b, hist[b] // page])
-            slots.append(blk * page + hist[b] % page)
-        slots[1] = -1
-        # what the plain functions make of the rows
-        x = raw.double()
-        ang = plain.rope_angles(pos, D, theta)
-        norm = (lambda t, w: plain.rms_norm(t, w.double(), eps)) if wq is not None else (lambda t, w: t)
-        q = plain.rope_neox(norm(x[:, :H * D].view(B, H, D), wq), ang).to(torch.bfloat16).double()
-        k = plain.rope_neox(norm(x[:, H * D:(H + Hkv) * D].view(B, Hkv, D), wk), ang).to(torch.bfloat16).double()
-        v = x[:, (H + Hkv) * D:].view(B, Hkv, D)
-        want_outs = []
-        for b, (_, kk, vv) in enumerate(outs):
-            kk, vv = kk.clone(), vv.clone()
-            if slots[b] >= 0:
-                kk[-1], vv[-1] = k[b], v[b]
-            want_outs.append((q[b:b + 1], kk, vv))
-        want = expected_attention(want_outs, hist, scale, window)
-        dev = lambda t: None if t is None else t.to(DEV)
-        args = dict(heads=H, kv_heads=Hkv, head_dim=D, page_size=page)
-        post = dict(q_off=0, k_off=H * D, v_off=(H + Hkv) * D, q_gain=dev(wq), k_gain=dev(wk), eps=eps, gain_offset=0.0,
-                    positions=torch.tensor(pos, dtype=torch.int32, device=DEV))
-        slot_t = torch.tensor(slots, dtype=torch.int64, device=DEV)
-        part = torch.full((B * H * splits * (D + 4),), float("nan"), device=DEV)
-        # the two kernels
-        kc2, vc2, qkv2 = kc.clone(), vc.clone(), raw.to(DEV)
-        out2 = torch.zeros(B, H * D, device=DEV, dtype=torch.bfloat16)
-        ops().qkv_post(qkv2, B, **args, **post, cos_sin=table, rotary_dim=D, rope_style=0, k_cache=kc2, v_cache=vc2,
-                       slot_mapping=slot_t, token_runs=False)
-        ops().attn_decode(qkv2, out2, part, kc2, vc2, m["bt"], None, m["sl"], B, splits, scale=scale, window=window,
-                          **args)
-        # the one
-        kc1, vc1, qkv1 = kc.clone(), vc.clone(), raw.to(DEV)
-        out1 = torch.zeros(B, H * D, device=DEV, dtype=torch.bfloat16)
-        part.fill_(float("nan"))
-        ops().attn_decode_post(qkv1, out1, part, kc1, vc1, m["bt"], m["sl"], B, splits, scale=scale, window=window,
-                               **args, **post, cos_sin=table, slot_mapping=slot_t)
-        assert torch.equal(qkv1.cpu(), raw), "the product's rows are left as they were"
-        assert torch.equal(vc1, vc2) and torch.equal(kc1, kc2), "the pages hold the same bits as after the two kernels"
-        torch.testing.assert_close(out1.double().cpu().view(-1, H, D), want, rtol=2e-2, atol=2e-2)
-        assert torch.equal(out1, out2), f"differs from the two kernels by {float((out1.float() - out2.float()).abs().max())}"
+        decode_post_case(H, Hkv, D, page, window, gains, hist, splits)
+
+
+def decode_post_case(H, Hkv, D, page, window, gains, hist, splits, device="cpu", spike=None, sharp=1.0):
+    """One launch of the decode kernel that norms, rotates and writes the cache, against the plain functions and, bit
+    for bit, against the two kernels it stands for. Request 1 writes nothing (slot -1)."""
+    theta, eps, scale = 1e4, 1e-5, D ** -0.5
+    B = len(hist)
+    _, kc, vc, m, outs = paged_case(torch.bfloat16, H, Hkv, D, page, hist, [1] * B, seed=11)
+    g = torch.Generator().manual_seed(B)
+    raw = torch.randn(B, (H + 2 * Hkv) * D, generator=g).to(torch.bfloat16)
+    wq = wk = None
+    if gains != "none":
+        wq = ((torch.rand(D, generator=g) + 0.5) * sharp).to(torch.bfloat16)   # (a norm undoes any scale of q itself)
+        wk = (torch.rand(D, generator=g) + 0.5).to(torch.bfloat16)
+    else:
+        raw[:, :H * D] = (raw[:, :H * D].float() * sharp).to(torch.bfloat16)
+    pos = [h for h in hist]
+    table = rope_table(max(hist) + 25, D, theta).to(DEV)
+    slots = []
+    for b in range(B):
+        blk = int(m["bt"][b, hist[b] // page])
+        slots.append(blk * page + hist[b] % page)
+    slots[1] = -1
+    # what the plain functions make of the rows
+    x = raw.double()
+    ang = plain.rope_angles(pos, D, theta)
+    norm = (lambda t, w: plain.rms_norm(t, w.double(), eps)) if wq is not None else (lambda t, w: t)
+    q = plain.rope_neox(norm(x[:, :H * D].view(B, H, D), wq), ang).to(torch.bfloat16).double()
+    k = plain.rope_neox(norm(x[:, H * D:(H + Hkv) * D].view(B, Hkv, D), wk), ang).to(torch.bfloat16).double()
+    v = x[:, (H + Hkv) * D:].view(B, Hkv, D)
+    want_outs = []
+    for b, (_, kk, vv) in enumerate(outs):
+        kk, vv = kk.clone(), vv.clone()
+        if slots[b] >= 0:
+            kk[-1], vv[-1] = k[b], v[b]
+        sp = spike.get(b) if isinstance(spike, dict) else spike
+        if sp is not None:   # a cached key along the row's first query head of each group, as it is after norm and rotation
+            key, amp = sp
+            kk[key] = (q[b, ::H // Hkv] * amp).to(torch.bfloat16).double()
+            blk, off = int(m["bt"][b, key // page]), key % page
+            kc[blk, :, :, off, :] = kk[key].to(torch.bfloat16).view(Hkv, D // 8, 8).to(DEV)
+        want_outs.append((q[b:b + 1], kk, vv))
+    want = expected_attention(want_outs, hist, scale, window, device)
+    dev = lambda t: None if t is None else t.to(DEV)
+    args = dict(heads=H, kv_heads=Hkv, head_dim=D, page_size=page)
+    post = dict(q_off=0, k_off=H * D, v_off=(H + Hkv) * D, q_gain=dev(wq), k_gain=dev(wk), eps=eps, gain_offset=0.0,
+                positions=torch.tensor(pos, dtype=torch.int32, device=DEV))
+    slot_t = torch.tensor(slots, dtype=torch.int64, device=DEV)
+    part = torch.full((B * H * splits * (D + 4),), float("nan"), device=DEV)
+    # the two kernels
+    kc2, vc2, qkv2 = kc.clone(), vc.clone(), raw.to(DEV)
+    out2 = torch.zeros(B, H * D, device=DEV, dtype=torch.bfloat16)
+    ops().qkv_post(qkv2, B, **args, **post, cos_sin=table, rotary_dim=D, rope_style=0, k_cache=kc2, v_cache=vc2,
+                   slot_mapping=slot_t, token_runs=False)
+    ops().attn_decode(qkv2, out2, part, kc2, vc2, m["bt"], None, m["sl"], B, splits, scale=scale, window=window,
+                      **args)
+    # the one
+    kc1, vc1, qkv1 = kc.clone(), vc.clone(), raw.to(DEV)
+    out1 = torch.zeros(B, H * D, device=DEV, dtype=torch.bfloat16)
+    part.fill_(float("nan"))
+    ops().attn_decode_post(qkv1, out1, part, kc1, vc1, m["bt"], m["sl"], B, splits, scale=scale, window=window,
+                           **args, **post, cos_sin=table, slot_mapping=slot_t)
+    assert torch.equal(qkv1.cpu(), raw), "the product's rows are left as they were"
+    assert torch.equal(vc1, vc2) and torch.equal(kc1, kc2), "the pages hold the same bits as after the two kernels"
+    torch.testing.assert_close(out1.double().cpu().view(-1, H, D), want, rtol=2e-2, atol=2e-2)
+    assert torch.equal(out1, out2), f"differs from the two kernels by {float((out1.float() - out2.float()).abs().max())}"
 
 
 @pytest.mark.parametrize("window", [0, 200])
@@ -419,6 +439,121 @@ def test_attention_window_edge(kernel, inside):
 
 
 # ---- sampling -------------------------------------------------------------------------------------
+def table_refetches(k_lo, k_hi, page):
+    """Where a wave that walks the keys [k_lo, k_hi) in blocks of 32 with the block-table entries of 64 pages on board
+    takes the next 64: the first key of each block that no longer fits (csrc/attention.hip, Pages::ensure). Used to put
+    a spiked key on each side of such a line; if the rule here were wrong the spikes would only sit somewhere else."""
+    lines, base = [], (k_lo & ~31) // page
+    for kb in range(k_lo & ~31, k_hi, 32):
+        if (kb + 31) // page - base >= 64:
+            base = kb // page
+            lines.append(kb)
+    return lines
+
+
+def decode_parts(seq, window, splits):
+    """The parts [lo, hi) a request's visible keys are cut into (csrc/attention.hip, split_range)."""
+    first = max(seq - window, 0) if window else 0
+    base = first & ~31
+    per = (-(-(seq - base) // splits) + 31) & ~31
+    parts = [(max(base + s * per, first), min(base + (s + 1) * per, seq)) for s in range(splits)]
+    return [(lo, hi) for lo, hi in parts if lo < hi]
+
+
+LONG_DECODE = [
+    # 64 requests of 2,064 keys in two parts each: the parts meet inside a workgroup and the keys are read past the caches
+    ([2063] * 64, 2),
+    # one part walks the whole request; three parts of 1,376 keys
+    ([4095, 2063, 70], 1), ([4095, 2063, 70], 3),
+]
+
+
+@pytest.mark.parametrize("entry", ["plain", "post"])
+@pytest.mark.parametrize("side", [0, 1], ids=["spike_before_the_line", "spike_behind_the_line"])
+@pytest.mark.parametrize("window", [0, 3000])
+@pytest.mark.parametrize("page", [16, 8])
+def test_attention_decode_parts_longer_than_64_pages(page, window, side, entry):
+    """Contexts of 2,064 and 4,096 keys with so few parts that one wave walks more than 64 pages and takes the next
+    block-table entries on the way. Sharp scores: each row's softmax rests on a few keys anywhere in its context; and
+    in every request the key just before (or just behind) the first such line of one of its parts decides the row."""
+    H, Hkv, D = 8, 2, 128
+    for hist, splits in LONG_DECODE:
+        B, spikes, with_line = len(hist), {}, 0
+        for b, h in enumerate(hist):
+            lines = [l for lo, hi in decode_parts(h + 1, window, splits) for l in table_refetches(lo, hi, page)]
+            with_line += bool(lines)
+            spikes[b] = ((lines[b % len(lines)] if lines else h // 2) - 1 + side, 3.0)
+        assert with_line >= 1 or splits == 3, "the case must make waves walk more than 64 pages"
+        if entry == "post":
+            decode_post_case(H, Hkv, D, page, window, "bf16", hist, splits, device=DEV, spike=spikes, sharp=3.0)
+            continue
+        q, kc, vc, m, outs = paged_case(torch.bfloat16, H, Hkv, D, page, hist, [1] * B, seed=17, spike=spikes, sharp=3.0)
+        out = torch.zeros(B, H * D, device=DEV, dtype=torch.bfloat16)
+        part = torch.full((B * H * splits * (D + 4),), float("nan"), device=DEV)
+        ops().attn_decode(q, out, part, kc, vc, m["bt"], None, m["sl"], B, splits, scale=D ** -0.5, window=window,
+                          heads=H, kv_heads=Hkv, head_dim=D, page_size=page)
+        want = expected_attention(outs, hist, D ** -0.5, window, DEV)
+        got = out.double().cpu().view(B, H, D)
+        torch.testing.assert_close(got, want, rtol=2e-2, atol=2e-2)
+        for b, (_, _, vv) in enumerate(outs):
+            for hk in range(Hkv):
+                assert (got[b, hk * (H // Hkv)] - vv[spikes[b][0], hk]).abs().max() < 0.1, f"request {b}: the spiked key"
+
+
+def flash_wave_runs(hist, q_len, window, rows):
+    """The runs of keys the four waves of the last workgroup of a request walk (csrc/attention.hip, attn_flash_kernel)."""
+    q0 = (q_len - 1) // rows * rows
+    lo = max(hist + q0 - window + 1, 0) if window else 0
+    hi = hist + q_len
+    b0, b1 = lo >> 5, (hi + 31) >> 5
+    per = (b1 - b0 + 3) >> 2
+    runs = [(max((b0 + w * per) * 32, lo), min((b0 + (w + 1) * per) * 32, hi)) for w in range(4)]
+    return [(a, b) for a, b in runs if a < b]
+
+
+@pytest.mark.parametrize("side", [0, 1], ids=["spike_before_the_line", "spike_behind_the_line"])
+@pytest.mark.parametrize("windowed", [False, True])
+@pytest.mark.parametrize("page,rows", [(16, 4500), (8, 4500), (24, 6400)])
+def test_attention_flash_a_prompt_of_thousands_of_rows(page, rows, windowed, side):
+    """One prompt of 4,500 (6,400) rows of 24 heads of 128: 48 rows a workgroup, and the waves of the late row tiles
+    walk more than 64 pages each. Sharp scores; the last row's softmax rests on the key beside a wave's refetch line."""
+    H, Hkv, D = 24, 4, 128
+    window = rows - 300 if windowed else 0
+    lines = [l for lo, hi in flash_wave_runs(0, rows, window, 48) for l in table_refetches(lo, hi, page)]
+    assert lines, "the case must make a wave walk more than 64 pages"
+    key = lines[len(lines) // 2] - 1 + side
+    q, kc, vc, m, outs = paged_case(torch.bfloat16, H, Hkv, D, page, [0], [rows], seed=23, spike=(key, 3.0), sharp=3.0)
+    out = torch.zeros(rows, H * D, device=DEV, dtype=torch.bfloat16)
+    ops().attn_flash(q, out, kc, vc, m["bt"], m["cu"], m["sl"], 1, rows, rows, scale=D ** -0.5, window=window, heads=H,
+                     kv_heads=Hkv, head_dim=D, page_size=page)
+    want = expected_attention(outs, [0], D ** -0.5, window, DEV)
+    got = out.double().cpu().view(rows, H, D)
+    torch.testing.assert_close(got, want, rtol=2e-2, atol=2e-2)
+    for hk in range(Hkv):
+        assert (got[-1, hk * (H // Hkv)] - outs[0][2][key, hk]).abs().max() < 0.1
+
+
+@pytest.mark.parametrize("side", [0, 1], ids=["spike_before_the_line", "spike_behind_the_line"])
+@pytest.mark.parametrize("window", [0, 4200])
+@pytest.mark.parametrize("page", [16, 8])
+def test_attention_flash_a_portion_behind_thousands_of_keys(page, window, side):
+    """600 rows behind 4,000 keys (32 rows a workgroup: every wave walks 1,150 keys), beside a short request."""
+    H, Hkv, D = 8, 2, 128
+    hist, new = [4000, 20], [600, 40]
+    lines = [l for lo, hi in flash_wave_runs(hist[0], new[0], window, 32) for l in table_refetches(lo, hi, page)]
+    assert lines
+    key = lines[len(lines) // 2] - 1 + side
+    q, kc, vc, m, outs = paged_case(torch.bfloat16, H, Hkv, D, page, hist, new, seed=29, spike={0: (key, 3.0)}, sharp=3.0)
+    out = torch.zeros(sum(new), H * D, device=DEV, dtype=torch.bfloat16)
+    ops().attn_flash(q, out, kc, vc, m["bt"], m["cu"], m["sl"], 2, sum(new), max(new), scale=D ** -0.5, window=window,
+                     heads=H, kv_heads=Hkv, head_dim=D, page_size=page)
+    want = expected_attention(outs, hist, D ** -0.5, window, DEV)
+    got = out.double().cpu().view(sum(new), H, D)
+    torch.testing.assert_close(got, want, rtol=2e-2, atol=2e-2)
+    for hk in range(Hkv):
+        assert (got[new[0] - 1, hk * (H // Hkv)] - outs[0][2][key, hk]).abs().max() < 0.1
+
+
 @pytest.mark.parametrize("V", [163841, 16385, 4096 * 4, 1000])
 @pytest.mark.parametrize("spread", [False, True])
 def test_argmax_ties_to_lowest_index(V, spread):
