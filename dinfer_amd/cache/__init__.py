@@ -1,4 +1,3 @@
-from .block_pool import BlockPool
 from .manager import CacheManager, GroupSpec
 
-__all__ = ["BlockPool", "CacheManager", "GroupSpec"]
+__all__ = ["CacheManager", "GroupSpec"]

@@ -32,8 +32,6 @@ class EngineOptions:
     # the device), and only then the running step's tokens are read: the host's work between two steps is hidden
     # (the reference's engine does so by default too: crates/core/src/engine.rs:153-154,209)
     async_scheduling: bool = True
-    # bfloat16 products of more than 32 rows: the vendor library called directly (False: through torch.mm)
-    gemm_library: bool = True
     # "measured": the engine's warm-up times the library's candidates once per shape, keeps the choices in
     # gemm_plan_file and later processes reuse them; "heuristic": the library's first suggestion, nothing timed
     gemm_tuning: str = "measured"

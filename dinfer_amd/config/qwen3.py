@@ -9,7 +9,10 @@ Two things go beyond the reference: ``rope_scaling`` is read so that a non-null
 value is refused instead of silently ignored, and a sliding window is accepted
 (the reference refuses it, config.rs:48) with the meaning the keys themselves
 carry: with ``use_sliding_window`` the layers from index ``max_window_layers``
-on attend to the last ``sliding_window`` keys only.
+on attend to the last ``sliding_window`` keys only. Newer config.json files also
+spell the pattern out layer by layer (``layer_types``: "full_attention" or
+"sliding_attention"); it is read and must say what the three keys say, so a file
+whose list and keys disagree is refused rather than run with one of the two.
 """
 from __future__ import annotations
 
@@ -38,6 +41,7 @@ class Qwen3Config(ModelConfig):
     max_window_layers: int | None = key(int, None, nullable=True)
     eos_token_ids: tuple = field(default=())
     rope_scaling_present: bool = field(default=False)
+    layer_types: tuple | None = field(default=None)
 
     ARCHITECTURE = "Qwen3ForCausalLM"
 
@@ -54,7 +58,12 @@ class Qwen3Config(ModelConfig):
             ids = tuple(eos)
         else:
             raise ConfigError(f"config key 'eos_token_id' must be a number or a list of numbers, got {eos!r}")
-        return {"eos_token_ids": ids, "rope_scaling_present": d.get("rope_scaling") is not None}
+        kinds = d.get("layer_types")
+        if kinds is not None:
+            if not isinstance(kinds, list) or not all(isinstance(x, str) for x in kinds):
+                raise ConfigError(f"config key 'layer_types' must be a list of names, got {kinds!r}")
+            kinds = tuple(kinds)
+        return {"eos_token_ids": ids, "rope_scaling_present": d.get("rope_scaling") is not None, "layer_types": kinds}
 
     def extra_to_dict(self) -> dict:
         out = {"architectures": [self.ARCHITECTURE], "model_type": "qwen3"}
@@ -62,6 +71,8 @@ class Qwen3Config(ModelConfig):
             out["eos_token_id"] = self.eos_token_ids[0]
         elif self.eos_token_ids:
             out["eos_token_id"] = list(self.eos_token_ids)
+        if self.layer_types is not None:
+            out["layer_types"] = list(self.layer_types)
         return out
 
     def check(self) -> None:
@@ -90,6 +101,21 @@ class Qwen3Config(ModelConfig):
             if self.max_window_layers is None or not (0 <= self.max_window_layers <= self.num_hidden_layers):
                 raise ConfigError("use_sliding_window needs max_window_layers in [0, num_hidden_layers], "
                                   f"got {self.max_window_layers}")
+        if self.layer_types is not None:
+            names = {"full_attention": False, "sliding_attention": True}
+            unknown = sorted(set(self.layer_types) - set(names))
+            if unknown:
+                raise ConfigError(f"config key 'layer_types' names unknown kinds {unknown} (known: {sorted(names)})")
+            if len(self.layer_types) != self.num_hidden_layers:
+                raise ConfigError(f"config key 'layer_types' lists {len(self.layer_types)} layers, "
+                                  f"num_hidden_layers is {self.num_hidden_layers}")
+            derived = [self.layer_window(i) is not None for i in range(self.num_hidden_layers)]
+            listed = [names[x] for x in self.layer_types]
+            if listed != derived:
+                i = next(i for i in range(len(listed)) if listed[i] != derived[i])
+                raise ConfigError(f"config key 'layer_types' says layer {i} is {self.layer_types[i]!r}, but "
+                                  f"use_sliding_window = {self.use_sliding_window}, max_window_layers = "
+                                  f"{self.max_window_layers} make it {'sliding' if derived[i] else 'full'} attention")
 
     # sizes derived as the reference does (config.rs:66-77)
     @property

@@ -195,6 +195,9 @@ public:
     // once more" and preempts nobody. Anything else is planned after the running step's update, as before.
     bool can_look_ahead() const {
         if (!plan_.open || prev_.open || !waiting_.empty() || plan_.scheduled.empty()) return false;
+        // a running request the step left out (no budget for it, a portion that could not be aligned) would come into
+        // the step ahead with a token the host already knows, where every row is taken to wait for the running step
+        if (plan_.scheduled.size() != running_.size()) return false;
         for (const Scheduled& s : plan_.scheduled)
             if (s.num_new != 1 || !s.samples) return false;
         for (int g = 0; g < cache_->num_groups(); ++g)

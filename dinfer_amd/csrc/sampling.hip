@@ -197,29 +197,33 @@ __device__ void row_topk_topp(float* row, int vocab, int k, float p, float* red)
   __syncthreads();
 }
 
-__device__ __forceinline__ uint32_t mulhilo(uint32_t a, uint32_t b, uint32_t* hi) {
-  const uint64_t p = (uint64_t)a * b;
-  *hi = (uint32_t)(p >> 32);
-  return (uint32_t)p;
-}
+// Philox4x32-10 (Salmon, Moraes, Dror, Shaw: "Parallel random numbers: as easy as 1, 2, 3", SC'11): ten rounds, each
+// of which multiplies words 0 and 2 of the counter by the two round constants to 64 bits, crosses the halves over
+// and mixes in the key, which grows by the two Weyl constants from round to round. The uniform number of a draw is
+// made of (seed, offset) alone, as the reference makes it (crates/kernels/cuda/sampling.cu:137-157): key = seed,
+// counter = (offset, 0, 0), the top 24 bits of the first output word.
+struct Philox {
+  static constexpr uint64_t MUL_A = 0xD2511F53u, MUL_B = 0xCD9E8D57u;
+  static constexpr uint32_t WEYL_A = 0x9E3779B9u, WEYL_B = 0xBB67AE85u;
+  uint32_t x0, x1, x2, x3, ka, kb;
 
-__device__ void philox4x32_10(uint32_t c[4], uint32_t k0, uint32_t k1) {
-#pragma unroll
-  for (int r = 0; r < 10; ++r) {
-    uint32_t hi0, hi1;
-    const uint32_t lo0 = mulhilo(0xD2511F53u, c[0], &hi0);
-    const uint32_t lo1 = mulhilo(0xCD9E8D57u, c[2], &hi1);
-    const uint32_t n0 = hi1 ^ c[1] ^ k0, n1 = lo1, n2 = hi0 ^ c[3] ^ k1, n3 = lo0;
-    c[0] = n0; c[1] = n1; c[2] = n2; c[3] = n3;
-    k0 += 0x9E3779B9u;
-    k1 += 0xBB67AE85u;
+  __device__ void round() {
+    const uint64_t pa = MUL_A * x0, pb = MUL_B * x2;
+    const uint32_t y0 = (uint32_t)(pb >> 32) ^ x1 ^ ka, y2 = (uint32_t)(pa >> 32) ^ x3 ^ kb;
+    x1 = (uint32_t)pb;
+    x3 = (uint32_t)pa;
+    x0 = y0;
+    x2 = y2;
+    ka += WEYL_A;
+    kb += WEYL_B;
   }
-}
+};
 
 __device__ float philox_uniform(uint64_t seed, uint64_t offset) {
-  uint32_t c[4] = {(uint32_t)offset, (uint32_t)(offset >> 32), 0u, 0u};
-  philox4x32_10(c, (uint32_t)seed, (uint32_t)(seed >> 32));
-  return (float)(c[0] >> 8) * (1.f / 16777216.f);
+  Philox g{(uint32_t)offset, (uint32_t)(offset >> 32), 0u, 0u, (uint32_t)seed, (uint32_t)(seed >> 32)};
+#pragma unroll
+  for (int r = 0; r < 10; ++r) g.round();
+  return (float)(g.x0 >> 8) * 0x1p-24f;
 }
 
 struct DrawShared {
@@ -375,31 +379,6 @@ __global__ void __launch_bounds__(64) argmax_join_kernel(const float* __restrict
   }
   if (threadIdx.x == 0) out[r] = besti == 0x7fffffff ? 0 : besti;
 }
-
-// One entry per distinct token of a row's history: ids[e], count among the
-// outputs cnt[e] (0 if it occurs in the prompt only). Row b owns the entries
-// offsets[b] .. offsets[b+1].
-__global__ void __launch_bounds__(256) penalties_kernel(float* __restrict__ logits, int64_t ld,
-                                                        const int32_t* __restrict__ ids,
-                                                        const int32_t* __restrict__ cnt,
-                                                        const int32_t* __restrict__ offsets,
-                                                        const float* __restrict__ rep, const float* __restrict__ freq,
-                                                        const float* __restrict__ pres, int vocab) {
-  const int b = blockIdx.x;
-  const float r = rep[b], f = freq[b], pr = pres[b];
-  if (r == 1.f && f == 0.f && pr == 0.f) return;
-  float* row = logits + (int64_t)b * ld;
-  for (int e = offsets[b] + threadIdx.x; e < offsets[b + 1]; e += blockDim.x) {
-    const int t = ids[e];
-    if (t < 0 || t >= vocab) continue;
-    float v = row[t];
-    if (r != 1.f) v = v > 0.f ? v / r : v * r;
-    const int c = cnt[e];
-    if (c > 0) v -= f * (float)c + pr;
-    row[t] = v;
-  }
-}
-
 
 // ---- the same rule in a few passes over many workgroups -----------------------------------------
 // One workgroup per row needs about a hundred passes over the row for top-k and top-p (two
@@ -1098,17 +1077,6 @@ extern "C" int dinfer_sample(const float* logits, int64_t ld, float* work, const
   return launch_status();
 }
 
-extern "C" int dinfer_penalties(float* logits, int64_t ld, const int32_t* ids, const int32_t* counts,
-                                const int32_t* offsets, const float* repetition, const float* frequency,
-                                const float* presence, int64_t rows, int64_t vocab, hipStream_t stream) {
-  if (rows <= 0) return OK;
-  if (vocab <= 0 || ld < vocab || rows > 0x7fffffff) return ERR_BAD_SHAPE;
-  penalties_kernel<<<(unsigned)rows, 256, 0, stream>>>(logits, ld, ids, counts, offsets, repetition, frequency,
-                                                       presence, (int)vocab);
-  return launch_status();
-}
-
-
 // Bytes of scratch that dinfer_sample_rows needs for this many rows and this vocabulary.
 extern "C" int dinfer_sample_scratch_bytes(int64_t rows, int64_t vocab, int64_t* bytes) {
   if (rows <= 0 || vocab <= 0 || !bytes) return ERR_BAD_SHAPE;
@@ -1157,7 +1125,9 @@ extern "C" int dinfer_history_add(int32_t* history, int64_t slots, int64_t vocab
 }
 
 // In place on logits [rows, ld]: rows packed as {int32 slot; float repetition, frequency, presence} (slot < 0:
-// untouched) take their penalties from history[slot] (the rule of dinfer_penalties).
+// untouched) take their penalties from history[slot]: a token seen in the prompt or among the outputs has a positive
+// logit divided by `repetition` and a negative one multiplied by it; one seen c > 0 times among the outputs loses
+// frequency * c + presence on top (crates/kernels/cuda/sampling.cu:318-349).
 extern "C" int dinfer_penalties_dense(float* logits, int64_t ld, const int32_t* history, int64_t slots,
                                       const void* rows_packed, int64_t rows, int64_t vocab, hipStream_t stream) {
   if (rows <= 0) return OK;

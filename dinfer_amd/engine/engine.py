@@ -86,7 +86,8 @@ class Engine:
         self.options = self.runner.options
         spec = self.runner.model.spec
         self.vocab_size = spec.vocab_size
-        self.scheduler = Scheduler(self.options, self.runner.cache, spec.eos_token_ids)
+        self.scheduler = Scheduler(self.options, self.runner.cache, spec.eos_token_ids,
+                                   chunk_alignment=getattr(self.runner, "chunk_alignment", None))
         # the sampled tokens land where the next step can take them from as its input, if it is launched before
         # the host has read them
         last = getattr(getattr(self.runner, "batch", None), "last_tokens", None)
@@ -102,6 +103,7 @@ class Engine:
                                         "num_preemptions_total", "prefix_cache_hit_tokens_total", "request_success_stop",
                                         "request_success_length", "request_abort")}
         self._in_prompt: set = set()        # requests with prompt tokens still to compute (what the counters look at)
+        self.steps_launched_ahead = 0       # steps issued before the tokens of the step before them were read
         self.phases: dict | None = None     # see measure_phases
 
     # ---- requests ------------------------------------------------------------------------------
@@ -151,6 +153,7 @@ class Engine:
             self._running, held = None, self._running
             try:
                 outs += self._launch(ahead=True)        # (a plan ahead ends nobody: nothing is added)
+                self.steps_launched_ahead += 1
             finally:                                    # whatever happened, the running step is still the running step
                 self._running, nxt = held, self._running
         run = self._running

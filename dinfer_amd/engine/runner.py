@@ -78,7 +78,9 @@ class ModelRunner:
         self.max_tokens = options.max_num_batched_tokens + (options.max_num_seqs if options.decode_exempt_from_budget else 0)
         self.ctx = BuildContext(device, self.dtype, self.max_tokens, self.max_rows, self.page_size,
                                 options.max_num_seqs, max_seq_len=options.max_model_len)
-        blaslt.configure(enabled=options.gemm_library, tuning=options.gemm_tuning, plan_file=options.gemm_plan_file)
+        blaslt.configure(tuning=options.gemm_tuning, plan_file=options.gemm_plan_file)
+        if self.dtype == torch.bfloat16:
+            blaslt.require()
         model.bind(self.ctx)
         self._build_caches()
         self.batch = StepBatch(device, self.max_tokens, options.max_num_seqs, self.max_rows,
@@ -151,11 +153,13 @@ class ModelRunner:
                 raise ValueError(f"cache group {k!r} is asked for with windows {windows[keys.index(k)]} and {need.window}: "
                                  "the group key must tell them apart")
             entry_group.append(keys.index(k))
-        # prompt portions end where every layer's own chunks end
+        # prompt portions end where every layer's own chunks end: the user's alignment raised to what this model's
+        # caches ask (kept here, for the scheduler of this runner: the options object may serve another model too)
         import math
+        self.chunk_alignment = int(opt.prefill_chunk_alignment or 1)
         for n in needs:
             if n is not None and n.chunk_alignment > 1:
-                opt.prefill_chunk_alignment = math.lcm(opt.prefill_chunk_alignment, n.chunk_alignment)
+                self.chunk_alignment = math.lcm(self.chunk_alignment, n.chunk_alignment)
         page_bytes = sum(n.page_bytes(self.page_size, self.dtype) for n in needs if n is not None)
         slot_bytes = sum(n.slot_bytes(self.dtype) for n in needs if n is not None) * self.num_slots
         if opt.num_blocks is not None:

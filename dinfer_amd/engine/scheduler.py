@@ -89,14 +89,16 @@ class SchedulerOutput:
 
 
 class Scheduler:
-    def __init__(self, options: EngineOptions, cache: CacheManager, eos_token_ids=()):
+    def __init__(self, options: EngineOptions, cache: CacheManager, eos_token_ids=(), chunk_alignment: int | None = None):
+        """chunk_alignment: where prompt portions may end (None: the options' own prefill_chunk_alignment; a runner
+        passes that value raised to what its model's caches ask)."""
         self.opt, self.cache = options, cache
         self.eos = set(eos_token_ids)
         o = native.SchedOptions(options.max_num_batched_tokens, options.max_num_seqs, options.max_model_len,
                                 options.prefill_tokens_per_step or 0, options.long_prefill_token_threshold or 0,
                                 int(options.enable_chunked_prefill), int(options.decode_exempt_from_budget),
                                 int(cache.prefix_caching if options.enable_prefix_caching is None
-                                    else options.enable_prefix_caching), int(options.prefill_chunk_alignment or 1),
+                                    else options.enable_prefix_caching), int(chunk_alignment or options.prefill_chunk_alignment or 1),
                                 int(options.max_logits_rows or 0))
         eos = np.array(sorted(self.eos) or [0], dtype=np.int32)
         self._h = native.created("dh_sched_create", o, cache._h, eos.ctypes.data, len(self.eos))

@@ -1,7 +1,7 @@
 """bf16 matrix products of many rows through hipBLASLt, the algorithm chosen per shape by measurement.
 
 The reference hands these products to its vendor library too (crates/kernels/src/gemm.rs:605-647).
-torch.mm asks hipBLASLt for its first suggestion; for few output tiles and a long K that suggestion is
+The library's first suggestion is what a framework's own matmul runs; for few output tiles and a long K it is
 far off (N 5,120, K 17,408 at 520 rows: 167 us against 102 us for the best of the library's own list),
 so here the library is called directly and its candidate list for a shape is timed.
 
@@ -14,7 +14,8 @@ When it is timed, and what a product runs with otherwise, is settled so that res
   * the choices are kept in a plan file beside the built libraries, keyed by device, library and shape; a later
     process finds them there, measures nothing and computes the same bits as the one that measured.
   * `configure(tuning="heuristic")` takes the library's first suggestion everywhere (no measurement, no file).
-These are engine options (EngineOptions.gemm_library, gemm_tuning, gemm_plan_file), not environment switches.
+These are engine options (EngineOptions.gemm_tuning, gemm_plan_file), not environment switches. A shape the
+library names no algorithm for is left to the caller (`matmul` returns False), who runs the plain kernel.
 
 out[M, N] = a[M, K] . w[N, K]^T in row-major storage is, in the library's column-major terms,
 D (N x M, ld = ldc) = op_T(w as K x N, ld = ldw) . (a as K x M, ld = lda).
@@ -62,22 +63,21 @@ _flush: dict = {}
 _one, _zero = c_float(1.0), c_float(0.0)
 
 # settings of the process (the engine sets them from its options when it is built)
-_settings = {"enabled": True, "tuning": "measured", "plan_file": None, "log": False}
+_settings = {"tuning": "measured", "plan_file": None, "log": False}
 _measuring = False            # inside measuring(): shapes without a choice are timed
 _stored: dict | None = None   # the plan file's contents: shape key -> {"index": i, "algo": hex of the algorithm's bytes}
 _stored_path = None
 
 
-def configure(enabled: bool | None = None, tuning: str | None = None, plan_file=..., log: bool | None = None) -> None:
-    """enabled False: the library is not called directly (torch.mm serves the products of many rows).
-    tuning "measured": candidates are timed inside measuring() and the choices kept in the plan file;
+def configure(tuning: str | None = None, plan_file=..., log: bool | None = None) -> None:
+    """tuning "measured": candidates are timed inside measuring() and the choices kept in the plan file;
     "heuristic": the library's first suggestion for every shape. plan_file: where choices are kept between
     processes ("" for nowhere; None: beside the built libraries; left out: as it was). Arguments left out or None
     (plan_file aside) change nothing. Shapes that already have a plan keep it."""
     global _stored, _stored_path
     if tuning is not None and tuning not in ("measured", "heuristic"):
         raise ValueError(f"gemm tuning must be 'measured' or 'heuristic', got {tuning!r}")
-    for k, v in (("enabled", enabled), ("tuning", tuning), ("log", log)):
+    for k, v in (("tuning", tuning), ("log", log)):
         if v is not None:
             _settings[k] = v
     if plan_file is not ... and plan_file != _settings["plan_file"]:
@@ -186,7 +186,13 @@ def _load():
 
 
 def available() -> bool:
-    return _settings["enabled"] and _load() is not None and ctypes.sizeof(_Heuristic) == 56
+    return _load() is not None and ctypes.sizeof(_Heuristic) == 56
+
+
+def require() -> None:
+    if not available():
+        raise RuntimeError("hipBLASLt cannot be loaded (looked beside torch's libraries and in /opt/rocm/lib): the "
+                           "bfloat16 products of more than 32 rows have no other library")
 
 
 def _ok(status: int, what: str) -> None:
@@ -297,9 +303,13 @@ def chosen() -> list:
     return out
 
 
-def matmul(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, accumulate: bool = False) -> torch.Tensor:
+def matmul(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, accumulate: bool = False) -> bool:
     """out[:m] = a[:m] @ w.T; a, w bfloat16 with contiguous rows, out bfloat16 or float32. accumulate: out[:m] +=
-    instead, the sum of the float accumulators and out rounded once."""
+    instead, the sum of the float accumulators and out rounded once. False, and nothing done, where the library has
+    no algorithm for the shape."""
+    require()
+    if not (a.stride(1) == 1 and w.stride(1) == 1 and out.stride(1) == 1):
+        raise ValueError("library products take operands with contiguous rows")
     beta = _one if accumulate else _zero
     dev = a.device
     handle = _handles.get(dev)
@@ -316,22 +326,16 @@ def matmul(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, accumula
         try:
             plan = _Plan(handle, m, n, k, a.stride(0), w.stride(0), out.stride(0), out.dtype)
         except RuntimeError:
-            plan = False   # a shape the direct interface does not take: torch's own call of the library serves it
+            plan = False   # a shape the library takes no algorithm for
         _plans[key] = plan
     if plan is False:
-        if accumulate:
-            out[:m].addmm_(a[:m].to(out.dtype), w.t().to(out.dtype))
-        elif out.dtype == a.dtype:
-            torch.mm(a[:m], w.t(), out=out[:m])
-        else:
-            out[:m].copy_(torch.mm(a[:m], w.t()))
-        return out
+        return False
     workspace = _workspaces[dev]
     if (not plan.tuned and _settings["tuning"] == "measured" and m >= TUNE_FROM_ROWS and m * n * k >= TUNE_FROM_WORK
             and len(plan.candidates) > 1):
         _choose(handle, plan, key, a, w, out, workspace, beta)
     _run(handle, plan, plan.algo, a, w, out, workspace, beta)
-    return out
+    return True
 
 
 def _choose(handle, plan, key, a, w, out, workspace, beta) -> None:

@@ -4,8 +4,8 @@ float32 operands: the vector-ALU kernel with a fixed summation order (the true
 32-bit path). bfloat16 operands: up to 32 rows the hand-written MFMA kernel that
 streams the weight once (decode, LM head); beyond, the vendor library, where the
 reference uses a library too (crates/kernels/src/gemm.rs:605-647): hipBLASLt
-called directly with the algorithm measured per shape (blaslt.py), or through
-torch.mm where that library cannot be loaded. One shape is taken from both at 17
+called directly with the algorithm measured per shape (blaslt.py); a shape it
+names no algorithm for runs the plain kernel. One shape is taken from both at 17
 to 64 rows: a weight with far more columns than rows (the down projection of a
 feed-forward), where the few-row kernel drowns in loads of the activations and
 the library has few output tiles to spread; the kernel that keeps a slice of the
@@ -73,15 +73,10 @@ def _mid_workspace(dev, need: int) -> torch.Tensor | None:
 
 
 def _library(a, w, out, m, may_pad):
-    if blaslt.available() and a.stride(1) == 1 and w.stride(1) == 1 and out.stride(1) == 1:
-        # float32 out (logits at many positions): straight from the accumulators, as the few-row kernel gives them
-        rows = min(a.shape[0], out.shape[0], row_bucket(m)) if may_pad else m
-        return blaslt.matmul(a, w, out, rows)
-    if out.dtype == torch.float32:
-        tmp = torch.mm(a[:m], w.t())
-        ops.widen(tmp, out, m * w.shape[0]) if out.is_contiguous() else out[:m].copy_(tmp)
-        return out
-    torch.mm(a[:m], w.t(), out=out[:m])
+    # float32 out (logits at many positions): straight from the accumulators, as the few-row kernel gives them
+    rows = min(a.shape[0], out.shape[0], row_bucket(m)) if may_pad else m
+    if not blaslt.matmul(a, w, out, rows):
+        ops.gemm_ref(a, w, out, m)      # a shape the library names no algorithm for: the plain kernel takes any
     return out
 
 
@@ -144,11 +139,10 @@ def add_nt(a: torch.Tensor, w: torch.Tensor, stream: torch.Tensor, m: int) -> bo
     (rows beyond m hold nothing of value). False (nothing done) where the library does not run the product."""
     n, k = w.shape
     if not (a.is_cuda and a.dtype == torch.bfloat16 and stream.dtype == torch.bfloat16 and m > SMALL_M
-            and not _tall(m, n, k) and blaslt.available() and a.stride(1) == 1 and w.stride(1) == 1 and stream.stride(1) == 1):
+            and not _tall(m, n, k)):
         return False
     rows = min(a.shape[0], stream.shape[0], row_bucket(m))
-    blaslt.matmul(a, w, stream, rows, accumulate=True)
-    return True
+    return blaslt.matmul(a, w, stream, rows, accumulate=True)
 
 
 def scaled_nt(xg: torch.Tensor, stats: torch.Tensor, cols: int, eps: float, width: int, w: torch.Tensor, out: torch.Tensor,

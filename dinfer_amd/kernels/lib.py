@@ -66,7 +66,6 @@ SIGNATURES = {
     "dinfer_sample_scratch_bytes": ("sampling", [_L, _L, _P]),
     "dinfer_history_add": ("sampling", [_P, _L, _L, _P, _L, _P]),
     "dinfer_penalties_dense": ("sampling", [_P, _L, _P, _L, _P, _L, _L, _P]),
-    "dinfer_penalties": ("sampling", [_P, _L, _P, _P, _P, _P, _P, _P, _L, _L, _P]),
     "dinfer_logit_bias": ("sampling", [_P, _L, _P, _P, _L, _L, _L, _P]),
     "dinfer_logprobs": ("sampling", [_P, _L, _P, _P, _L, _P, _P, _P, _L, _L, _P]),
 }

@@ -494,18 +494,6 @@ def penalties_dense(logits: torch.Tensor, rows: int, history: torch.Tensor, pack
              packed.data_ptr(), rows, logits.shape[1], _stream())
 
 
-def penalties(logits: torch.Tensor, rows: int, ids: torch.Tensor, counts: torch.Tensor, offsets: torch.Tensor,
-              repetition: torch.Tensor, frequency: torch.Tensor, presence: torch.Tensor) -> None:
-    """In place on logits: per row, entries offsets[b]..offsets[b+1] list the distinct tokens of the
-    row's history with their count among the outputs (0: prompt only)."""
-    _need_gpu(logits, ids, counts, offsets, repetition, frequency, presence)
-    assert logits.dtype == torch.float32
-    assert ids.dtype == counts.dtype == offsets.dtype == torch.int32 and offsets.numel() >= rows + 1
-    lib.call("dinfer_penalties", logits.data_ptr(), _rows(logits), ids.data_ptr(), counts.data_ptr(),
-             offsets.data_ptr(), repetition.data_ptr(), frequency.data_ptr(), presence.data_ptr(), rows,
-             logits.shape[1], _stream())
-
-
 MAX_TOP_LOGPROBS = 32
 
 

@@ -61,21 +61,12 @@ class DecoderModel:
         self._load_from(lambda name, compute=False: loader.fetch(name, compute=compute), loader.has)
 
     def load_random(self, seed: int, device, dtype: torch.dtype) -> None:
-        """Draws every tensor on the device (matrix weights N(0, 0.02), gains 1 + N(0, 0.1));
-        for measurements at sizes where writing a file first would only cost time."""
+        """Draws every tensor on the device by the rule of the random-weights mode (weights/random_init.py: each
+        tensor from (seed, its name)); for measurements at sizes where writing a file first would only cost time."""
+        from ..weights.random_init import draw_on_device
         exp, _ = self.expected_tensors()
-        gen = torch.Generator(device=device)
-        gen.manual_seed(seed)
-
-        def get(name, compute=False):
-            s = exp[name]
-            if s.init == "gain":
-                t = torch.randn(s.shape, generator=gen, device=device, dtype=torch.float32) * 0.1 + 1.0
-            else:
-                t = torch.randn(s.shape, generator=gen, device=device, dtype=torch.float32) * 0.02
-            return t.to(dtype)
-
-        self._load_from(get, lambda name: name in exp)
+        self._load_from(lambda name, compute=False: draw_on_device(seed, name, exp[name], dtype, device),
+                        lambda name: name in exp)
 
     def _load_from(self, get, has) -> None:
         s = self.spec

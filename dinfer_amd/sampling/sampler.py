@@ -87,6 +87,7 @@ class Sampler:
         self._given_dev: torch.Tensor | None = None
         self._given_read: list | None = None
         self._given_turn = 0
+        self._arena: list | None = None             # per turn: [pinned bytes, bytes used, outgrown arenas still in flight]
 
     def _buffers(self) -> None:
         if self.work is not None:
@@ -138,10 +139,12 @@ class Sampler:
                 ops.argmax(logits, self.out, R, self._arg_scratch)
         else:
             assert not done
+            if self._arena is not None:
+                self._arena[turn][1], self._arena[turn][2] = 0, []
             if any(p.logit_bias for p, *_ in rows):         # before the penalties (sampling.cu:286)
-                self._bias(logits, rows)
+                self._bias(logits, rows, turn)
             if any(p.has_penalties for p, *_ in rows):
-                self._penalties(logits, rows)
+                self._penalties(logits, rows, turn)
             self._buffers()
             rec = self._rows_np[turn]
             for i, (p, n_out, _prompt, _output, seed, *_key) in enumerate(rows):
@@ -182,12 +185,31 @@ class Sampler:
         self._given_read[turn].record()
         return Sampled(self, R, host, self._given_read[turn], asked, about)
 
-    def _bias(self, logits, rows) -> None:
+    def _staged(self, turn: int, arr: np.ndarray, dtype: torch.dtype) -> torch.Tensor:
+        """arr on the device, sent through this turn's pinned arena without the host waiting for the stream (a copy
+        from pageable memory would wait for the kernels of the step before, and a step launched ahead would no longer
+        overlap with it). The arena of a turn was last read by the launch before the last, whose tokens have been
+        waited for since; one that has to grow is kept until the turn comes round again."""
+        if self._arena is None:
+            self._arena = [[torch.empty(1 << 16, dtype=torch.uint8, pin_memory=True), 0, []] for _ in range(2)]
+        raw = np.ascontiguousarray(arr).view(np.uint8).reshape(-1)
+        a = self._arena[turn]
+        start = (a[1] + 15) & ~15
+        if start + raw.size > a[0].numel():
+            a[2].append(a[0])
+            a[0], start = torch.empty(max(2 * a[0].numel(), raw.size), dtype=torch.uint8, pin_memory=True), 0
+        a[0].numpy()[start:start + raw.size] = raw
+        a[1] = start + raw.size
+        dev = torch.empty(raw.size, dtype=torch.uint8, device=self.device)
+        dev.copy_(a[0][start:start + raw.size], non_blocking=True)
+        return dev.view(dtype).view(arr.shape)
+
+    def _bias(self, logits, rows, turn: int) -> None:
         entries = [(i, t, b) for i, (p, *_rest) in enumerate(rows) for t, b in p.logit_bias.items() if t < self.vocab]
         if not entries:
             return
-        where = torch.tensor([(i, t) for i, t, _ in entries], dtype=torch.int32).to(self.device)
-        what = torch.tensor([b for *_, b in entries], dtype=torch.float32).to(self.device)
+        where = self._staged(turn, np.array([(i, t) for i, t, _ in entries], dtype=np.int32), torch.int32)
+        what = self._staged(turn, np.array([b for *_, b in entries], dtype=np.float32), torch.float32)
         ops.logit_bias(logits, len(rows), where, what)
 
     def _logprobs(self, given, asked, R: int, turn: int, chosen=None) -> tuple:
@@ -221,7 +243,7 @@ class Sampler:
         if st is not None:
             self._free.append(st[0])
 
-    def _penalties(self, logits, rows) -> None:
+    def _penalties(self, logits, rows, turn: int) -> None:
         """Repetition, frequency and presence penalties, in place. The tokens a request has seen live on the
         device ([max_rows, vocab] int32, a slot per request with penalties); only what is new goes there:
         the distinct prompt tokens once, then the outputs since the last step."""
@@ -254,7 +276,7 @@ class Sampler:
                 st[1] = len(output)
                 pen[i] = (slot, p.repetition_penalty, p.frequency_penalty, p.presence_penalty)
             if entries:
-                ops.history_add(self.history, torch.from_numpy(np.asarray(entries, dtype=np.int32)).to(self.device))
-            ops.penalties_dense(logits, R, self.history, torch.from_numpy(pen.view(np.uint8)).to(self.device))
+                ops.history_add(self.history, self._staged(turn, np.asarray(entries, dtype=np.int32), torch.int32))
+            ops.penalties_dense(logits, R, self.history, self._staged(turn, pen.view(np.uint8), torch.uint8))
         finally:
             self._free += passing

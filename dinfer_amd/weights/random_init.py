@@ -44,6 +44,24 @@ def draw(seed: int, name: str, spec: TensorSpec, dtype: torch.dtype) -> torch.Te
     return t.to(dtype)
 
 
+def draw_on_device(seed: int, name: str, spec: TensorSpec, dtype: torch.dtype, device) -> torch.Tensor:
+    """The same rule as draw() (one generator per tensor, seeded by (seed, name); the same distributions), drawn by
+    the device's generator: for measurements at sizes where a file would only cost time. The device's generator is
+    another algorithm than the host's, so the values are not those of a folder written with the same seed."""
+    if spec.integer or spec.init in ("zeros", "ones"):
+        return draw(seed, name, spec, dtype).to(device)
+    g = torch.Generator(device=device)
+    g.manual_seed(tensor_seed(seed, name))
+    t = torch.randn(spec.shape, generator=g, device=device, dtype=torch.float32)
+    if spec.init == "linear":
+        t *= LINEAR_STD
+    elif spec.init == "gain":
+        t = 1.0 + t * GAIN_STD
+    else:
+        raise ValueError(f"tensor {name!r}: unknown init {spec.init!r}")
+    return t.to(dtype)
+
+
 def write_random_model(config, out_dir: str | Path, seed: int = 0, dtype: str = "bfloat16") -> Path:
     """config: a typed configuration of a registered architecture. Returns the folder."""
     from ..config.registry import get_architecture

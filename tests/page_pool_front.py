@@ -1,4 +1,5 @@
-"""A pool of cache pages (front of the C++ class in csrc/host/block_pool.hpp).
+"""A pool of cache pages on its own, for the tests of the C++ class in csrc/host/block_pool.hpp (the engine reaches
+that class only through the cache manager, which holds one pool per group).
 
 ``allocate(n)`` is all-or-nothing and takes pages from the head of the free
 list; ``free(ids)`` puts the pages back at the head in the order given, so pages
@@ -10,7 +11,7 @@ from __future__ import annotations
 
 import ctypes
 
-from .. import native
+from dinfer_amd import native
 
 
 class BlockPool:

@@ -4,7 +4,8 @@ import random
 
 import pytest
 
-from dinfer_amd.cache import BlockPool, CacheManager, GroupSpec
+from dinfer_amd.cache import CacheManager, GroupSpec
+from page_pool_front import BlockPool
 
 
 def test_alloc_free_roundtrip():

@@ -63,6 +63,20 @@ def test_window_layers():
     assert Qwen3Config.from_dict(BASE).layer_window(2) is None
 
 
+def test_layer_types_must_say_what_the_window_keys_say():
+    """Newer config.json files list each layer's kind; the list is read and a file whose list and keys disagree is refused."""
+    win = CONFIGS["C"][0]                                   # 5 layers, the window from layer 2 on
+    ok = ["full_attention"] * 2 + ["sliding_attention"] * 3
+    assert Qwen3Config.from_dict({**win, "layer_types": ok}).layer_types == tuple(ok)
+    assert Qwen3Config.from_dict({**BASE, "layer_types": ["full_attention"] * BASE["num_hidden_layers"]}).layer_window(0) is None
+    for bad, needle in ((["full_attention"] * 5, "layer 2"), (ok[:4], "lists 4"), (ok[:4] + ["chunked"], "chunked"),
+                        ("full_attention", "layer_types")):
+        with pytest.raises(ConfigError, match=needle):
+            Qwen3Config.from_dict({**win, "layer_types": bad})
+    with pytest.raises(ConfigError, match="layer 0"):       # a list that asks for windows the keys switch off
+        Qwen3Config.from_dict({**BASE, "layer_types": ["sliding_attention"] * BASE["num_hidden_layers"]})
+
+
 def test_round_trip_through_config_json(tmp_path):
     for name, (cfg, _) in CONFIGS.items():
         c = Qwen3Config.from_dict(cfg)

@@ -69,13 +69,20 @@ def judge_greedy(cfg, w, prompt, tokens, slack=0.1):
     return best
 
 
-def test_bfloat16_generation_follows_plain_up_to_near_ties(model_dirs):
+@pytest.mark.parametrize("fast", [True, False], ids=["graphs_and_steps_ahead", "eager_step_by_step"])
+def test_bfloat16_generation_follows_plain_up_to_near_ties(model_dirs, fast):
+    """fast: as the engine serves by default: decode steps replayed from graphs that find their best tokens
+    themselves, each launched before the tokens of the one before it are read (its input stays on the device).
+    Every token is judged against the plain model's logits after the tokens before it."""
     from dinfer_amd import SamplingParams
     name = "B"
     cfg, w = plain.load(model_dirs[name])
     prompts = prompts_for(name, [9, 40, 70], 8)
-    got = engine(model_dirs[name], name, dtype="bfloat16").generate(
-        prompts, SamplingParams(max_tokens=12, temperature=0.0, ignore_eos=True))
+    eng = engine(model_dirs[name], name, dtype="bfloat16", hip_graph=fast, async_scheduling=fast)
+    got = eng.generate(prompts, SamplingParams(max_tokens=12, temperature=0.0, ignore_eos=True))
+    assert bool(eng.runner._graphs) == fast and (eng.steps_launched_ahead >= 8) == fast
+    if fast:
+        assert all(greedy for _, greedy in eng.runner._graphs), "the graphs' own argmax chose the tokens"
     best = sum(judge_greedy(cfg, w, p, g) for p, g in zip(prompts, got))
     assert best >= 30, f"only {best} of 36 tokens are the plain model's first choice"
 

@@ -766,22 +766,21 @@ def test_sample_paths_agree_at_the_edges_of_the_options():
 
 
 def test_penalties_match_plain_rule():
+    import numpy as np
     V = 512
-    logits = torch.randn(4, V, device=DEV) * 3
-    hist = [([1, 5, 9, 5], [9, 9, 20]), ([3], []), ([7, 7, 7], [7, 100]), ([], [2, 4, 6, 4])]
-    rep, freq, pres = [1.5, 1.0, 1.2, 1.0], [0.0, 0.0, 0.3, 0.5], [0.0, 0.0, 0.2, 0.1]
-    ids, cnt, offs = [], [], [0]
-    for p, o in hist:
-        for t in sorted(set(p) | set(o)):
-            ids.append(t)
-            cnt.append(o.count(t))
-        offs.append(len(ids))
+    logits = torch.randn(5, V, device=DEV) * 3
+    hist = [([1, 5, 9, 5], [9, 9, 20]), ([3], []), ([7, 7, 7], [7, 100]), ([], [2, 4, 6, 4]), ([8], [8])]
+    rep, freq, pres = [1.5, 1.0, 1.2, 1.0, 2.0], [0.0, 0.0, 0.3, 0.5, 1.0], [0.0, 0.0, 0.2, 0.1, 0.5]
+    slots = [2, 0, 3, 1, -1]                                # the last row takes no penalties at all
+    history = torch.zeros(4, V, dtype=torch.int32, device=DEV)
+    entries = [(s, t, 0) for s, (p, _) in zip(slots, hist) if s >= 0 for t in set(p)]
+    entries += [(s, t, 1) for s, (_, o) in zip(slots, hist) if s >= 0 for t in o]
+    ops().history_add(history, torch.tensor(entries, dtype=torch.int32, device=DEV))
+    pen = np.array(list(zip(slots, rep, freq, pres)), dtype=ops().PENALTY_ROW)
     got = logits.clone()
-    i32 = lambda xs: torch.tensor(xs, device=DEV, dtype=torch.int32)
-    f32 = lambda xs: torch.tensor(xs, device=DEV, dtype=torch.float32)
-    ops().penalties(got, 4, i32(ids), i32(cnt), i32(offs), f32(rep), f32(freq), f32(pres))
+    ops().penalties_dense(got, 5, history, torch.from_numpy(pen.view(np.uint8)).to(DEV))
     for r, (p, o) in enumerate(hist):
-        want = plain.apply_penalties(logits[r].cpu().double(), p, o, rep[r], freq[r], pres[r])
+        want = logits[r].cpu().double() if slots[r] < 0 else plain.apply_penalties(logits[r].cpu().double(), p, o, rep[r], freq[r], pres[r])
         torch.testing.assert_close(got[r].cpu().double(), want, rtol=1e-6, atol=1e-6)
 
 
@@ -854,7 +853,7 @@ def test_library_gemm_with_measured_algorithm(tmp_path):
     buffers: the rows asked for are right, rows past the bucket untouched."""
     import json
     from dinfer_amd.kernels import blaslt, gemm
-    blaslt.configure(enabled=True, tuning="measured", plan_file=str(tmp_path / "plans.json"))
+    blaslt.configure(tuning="measured", plan_file=str(tmp_path / "plans.json"))
     blaslt._plans.clear()                                                    # what earlier tests of this process met
     assert blaslt.available()
     a = torch.randn(200, 1096, device=DEV).to(torch.bfloat16)
@@ -903,7 +902,7 @@ def test_library_gemm_adds_into_its_output(tmp_path):
     itself gets the product once), later calls add once each; rows past the bucket are untouched; the few-row and
     tall shapes are refused (other kernels serve them)."""
     from dinfer_amd.kernels import blaslt, gemm
-    blaslt.configure(enabled=True, tuning="measured", plan_file=str(tmp_path / "plans.json"))
+    blaslt.configure(tuning="measured", plan_file=str(tmp_path / "plans.json"))
     blaslt._plans.clear()
     assert blaslt.available()
     with blaslt.measuring():

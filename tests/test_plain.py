@@ -130,6 +130,119 @@ def test_model_options_matter(tiny):
     assert "lm_head.weight" not in wA
 
 
+def variant_forward(cfg, w, ids, first_position=0, mistake=None):
+    """The model put together again from the plain parts, with one mistake of composition at a time (None: none, and
+    then it must be plain.forward). Used to show that the pins below tell each mistake from the right composition."""
+    T, eps = len(ids), cfg["rms_norm_eps"]
+    H, Hkv, D = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    norm = (lambda x, g: plain.rms_norm(x, 1 + g, eps)) if mistake == "gain_is_one_plus_w" else (lambda x, g: plain.rms_norm(x, g, eps))
+    ang = plain.rope_angles(list(range(first_position, first_position + T)), D, cfg["rope_theta"])
+    h = plain.embedding(ids, w["model.embed_tokens.weight"])
+    for l in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{l}."
+        a = p + "self_attn."
+        x = h if mistake == "post_norm" else norm(h, w[p + "input_layernorm.weight"])
+        q = (x @ w[a + "q_proj.weight"].T).view(T, H, D)
+        k = (x @ w[a + "k_proj.weight"].T).view(T, Hkv, D)
+        v = (x @ w[a + "v_proj.weight"].T).view(T, Hkv, D)
+        gq, gk = w[a + "q_norm.weight"], w[a + "k_norm.weight"]
+        if mistake == "rotation_before_norm":
+            q, k = norm(plain.rope_neox(q, ang), gq), norm(plain.rope_neox(k, ang), gk)
+        elif mistake == "norm_over_all_heads":
+            q = norm(q.reshape(T, 1, H * D), gq.repeat(H)).view(T, H, D)
+            k = norm(k.reshape(T, 1, Hkv * D), gk.repeat(Hkv)).view(T, Hkv, D)
+            q, k = plain.rope_neox(q, ang), plain.rope_neox(k, ang)
+        else:
+            q, k = plain.rope_neox(norm(q, gq), ang), plain.rope_neox(norm(k, gk), ang)
+        if mistake == "v_normed":
+            v = norm(v, gk)
+        if mistake == "v_rotated":
+            v = plain.rope_neox(v, ang)
+        o = plain.causal_attention(q, k, v, D ** -0.5, plain.layer_window(cfg, l)).reshape(T, H * D) @ w[a + "o_proj.weight"].T
+        h_mid = norm(h + o, w[p + "input_layernorm.weight"]) if mistake == "post_norm" else h + o
+        y = h_mid if mistake == "post_norm" else norm(h if mistake == "mlp_reads_the_layer_input" else h_mid,
+                                                      w[p + "post_attention_layernorm.weight"])
+        m = plain.swiglu_mlp(y, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+        h = norm(h_mid + m, w[p + "post_attention_layernorm.weight"]) if mistake == "post_norm" else h_mid + m
+    h = norm(h, w["model.norm.weight"])
+    return h @ (w["lm_head.weight"] if "lm_head.weight" in w else w["model.embed_tokens.weight"]).T
+
+
+def pin_shift(f, cfg, w, ids):
+    """Only distances between positions count."""
+    return torch.allclose(f(cfg, w, ids, 0), f(cfg, w, ids, 37), rtol=1e-9, atol=1e-9)
+
+
+def pin_single_token(f, cfg, w, ids):
+    """A sequence of one token attends to itself alone: its attention is its value row as the projection left it,
+    whatever the q and k norms, the rotation and the position are; library operations only."""
+    G = cfg["num_attention_heads"] // cfg["num_key_value_heads"]
+    D, eps = cfg["head_dim"], cfg["rms_norm_eps"]
+    rms = lambda x, g: x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * g
+    h = w["model.embed_tokens.weight"][ids[:1]]
+    for l in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{l}."
+        v = F.linear(rms(h, w[p + "input_layernorm.weight"]), w[p + "self_attn.v_proj.weight"])
+        h = h + F.linear(v.view(-1, D).repeat_interleave(G, 0).reshape(1, -1), w[p + "self_attn.o_proj.weight"])
+        y = rms(h, w[p + "post_attention_layernorm.weight"])
+        h = h + F.linear(F.silu(F.linear(y, w[p + "mlp.gate_proj.weight"])) * F.linear(y, w[p + "mlp.up_proj.weight"]),
+                         w[p + "mlp.down_proj.weight"])
+    want = F.linear(rms(h, w["model.norm.weight"]), w.get("lm_head.weight", w["model.embed_tokens.weight"]))
+    return torch.allclose(f(cfg, w, ids[:1], 5), want, rtol=1e-9, atol=1e-9)
+
+
+def pin_head_scale(f, cfg, w, ids):
+    """The q and k norms are per head: making one head's projection rows larger changes nothing (eps aside)."""
+    D = cfg["head_dim"]
+    cfg0 = {**cfg, "rms_norm_eps": 1e-30}
+    w2 = dict(w)
+    for l in range(cfg["num_hidden_layers"]):
+        a = f"model.layers.{l}.self_attn."
+        w2[a + "q_proj.weight"] = w[a + "q_proj.weight"].clone()
+        w2[a + "q_proj.weight"][D:2 * D] *= 7.0
+        w2[a + "k_proj.weight"] = w[a + "k_proj.weight"].clone()
+        w2[a + "k_proj.weight"][:D] *= 0.3
+    return torch.allclose(f(cfg0, w2, ids, 0), f(cfg0, w, ids, 0), rtol=1e-8, atol=1e-8)
+
+
+def pin_silent_branches(f, cfg, w, ids):
+    """With output and down projections of zero both branches add nothing: the logits are the final norm of the
+    embeddings times the head (the stream passes every layer untouched, and is normed once, at the end)."""
+    w2 = {k: (torch.zeros_like(v) if k.endswith(("o_proj.weight", "down_proj.weight")) else v) for k, v in w.items()}
+    h = w["model.embed_tokens.weight"][ids]
+    h = h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + cfg["rms_norm_eps"]) * w["model.norm.weight"]
+    return torch.allclose(f(cfg, w2, ids, 0), F.linear(h, w.get("lm_head.weight", w["model.embed_tokens.weight"])), rtol=1e-9, atol=1e-9)
+
+
+def pin_zero_gain_silences(f, cfg, w, ids):
+    """The gain multiplies (no 1 + w): layer norms with gains of zero feed zeros to both branches."""
+    w2 = {k: (torch.zeros_like(v) if k.endswith(("input_layernorm.weight", "post_attention_layernorm.weight")) else v)
+          for k, v in w.items()}
+    return pin_silent_branches(lambda c, ww, i, p: f(c, w2, i, p), cfg, w, ids)
+
+
+def test_each_mistake_of_composition_fails_a_pin(tiny):
+    """What fixes the composition of a layer besides the reference's text (models/qwen3/src/model.rs:708-813,
+    crates/kernels/cuda/qkv_post.cu:48-76; the same formulas a second time in the reference's own Python,
+    scripts/verify/gen_kernel_refs.py:289-322): invariants and special cases that reduce to library routines. The
+    right composition keeps all of them; each plausible mistake breaks the one named beside it. Two conventions have
+    no anchor but those texts: that a gain multiplies as it is (and not as 1 + w), which the last pin spells out, and
+    the order of a block (norm, branch, add; the feed-forward reads the stream after attention), which the one-token
+    case spells out in library operations. An installed package's model code is no source here and is not imported."""
+    pins = {"rotation_before_norm": pin_shift, "v_rotated": pin_shift, "v_normed": pin_single_token,
+            "norm_over_all_heads": pin_head_scale, "post_norm": pin_silent_branches,
+            "mlp_reads_the_layer_input": pin_single_token, "gain_is_one_plus_w": pin_zero_gain_silences}
+    for name, (cfg, w) in tiny.items():
+        ids = [(11 * i + 2) % cfg["vocab_size"] for i in range(30)]
+        torch.testing.assert_close(variant_forward(cfg, w, ids), plain.forward(cfg, w, ids), rtol=0, atol=0)
+        for pin in set(pins.values()):
+            assert pin(plain.forward, cfg, w, ids), f"{name}: the plain model breaks {pin.__name__}"
+        for mistake, pin in pins.items():
+            wrong = lambda c, ww, i, p=0, m=mistake: variant_forward(c, ww, i, p, m)
+            assert not torch.allclose(wrong(cfg, w, ids), plain.forward(cfg, w, ids), atol=1e-6), f"{mistake} changes nothing"
+            assert not pin(wrong, cfg, w, ids), f"{name}: {mistake} passes {pin.__name__}"
+
+
 def test_layer_against_a_hand_rolled_single_head_case():
     """One layer, one head, identity-like weights: every step can be followed by hand."""
     Hd = 8

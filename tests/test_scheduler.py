@@ -518,6 +518,25 @@ def test_nothing_is_planned_ahead_when_someone_waits_or_pages_are_short():
     assert not s.can_look_ahead()                       # a step ahead might have to preempt: it waits
 
 
+def test_nothing_is_planned_ahead_while_a_running_request_is_left_out_of_the_step():
+    """A request in mid-prompt whose next portion cannot end at an aligned position is left out of a step; the step
+    then holds one decoding row only, but not everyone who runs is in it: a step planned ahead would take "every
+    row waits for the running step" for granted of a request that does not, so it is planned after the update."""
+    s = mk(8, 20, 32, prefill_chunk_alignment=16, long_prefill_token_threshold=10)
+    s.add_request(req(2, 40, 100))
+    out = s.schedule()                                  # alone: no threshold, 20 tokens cut to the aligned 16
+    assert [(x.request.id, x.num_new) for x in out.scheduled] == [(2, 16)]
+    s.update(out, {})
+    s.add_request(req(1, 1, 100))
+    out = s.schedule()                                  # two are eligible: portions of 10 at most, none ends at 32
+    assert [(x.request.id, x.num_new, x.samples) for x in out.scheduled] == [(1, 1, True)]
+    assert not s.can_look_ahead()
+    with pytest.raises(ValueError):
+        s.schedule(ahead=True)
+    s.update(out, {1: 7})
+    s.cache.check()
+
+
 def test_random_loads_planned_ahead_match_step_by_step():
     import random
     looked = 0
