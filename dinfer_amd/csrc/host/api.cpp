@@ -189,6 +189,13 @@ int32_t dh_batch_fill(void* cache, const dh_batch_buffers* buf, int32_t n, const
     });
 }
 
+int32_t dh_batch_pad(const dh_batch_buffers* buf, dh_batch_facts* facts, int32_t reqs, int32_t tokens, int32_t rows) {
+    return guarded([&] {
+        pad_batch(*reinterpret_cast<const BatchBuffers*>(buf), reinterpret_cast<BatchFacts*>(facts), reqs, tokens, rows);
+        return 0;
+    });
+}
+
 // ---- scheduler
 void* dh_sched_create(const dh_sched_options* opt, void* cache, const int32_t* eos, int32_t n_eos) {
     void* out = nullptr;

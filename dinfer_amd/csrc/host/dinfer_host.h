@@ -75,6 +75,10 @@ int32_t dh_batch_fill(void* cache, const dh_batch_buffers* buf, int32_t n, const
                       const int32_t* counts, const int32_t* tokens, const int32_t* want_counts, const int32_t* wants,
                       int32_t pad_to, dh_batch_facts* facts);
 
+/* Fills a written step up to `reqs` requests, `tokens` tokens and `rows` logits rows with made-up requests that
+ * write nothing (one token each, the last one the rest), so that it can replay a graph captured for those counts. */
+int32_t dh_batch_pad(const dh_batch_buffers* buf, dh_batch_facts* facts, int32_t reqs, int32_t tokens, int32_t rows);
+
 /* ---- scheduler */
 typedef struct {
     int32_t max_num_batched_tokens, max_num_seqs, max_model_len, prefill_tokens_per_step,

@@ -17,6 +17,8 @@
 // is filled up with requests of one token at position 0 that write no cache slot (slot -1) and
 // read page 0, which always exists (crates/layers/src/exec.rs:388-426). Their state slot is max_reqs,
 // one past the slots requests can hold: per-request state is allocated with that spare slot at its end.
+// pad_batch() does the same for any step after it was filled: requests and tokens up to given counts (the made-up
+// requests bring one token each, the last of them the rest), logits rows up to a given count.
 #pragma once
 #include <cstdint>
 #include <cstring>
@@ -156,6 +158,47 @@ inline void fill_batch(const CacheManager& cache, const BatchBuffers& buf, const
     facts->num_tokens = static_cast<int32_t>(T);
     facts->num_reqs = Bp;
     facts->num_rows = static_cast<int32_t>(R);
+    facts->max_q_len = max_q;
+    facts->max_seq_len = max_len;
+    facts->num_singles = singles;
+}
+
+// Fills a step that fill_batch has written up to reqs requests, tokens tokens and rows logits rows, so that it
+// can replay a graph captured for those counts. The made-up requests start at position 0, write no cache slot
+// (slot -1), hold page 0 in every column of their block table (it always exists; what they read there counts for
+// nothing) and the spare state slot; each brings one token, the last one whatever is still missing. The made-up
+// logits rows point at the first made-up token (or at row 0). facts: the step's, brought up to date.
+inline void pad_batch(const BatchBuffers& buf, BatchFacts* facts, int reqs, int tokens, int rows) {
+    const int B = facts->num_reqs, T = facts->num_tokens, R = facts->num_rows;
+    if (reqs < B || tokens < T || rows < R || reqs > buf.max_reqs || tokens > buf.max_tokens || rows > buf.max_rows)
+        throw Error(ERR_VALUE, "a step can be padded up to the engine's sizes only, never cut");
+    const int more_reqs = reqs - B, more_tokens = tokens - T;
+    if ((more_reqs == 0) != (more_tokens == 0) || more_tokens < more_reqs)
+        throw Error(ERR_VALUE, "made-up requests bring at least one token each, and made-up tokens need a request");
+    int t = T, max_q = facts->max_q_len, max_len = facts->max_seq_len, singles = facts->num_singles;
+    for (int b = B; b < reqs; ++b) {
+        const int n = b + 1 < reqs ? 1 : tokens - t;
+        for (int i = 0; i < n; ++i) {
+            buf.input_ids[t + i] = 0;
+            buf.feedback_src[t + i] = -1;
+            buf.positions[t + i] = i;
+            for (int g = 0; g < buf.n_groups; ++g) buf.slot_mapping[g][t + i] = -1;
+        }
+        for (int g = 0; g < buf.n_groups; ++g)
+            std::memset(buf.block_table[g] + static_cast<int64_t>(b) * buf.max_blocks[g], 0,
+                        sizeof(int32_t) * buf.max_blocks[g]);
+        buf.cu_seqlens[b + 1] = t + n;
+        buf.seq_lens[b] = n;
+        buf.state_slots[b] = buf.max_reqs;
+        max_q = n > max_q ? n : max_q;
+        max_len = n > max_len ? n : max_len;
+        singles += n == 1;
+        t += n;
+    }
+    for (int r = R; r < rows; ++r) buf.logits_rows[r] = more_tokens > 0 ? T : 0;
+    facts->num_tokens = tokens;
+    facts->num_reqs = reqs;
+    facts->num_rows = rows;
     facts->max_q_len = max_q;
     facts->max_seq_len = max_len;
     facts->num_singles = singles;

@@ -149,6 +149,14 @@ class StepBatch:
         self.max_q_len, self.max_seq_len, self.num_singles = f.max_q_len, f.max_seq_len, f.num_singles
         self.all_decode = f.num_singles == f.num_reqs
 
+    def pad(self, reqs: int, tokens: int, rows: int) -> None:
+        """After fill(): made-up requests that write nothing bring the step to these counts (csrc/host/step_batch.hpp,
+        pad_batch), so that it has the launch shapes of a graph captured for them."""
+        rc = native.fn("dh_batch_pad")(self._buffers, self._facts, reqs, tokens, rows)
+        if rc < 0:
+            raise native.error(rc)
+        self._take_facts()
+
     def upload(self) -> None:
         self._dev.copy_(self._host, non_blocking=True)
         if self._copied is not None:

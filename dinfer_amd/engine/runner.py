@@ -99,6 +99,12 @@ class ModelRunner:
         self._capture_stream = None
         # a step is replayed from a graph only where every part reads what changes between steps from device memory
         self._graphs_allowed = bool(options.hip_graph) and model.capturable()
+        # steps with prompt portions: padded up to a few counts, and replayed from a graph of their own once the same
+        # counts have come up PORTION_GRAPH_AFTER times (a capture costs about two eager steps)
+        self._portion_graphs_allowed = self._graphs_allowed and model.capturable_portions()
+        self._portion_graphs: dict[tuple, torch.cuda.CUDAGraph] = {}
+        self._portion_seen: dict[tuple, int] = {}
+        self.portion_replays = 0            # steps with prompt portions served by a replay
         if self._graphs_allowed and self.device.type == "cuda":
             _first_graph(self.device)
         self.warm_up()
@@ -280,6 +286,8 @@ class ModelRunner:
         self.argmax_done = False
         if self._graphs_allowed and single_rows and 0 < n <= self._buckets[-1]:
             out = self._graph_step(n, fill, greedy)
+        elif self._portion_graphs_allowed and not single_rows:
+            out = self._portion_step(fill)
         else:
             self._send(fill, None)
             self._reset_fresh_slots()
@@ -289,12 +297,17 @@ class ModelRunner:
             self.phases["launch"] += time.perf_counter() - self._began
         return out
 
-    def _send(self, fill, pad) -> None:
+    def _send(self, fill, pad, shape=None):
         """Writes the step into the pinned buffer and starts its copy to the device. While phases are measured
         (Engine.measure_phases) the host's time up to here counts as "fill", what follows as "launch", and two events
-        bracket the step on the device."""
+        bracket the step on the device. shape: called between the two, may pad the step; its result is returned."""
         fill(pad)
+        shaped = shape() if shape is not None else None
         self.batch.upload()
+        self._mark_sent()
+        return shaped
+
+    def _mark_sent(self) -> None:
         if self.phases is not None:
             import time
             now = time.perf_counter()
@@ -332,6 +345,70 @@ class ModelRunner:
                 ops.argmax(logits, b.last_tokens, bucket, self._argmax_scratch)
 
         forward()
+        self._graphs[(bucket, greedy)] = self._capture(forward)
+        return self.model.logits[:n]
+
+    PORTION_GRAPH_AFTER = 2     # a step's counts must have come up this often before a graph is captured for them
+    MAX_PORTION_GRAPHS = 96
+
+    def _portion_shape(self):
+        """Pads the step just filled up to counts that a graph can stand for, and makes the host-side facts parts
+        choose kernels by a function of those counts alone. Returns (key, logits rows of the real requests), or None
+        where the step stays as it is (and runs eagerly): it wants more rows than it has requests, or no padding fits.
+
+        The counts: tokens up to the next row count the matrix products round to anyway (16 at most where the
+        step has no more: the few-row products take other forms there), requests up to the next
+        bucket of the decode graphs, one logits row a request (none if the step wants none), the longest portion up
+        to the next power of two, and which of the three ways single rows are served (all of them are, some, none)."""
+        b, opt = self.batch, self.options
+        T, B, R = b.num_tokens, b.num_reqs, b.num_rows
+        if R > B or B > self._buckets[-1]:
+            return None
+        later = [x for x in self._buckets if x >= B]
+        Bp = Tp = None
+        for cand in later:
+            need = T + (cand - B)               # a made-up request brings a token at least
+            # (up to 16 rows the products take the norms along: such a step stays one)
+            tp = 16 if need <= 16 else gemm.row_bucket(need)
+            if tp > T and cand == B:
+                continue                        # made-up tokens need a made-up request
+            Bp, Tp = cand, tp
+            break
+        if Bp is None or Tp > self.max_tokens or (R and Bp > self.max_rows):
+            return None
+        last = Tp - T - (Bp - B - 1) if Bp > B else 0         # tokens of the last made-up request
+        if last > opt.max_model_len:
+            return None
+        real_rows = R
+        b.pad(Bp, Tp, Bp if R else 0)
+        q = b.max_q_len
+        qp = min(Tp, max(16, 1 << (q - 1).bit_length()))
+        route = 2 if b.num_singles == Bp else 1 if b.num_singles >= 4 else 0
+        b.max_q_len, b.all_decode = qp, route == 2
+        b.num_singles = Bp if route == 2 else 4 if route == 1 else 0
+        return (Tp, Bp, b.num_rows, qp, route), real_rows
+
+    def _portion_step(self, fill) -> torch.Tensor:
+        """A step with prompt portions: eager the first times its counts come up, then captured, then replayed."""
+        b = self.batch
+        shaped = self._send(fill, None, self._portion_shape)
+        self._reset_fresh_slots()
+        if shaped is None:
+            return self.model.forward(b, self.cache_views)
+        key, rows = shaped
+        g = self._portion_graphs.get(key)
+        if g is not None:
+            g.replay()
+            self.portion_replays += 1
+            return self.model.logits[:rows]
+        self.model.forward(b, self.cache_views)
+        seen = self._portion_seen[key] = self._portion_seen.get(key, 0) + 1
+        if seen >= self.PORTION_GRAPH_AFTER and len(self._portion_graphs) < self.MAX_PORTION_GRAPHS:
+            self._portion_graphs[key] = self._capture(lambda: self.model.forward(b, self.cache_views))
+        return self.model.logits[:rows]
+
+    def _capture(self, forward) -> torch.cuda.CUDAGraph:
+        """Records forward()'s launches into a graph without running them (the step has run eagerly just before)."""
         torch.cuda.synchronize()
         g = torch.cuda.CUDAGraph()
         if self._capture_stream is None:
@@ -348,8 +425,7 @@ class ModelRunner:
         torch.cuda.current_stream().wait_stream(side)
         if self._graph_pool is None:
             self._graph_pool = g.pool()
-        self._graphs[(bucket, greedy)] = g
-        return self.model.logits[:n]
+        return g
 
     # ---- request bookkeeping shared by replay and tests ------------------------------------------
     def reserve(self, req_id, start: int, n: int) -> bool:

@@ -75,6 +75,7 @@ _SIGNATURES = {
     "dh_cache_free_list": (_I, [_P, _I, _P, _I]),
     "dh_cache_check": (_I, [_P]),
     "dh_batch_fill": (_I, [_P, POINTER(BatchBuffers), _I, _P, _P, _P, _P, _P, _P, _I, POINTER(BatchFacts)]),
+    "dh_batch_pad": (_I, [POINTER(BatchBuffers), POINTER(BatchFacts), _I, _I, _I]),
     "dh_sched_create": (_P, [POINTER(SchedOptions), _P, _P, _I]),
     "dh_sched_destroy": (None, [_P]),
     "dh_sched_add": (_I, [_P, _L, _P, _I, _I, _I, _I, _P, _I, _I]),

@@ -21,6 +21,7 @@ from .spec import KVSpec, PartSpec, TensorSpec
 class Attention(Mixer):
     carries_norms = True   # the q/k/v product takes a Carried, the output product an Into
     capturable = True      # every kernel reads tokens, positions, slots, tables and lengths from the batch's device buffers
+    capturable_portions = True   # the choice of kernels follows the step's counts alone
 
     def __init__(self, hidden: int, heads: int, kv_heads: int, head_dim: int, position: PartSpec,
                  qk_norm: PartSpec | None = None, window: int | None = None, scale: float | None = None):

@@ -63,6 +63,8 @@ class BuildContext:
 class Part:
     # True: forward reads what changes from step to step from the batch's device tensors only (see Mixer.capturable)
     capturable = True
+    # the same promise for steps with prompt portions (see Mixer.capturable_portions)
+    capturable_portions = True
 
     def tensors(self) -> dict[str, TensorSpec]:
         """Local tensor name -> what the weight file must hold for it."""
@@ -177,6 +179,11 @@ class Mixer(Part):
     # single rows captured once may be replayed for other requests. A mixer that leaves it False keeps every step of
     # its model eager.
     capturable = False
+    # True: the promise of `capturable` also holds for steps that bring prompt portions, and whatever forward decides
+    # on the host depends on batch.num_tokens, num_reqs, num_rows, max_q_len and num_singles alone (which such a
+    # graph fixes: a step is padded up to them), never on the single requests' lengths (batch.q_lens and the like).
+    # Then steps with portions whose counts come up again are replayed from graphs of their own.
+    capturable_portions = False
 
     def cache_spec(self) -> CacheSpec | None:
         """What this mixer keeps between steps (a KVSpec, a StateSpec, a CacheSpec of its own), or None."""
@@ -207,6 +214,7 @@ class Block(Part):
     """
     carries_norms = False
     capturable = False   # an arrangement says so itself once all its parts are (see Mixer.capturable)
+    capturable_portions = False
 
     def input_norm(self):
         """The norm this block applies to the stream first, if the block before may carry it; else None."""

@@ -49,6 +49,10 @@ class PreNormBlock(Block):
     def capturable(self):
         return all(part.capturable for _, part in self._parts())
 
+    @property
+    def capturable_portions(self):
+        return all(part.capturable and part.capturable_portions for _, part in self._parts())
+
     def tensors(self):
         return {p + n: s for p, part in self._parts() for n, s in part.tensors().items()}
 

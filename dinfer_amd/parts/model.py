@@ -93,6 +93,11 @@ class DecoderModel:
         """Whether a step of single rows may be captured once and replayed for other requests."""
         return all(self.blocks[e.layer].capturable for e in self.run) and self.final_norm.capturable
 
+    def capturable_portions(self) -> bool:
+        """The same for steps with prompt portions (Mixer.capturable_portions)."""
+        return (self.capturable() and all(self.blocks[e.layer].capturable_portions for e in self.run)
+                and self.final_norm.capturable_portions)
+
     # ---- execution -----------------------------------------------------------------------------
     def bind(self, ctx: BuildContext) -> None:
         self.ctx = ctx

@@ -89,6 +89,39 @@ def test_padding_for_a_graph_bucket():
     assert h["logits_rows"][:4].tolist() == [0, 1, 2, 3]
 
 
+def test_padding_a_step_with_portions_up_to_given_counts():
+    """Made-up requests bring a step to the counts of a captured graph: one token each, the last one the rest; they
+    write nothing (slot -1), hold page 0 everywhere and the spare state slot; made-up logits rows point at the first
+    made-up token. What the real requests brought stays as it was."""
+    import pytest
+    s, b = setup(1000)
+    s.cache.admit("x")
+    s.cache.admit("y")
+    assert s.cache.allocate("x", 0, 13) and s.cache.allocate("y", 0, 1)
+    b.fill([Entry("x", list(range(100, 113)), 0, [12]), Entry("y", [7], 0, [])], s.cache)
+    before = {k: b.h[k].copy() for k in ("input_ids", "positions", "slot_mapping0", "block_table0")}
+    assert (b.num_tokens, b.num_reqs, b.num_rows, b.max_q_len, b.num_singles) == (14, 2, 1, 13, 1)
+    b.pad(4, 32, 4)
+    h = b.h
+    assert (b.num_tokens, b.num_reqs, b.num_rows, b.max_q_len, b.num_singles) == (32, 4, 4, 17, 2)
+    assert b.q_lens == [13, 1, 1, 17] and h["cu_seqlens"][:5].tolist() == [0, 13, 14, 15, 32]
+    assert h["seq_lens"][:4].tolist() == [13, 1, 1, 17] and h["state_slots"][2:4].tolist() == [8, 8]
+    assert h["positions"][14:32].tolist() == [0] + list(range(17)) and (h["slot_mapping0"][14:32] == -1).all()
+    assert h["block_table0"][2:4].tolist() == [[0] * 4] * 2 and h["logits_rows"][:4].tolist() == [12, 14, 14, 14]
+    assert (h["feedback_src"][14:32] == -1).all()
+    for k, v in before.items():
+        assert (b.h[k][:14] == v[:14]).all() if k != "block_table0" else (b.h[k][:2] == v[:2]).all()
+    b.pad(4, 32, 4)                                        # nothing to add: nothing changes
+    assert (b.num_tokens, b.num_reqs, b.num_rows) == (32, 4, 4)
+    for reqs, tokens, rows, needle in ((3, 32, 4, "never cut"), (4, 33, 4, "need a request"), (6, 33, 4, "at least one token"),
+                                       (9, 64, 4, "never cut"), (4, 32, 9, "never cut")):
+        with pytest.raises(ValueError, match=needle):
+            b.pad(reqs, tokens, rows)
+    b.fill([Entry("x", list(range(100, 113)), 0, [])], s.cache)   # a step that wants no logits pads none
+    b.pad(2, 32, 0)
+    assert (b.num_tokens, b.num_reqs, b.num_rows) == (32, 2, 0) and b.q_lens == [13, 19]
+
+
 def test_limits_are_refused():
     import pytest
     s, b = setup(1000)

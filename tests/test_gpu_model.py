@@ -341,3 +341,56 @@ def test_decode_graph_replays_equal_eager(model_dirs, dtype):
     for k in eager:
         # same kernels; only the split of the keys differs (the graph splits for the longest possible request)
         torch.testing.assert_close(replayed[k], eager[k], rtol=1e-3, atol=1e-3, msg=lambda m: f"{k}: {m}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_steps_with_portions_replayed_from_graphs(model_dirs, name, dtype):
+    """A serving schedule: one request at a time brings its prompt in portions of 16 while up to four others decode,
+    each wanting one row at most. Steps whose counts (tokens, requests, longest portion) come up again are padded with
+    made-up requests and replayed from a graph captured the second time. Every wanted row against the plain model, and
+    against the same schedule run eagerly without padding: in 32-bit bit for bit (a row's arithmetic is its own), in
+    bfloat16 closely (a padded step of 17 to 32 rows does not take the norms along in its products where the unpadded
+    step of up to 16 rows does)."""
+    rng = random.Random(17)
+    ids = "abcdefghij"
+    plen = {k: rng.randrange(20, 75) for k in ids}
+    outs = {k: rng.randrange(6, 14) for k in ids}
+    seqs = {k: tokens_for(name, plen[k] + outs[k], 700 + i) for i, k in enumerate(ids)}
+    want = plain_logits_of(model_dirs, name, seqs)
+    todo, live, fed, steps = list(ids), [], {}, []
+    while todo or live:
+        filling = [k for k in live if fed[k] < plen[k]]
+        if todo and len(live) < 5 and not filling:
+            k = todo.pop(0)
+            live.append(k)
+            fed[k] = 0
+        entries, ends = [], []
+        for k in list(live):
+            n = min(16, plen[k] - fed[k]) if fed[k] < plen[k] else 1
+            last = fed[k] + n >= plen[k]                    # the row after the prompt's last token, then every row
+            entries.append((k, seqs[k][fed[k]:fed[k] + n], [n - 1] if last else []))
+            fed[k] += n
+            if fed[k] == len(seqs[k]):
+                ends.append(k)
+                live.remove(k)
+        steps.append((entries, ends))
+    page = PAGE[name]
+    got = {}
+    for graph in (False, True):
+        r = make_runner(model_dirs[name], name, dtype, max_tokens=64, max_len=128, max_seqs=8, graph=graph,
+                        num_blocks=8 * (-(-128 // page)) + 2)
+        got[graph] = replay(r, steps)
+        assert all(r.cache.num_free(g) == r.num_blocks for g in range(len(r.group_specs)))
+        if graph:
+            assert len(r._portion_graphs) >= 3 and r.portion_replays >= 10, (len(r._portion_graphs), r.portion_replays)
+        else:
+            assert not r._portion_graphs and r.portion_replays == 0
+    compare_rows(got[True], want, dtype, f"{name} portions from graphs")
+    assert got[True].keys() == got[False].keys()
+    for k in got[True]:
+        if dtype == "float32":
+            assert torch.equal(got[True][k], got[False][k]), f"{k}: the replayed step differs from the eager one"
+        else:
+            spread = got[False][k].std()
+            assert float((got[True][k] - got[False][k]).abs().max() / spread) < 0.08, k
