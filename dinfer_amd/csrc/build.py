@@ -32,6 +32,7 @@ SOURCES = {
     "gemm_ref": "gemm_ref.hip",
     "gemm": "gemm.hip",
     "gemm_mid": "gemm_mid.hip",
+    "gemm_wide": "gemm_wide.hip",
     "sampling": "sampling.hip",
     "ceilings": "ceilings.hip",
     "host": "host/api.cpp",

@@ -54,6 +54,7 @@ def row_buckets(most: int) -> list:
         m = b + 1
     return out
 
+WIDE_CUS = 256          # the CUs the rule for csrc/gemm_wide.hip was measured on (MI355X)
 _workspace: dict = {}   # device -> float32 buffer for partial sums
 _outgrown: list = []    # earlier, smaller buffers: graphs captured with them still write there
 
@@ -105,6 +106,16 @@ def matmul_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, may_p
     return _library(a, w, out, m, may_pad)
 
 
+def _wide(m: int, n: int, k: int) -> bool:
+    """33 to 64 rows of a gated product go to the kernel whose waves stage their own activations (csrc/gemm_wide.hip)
+    where its workgroups of 48 columns make one round over the CUs that is at least three quarters full. Measured
+    against the library's product plus the activation kernel, weights taken in turn: 12,288 columns of K = 4,096 (256
+    workgroups) 38.8 against 50.5 us at 33 rows, 40.9 against 48.6 at 48, 46.6 against 48.7 at 64; with a round and a
+    half of workgroups (17,408 columns: 363) it loses, 84 to 105 against 75 to 76 us, and with two it loses too."""
+    groups = -(-n // 48)
+    return SMALL_M < m <= MID_M and WIDE_CUS * 3 // 4 < groups <= WIDE_CUS and ops.gemm_wide_supports(m, n, k)
+
+
 def gated_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, scratch: torch.Tensor, m: int, act: str) -> torch.Tensor:
     """out[:m] = act(a @ wg.T) * (a @ wu.T) for w = [wg; wu] stacked [2N, K]: the two projections of a gated
     feed-forward and its activation, in one weight-streaming kernel at decode sizes (up to 32 rows). scratch
@@ -113,6 +124,8 @@ def gated_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, scratch: torch
         return out
     if a.dtype == torch.bfloat16 and act == "silu" and m <= SMALL_M and w.shape[1] % 8 == 0:
         return ops.gemm_small_m_gated(a, w, out, m)
+    if a.dtype == torch.bfloat16 and act == "silu" and _wide(m, w.shape[0] // 2, w.shape[1]):
+        return ops.gemm_wide(a, w, out, m, gated=True)
     matmul_nt(a, w, scratch, m, may_pad=True)
     ops.gated_act(scratch, out, m, act)
     return out

@@ -57,6 +57,8 @@ SIGNATURES = {
     "dinfer_gemm_mid_m_workspace": ("gemm_mid", [_L, _L, _L, _I, _I, _I, _P]),
     "dinfer_gemm_mid_m_static": ("gemm_mid", [_I, _P, _L, _P, _L, _P, _L, _L, _L, _L, _I, _I, _I, _P]),
     "dinfer_gemm_mid_m_static_init": ("gemm_mid", []),
+    "dinfer_gemm_wide_supports": ("gemm_wide", [_L, _L, _L]),
+    "dinfer_gemm_wide": ("gemm_wide", [_I, _P, _L, _P, _L, _P, _L, _L, _L, _L, _I, _P, _L, _I, _F, _L, _P]),
     "dinfer_stream_read": ("ceilings", [_P, _L, _I, _P, _P]),
     "dinfer_mfma_loop": ("ceilings", [_I, _I, _P, _P, _P]),
     "dinfer_argmax": ("sampling", [_P, _L, _P, _L, _L, _P, _L, _P]),

@@ -401,6 +401,30 @@ def gemm_mid_m(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, work
     return out
 
 
+def gemm_wide_supports(m: int, n: int, k: int) -> bool:
+    """Whether gemm_wide takes a product of m rows with a weight of n rows (gated: n of each half) and k columns."""
+    return bool(lib.get("dinfer_gemm_wide_supports")(m, n, k))
+
+
+def gemm_wide(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, *, gated: bool = False,
+              stats: torch.Tensor | None = None, cols: int = 0, eps: float = 0.0, width: int = 0) -> torch.Tensor:
+    """out[:m] = a[:m] @ w.T for m <= 64 and a weight of many rows (96 of them a workgroup), bf16 operands, out bf16 or
+    float32; gated: w = [wg; wu] stacked [2N, K] and out = silu(a @ wg.T) * (a @ wu.T). stats [m, >= cols] float32:
+    row r of the result is multiplied by rsqrt(sum(stats[r, :cols]) / width + eps) first (a norm carried by the
+    product before this one). K a multiple of 512, N of 16."""
+    _need_gpu(a, w, out, stats)
+    k = w.shape[1]
+    n = w.shape[0] // 2 if gated else w.shape[0]
+    assert a.dtype == w.dtype == torch.bfloat16 and a.shape[1] == k and out.shape[1] == n
+    assert a.shape[0] >= m and out.shape[0] >= m and out.dtype in (torch.bfloat16, torch.float32)
+    if stats is not None:
+        assert stats.dtype == torch.float32 and stats.shape[0] >= m and stats.shape[1] >= cols > 0 and width > 0
+    lib.call("dinfer_gemm_wide", 1 if out.dtype == torch.float32 else 0, a.data_ptr(), _rows(a), w.data_ptr(), _rows(w),
+             out.data_ptr(), _rows(out), m, n, k, 1 if gated else 0, _ptr(stats), _rows(stats) if stats is not None else 0,
+             int(cols), float(eps), int(width), _stream())
+    return out
+
+
 def argmax_scratch(rows: int, vocab: int, device) -> torch.Tensor:
     """The scratch with which argmax spreads each of up to `rows` rows over many workgroups."""
     n = ctypes.c_int64(0)

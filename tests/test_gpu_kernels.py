@@ -1037,14 +1037,47 @@ def test_gemm_mid_m(M):
     assert ran >= 60
 
 
+@pytest.mark.parametrize("M", [1, 17, 33, 48, 49, 64])
+def test_gemm_wide(M):
+    """The product for up to 64 rows whose waves stage their own activations in LDS: plain with bf16 and float output,
+    gated, and as the consumer of a carried norm; a weight whose last workgroup has tiles to spare (N / 16 no multiple
+    of six or three), K of one, two and three steps a wave."""
+    g = torch.Generator().manual_seed(M)
+    for N, K in ((16 * 13, 512), (16 * 31, 1024), (16 * 97, 1536)):
+        a = (torch.randn(M + 3, K, generator=g) * 0.5).to(torch.bfloat16).to(DEV)
+        w = (torch.randn(2 * N, K, generator=g) * 0.1).to(torch.bfloat16).to(DEV)
+        assert ops().gemm_wide_supports(M, N, K) and not ops().gemm_wide_supports(M, N + 8, K)
+        assert not ops().gemm_wide_supports(M, N, K + 64) and not ops().gemm_wide_supports(65, N, K)
+        ad, wd = a[:M].double().cpu(), w.double().cpu()
+        for dtype in (torch.bfloat16, torch.float32):
+            out = torch.full((M + 3, 2 * N), 7.0, dtype=dtype, device=DEV)
+            ops().gemm_wide(a, w, out, M)
+            torch.testing.assert_close(out[:M].double().cpu(), ad @ wd.T, rtol=2e-2, atol=2e-2)
+            assert bool((out[M:] == 7.0).all()), "rows beyond m are left alone"
+        gate, up = ad @ wd[:N].T, ad @ wd[N:].T
+        out = torch.zeros(M, N, dtype=torch.bfloat16, device=DEV)
+        ops().gemm_wide(a, w, out, M, gated=True)
+        torch.testing.assert_close(out.double().cpu(), plain.silu(gate) * up, rtol=2e-2, atol=2e-2)
+        # the consumer of a carried norm: rows scaled by rsqrt(sum of the partial sums / width + eps)
+        stats = torch.rand(M, 11, generator=g).to(DEV) * 40
+        scale = torch.rsqrt(stats[:, :9].double().cpu().sum(-1, keepdim=True) / 300 + 1e-5)
+        ops().gemm_wide(a, w, out, M, gated=True, stats=stats, cols=9, eps=1e-5, width=300)
+        torch.testing.assert_close(out.double().cpu(), plain.silu(gate * scale) * (up * scale), rtol=2e-2, atol=2e-2)
+        plainout = torch.zeros(M, 2 * N, dtype=torch.bfloat16, device=DEV)
+        ops().gemm_wide(a, w, plainout, M, stats=stats, cols=9, eps=1e-5, width=300)
+        torch.testing.assert_close(plainout.double().cpu(), (ad @ wd.T) * scale, rtol=2e-2, atol=2e-2)
+
+
 def test_products_of_17_to_64_rows_by_the_rule_of_sizes():
     """Between the few-row kernel and the library, a weight far wider than high goes to the LDS-resident kernel;
     whichever runs, the product is right, plain and gated, bfloat16 and float32 out, rows past the bucket untouched."""
     from dinfer_amd.kernels import gemm
-    seen = set()
+    seen, wide = set(), set()
     for M in (17, 32, 33, 50, 64):
-        for N, K in ((96, 512), (1000, 1096), (333, 264), (2048, 8192), (1024, 16384)):
+        # (the last: 10,000 gated columns are 209 workgroups of the kernel for wide weights, a round three quarters full)
+        for N, K in ((96, 512), (1000, 1096), (333, 264), (2048, 8192), (1024, 16384), (10000, 512)):
             seen.add(gemm._tall(M, 2 * N, K))
+            wide.add(gemm._wide(M, N, K))
             a = torch.randn(M + 70, K, device=DEV).to(torch.bfloat16)
             w = (torch.randn(2 * N, K, device=DEV) * 0.05).to(torch.bfloat16)
             z = a[:M].double() @ w.double().T
@@ -1061,7 +1094,8 @@ def test_products_of_17_to_64_rows_by_the_rule_of_sizes():
             err = (act[:M].double() - want).abs()
             assert bool((err <= 2e-2 * want.abs() + 2e-3 * want.std()).all()), f"gated {M}x{N}x{K}: {float(err.max())}"
             assert bool((act[M:] == 7.0).all())
-    assert seen == {True, False}          # both sides of the rule were met
+    assert seen == {True, False} and wide == {True, False}          # both sides of each rule were met
+    assert gemm._wide(64, 12288, 4096) and not gemm._wide(64, 17408, 5120) and not gemm._wide(32, 12288, 4096)
 
 
 def test_a_graph_keeps_its_partial_sums_when_the_buffer_grows():
