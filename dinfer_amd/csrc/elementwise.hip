@@ -80,6 +80,19 @@ __global__ void __launch_bounds__(256) widen_kernel(const S* __restrict__ src, f
     dst[i] = to_f32(src[i]);
 }
 
+// x[r][c] = cap * tanh(x[r][c] * scale / cap) (cap <= 0: x * scale), in place, rows of `width` at stride ld
+template <class S>
+__global__ void __launch_bounds__(256) scale_softcap_kernel(S* __restrict__ x, int64_t ld, int64_t width, float scale,
+                                                            float cap) {
+  S* row = x + (int64_t)blockIdx.y * ld;
+  const float inv = cap > 0.f ? 1.f / cap : 0.f;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < width; i += (int64_t)gridDim.x * blockDim.x) {
+    float v = to_f32(row[i]) * scale;
+    if (cap > 0.f) v = cap * tanhf(v * inv);
+    row[i] = from_f32<S>(v);
+  }
+}
+
 // Fills n 32-bit words; used where a captured graph must not hold a memset node.
 __global__ void __launch_bounds__(256) fill_u32_kernel(uint32_t* __restrict__ dst, uint32_t v, int64_t n) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
@@ -132,6 +145,17 @@ extern "C" int dinfer_gated_act(int dtype, int act, const void* in, void* out, i
       return ERR_BAD_DTYPE;
     }
   }
+  return launch_status();
+}
+
+// x[:rows, :width] (row stride ld) *= scale, then softly capped at +-cap (cap * tanh(x / cap); cap <= 0: no cap).
+extern "C" int dinfer_scale_softcap(int dtype, void* x, int64_t ld, int64_t rows, int64_t width, float scale, float cap,
+                                    hipStream_t stream) {
+  if (rows <= 0 || width <= 0) return OK;
+  if (ld < width || rows > 65535) return ERR_BAD_SHAPE;
+  DINFER_DISPATCH_DTYPE(dtype, {
+    scale_softcap_kernel<S><<<dim3(blocks_for(width, 256, 256), (unsigned)rows), 256, 0, stream>>>((S*)x, ld, width, scale, cap);
+  });
   return launch_status();
 }
 

@@ -21,6 +21,7 @@ SIGNATURES = {
     "dinfer_embedding": ("elementwise", [_I, _P, _P, _P, _L, _L, _L, _P, _P, _P]),
     "dinfer_gated_act": ("elementwise", [_I, _I, _P, _P, _L, _L, _L, _P]),
     "dinfer_add_inplace": ("elementwise", [_I, _P, _P, _L, _P]),
+    "dinfer_scale_softcap": ("elementwise", [_I, _P, _L, _L, _L, _F, _F, _P]),
     "dinfer_widen": ("elementwise", [_I, _P, _P, _L, _P]),
     "dinfer_fill_u32": ("elementwise", [_P, c_uint32, _L, _P]),
     "dinfer_rmsnorm": ("norm", [_I, _P, _P, _P, _P, _I, _P, _L, _L, _L, _L, _F, _F, _P]),

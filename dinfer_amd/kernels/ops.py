@@ -103,6 +103,14 @@ def add_inplace(dst: torch.Tensor, src: torch.Tensor, n: int | None = None) -> N
     lib.call("dinfer_add_inplace", dtype_code(dst.dtype), dst.data_ptr(), src.data_ptr(), n, _stream())
 
 
+def scale_softcap(x: torch.Tensor, rows: int, scale: float = 1.0, cap: float | None = None) -> None:
+    """In place on the first `rows` rows of x: x *= scale, then x = cap * tanh(x / cap) where a cap is given."""
+    _need_gpu(x)
+    assert x.shape[0] >= rows
+    lib.call("dinfer_scale_softcap", dtype_code(x.dtype), x.data_ptr(), _rows(x), rows, x.shape[1], float(scale),
+             float(cap) if cap else 0.0, _stream())
+
+
 def widen(src: torch.Tensor, dst: torch.Tensor, n: int | None = None) -> None:
     _need_gpu(src, dst)
     assert dst.dtype == torch.float32 and dst.is_contiguous() and src.is_contiguous()

@@ -1,5 +1,6 @@
-"""A decoder model assembled from a ModelSpec: embedding -> run list of blocks ->
-final norm on the wanted rows -> LM head. Knows no architecture by name.
+"""A decoder model assembled from a ModelSpec: embedding (-> an operation on it, if the spec names one) -> run list
+of blocks -> final norm on the wanted rows -> LM head (-> an operation on the logits, if the spec names one).
+Knows no architecture by name.
 """
 from __future__ import annotations
 
@@ -8,12 +9,20 @@ import torch
 from ..kernels import gemm, ops
 from .base import BuildContext, Carried
 from .linear import Linear
-from .registry import BLOCKS, NORMS
+from .registry import BLOCKS, NORMS, STREAM_OPS
 from .spec import ModelSpec, RunEntry, TensorSpec
 
 
 def _build_blocks(spec: ModelSpec):
     return [BLOCKS.get(l.block.kind)(hidden=spec.hidden_size, layer=l, **l.block.params) for l in spec.layers]
+
+
+def _stream_ops(spec: ModelSpec) -> list:
+    """[(weight-name prefix, part)] of the operations on the embeddings and on the logits, None where there is none."""
+    made = []
+    for part, width, prefix in ((spec.embed_post, spec.hidden_size, spec.embed_name), (spec.logits_post, spec.vocab_size, spec.head_name)):
+        made.append(None if part is None else (prefix + ".post.", STREAM_OPS.get(part.kind)(width, **part.params)))
+    return made
 
 
 def expected_tensors(spec: ModelSpec, blocks=None) -> tuple[dict[str, TensorSpec], set[str]]:
@@ -26,6 +35,10 @@ def expected_tensors(spec: ModelSpec, blocks=None) -> tuple[dict[str, TensorSpec
     fn = NORMS.get(spec.final_norm.kind)(spec.hidden_size, **spec.final_norm.params)
     for n, s in fn.tensors().items():
         exp[spec.final_norm_name + n] = s
+    for op in _stream_ops(spec):
+        if op is not None:
+            for n, ts in op[1].tensors().items():
+                exp[op[0] + n] = ts
     optional = set()
     if spec.tie_embeddings:
         # A tied checkpoint may still ship the head; it is used when present (model.rs:487-496).
@@ -41,6 +54,7 @@ class DecoderModel:
         self.blocks = _build_blocks(spec)
         self.final_norm = NORMS.get(spec.final_norm.kind)(spec.hidden_size, **spec.final_norm.params)
         self.head = Linear(spec.hidden_size, spec.vocab_size)
+        self.embed_post, self.logits_post = _stream_ops(spec)
         self.embed: torch.Tensor | None = None
         self.run = [RunEntry(e.layer, i if e.cache is None else e.cache) for i, e in enumerate(spec.run)]
         for i, e in enumerate(self.run):
@@ -80,6 +94,9 @@ class DecoderModel:
             self.head.set_weight(self.embed)  # one buffer for both
         else:
             raise ValueError(f"no {s.head_name} in the weights and tie_word_embeddings is false")
+        for op in (self.embed_post, self.logits_post):
+            if op is not None:
+                op[1].load(lambda n, _p=op[0], **kw: get(_p + n, **kw))
 
     # ---- cache needs ---------------------------------------------------------------------------
     def cache_needs(self) -> list:
@@ -91,7 +108,9 @@ class DecoderModel:
 
     def capturable(self) -> bool:
         """Whether a step of single rows may be captured once and replayed for other requests."""
-        return all(self.blocks[e.layer].capturable for e in self.run) and self.final_norm.capturable
+        ops_ = [op[1] for op in (self.embed_post, self.logits_post) if op is not None]
+        return (all(self.blocks[e.layer].capturable for e in self.run) and self.final_norm.capturable
+                and all(o.capturable for o in ops_))
 
     def capturable_portions(self) -> bool:
         """The same for steps with prompt portions (Mixer.capturable_portions)."""
@@ -103,6 +122,9 @@ class DecoderModel:
         self.ctx = ctx
         for b in self.blocks:
             b.bind(ctx)
+        for op in (self.embed_post, self.logits_post):
+            if op is not None:
+                op[1].bind(ctx)
         ws = ctx.workspace
         self.hidden = ws.buffer("hidden", self.spec.hidden_size)
         self.final_normed = ws.buffer("final_normed", self.spec.hidden_size, rows=ctx.max_rows)
@@ -114,6 +136,8 @@ class DecoderModel:
         T, R = batch.num_tokens, batch.num_rows
         ops.embedding(batch.input_ids[:T], self.embed, self.hidden, getattr(batch, "feedback_src", None),
                       getattr(batch, "last_tokens", None))
+        if self.embed_post is not None:
+            self.embed_post[1].forward(self.hidden, T)
         pending = None
         for i, e in enumerate(self.run):
             # the input norm of the block that runs next, if that block lets the one before carry it
@@ -131,4 +155,6 @@ class DecoderModel:
             # the last add happens on the wanted rows only, inside the norm kernel
             self.final_norm.forward(pending, self.final_normed, R, residual=self.hidden, rows=batch.logits_rows)
         gemm.matmul_nt(self.final_normed, self.head.weight, self.logits, R, may_pad=True)  # both are buffers of max_rows rows
+        if self.logits_post is not None:
+            self.logits_post[1].forward(self.logits, R)
         return self.logits[:R]

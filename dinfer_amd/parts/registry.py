@@ -2,7 +2,8 @@
 
 One registry per kind of part. A model is assembled only through these, so a
 new mixer, feed-forward, norm, position encoding or block arrangement becomes
-usable by registering a class; no file of the framework changes.
+usable by registering a class; no file of the framework changes. STREAM_OPS holds what a
+model may do to its embeddings before the first layer or to its logits after the head.
 """
 from __future__ import annotations
 
@@ -42,3 +43,4 @@ FEED_FORWARDS = Registry("feed-forward")
 NORMS = Registry("norm")
 POSITION_ENCODINGS = Registry("position encoding")
 BLOCKS = Registry("block arrangement")
+STREAM_OPS = Registry("stream operation")

@@ -166,3 +166,7 @@ class ModelSpec:
     head_name: str
     tie_embeddings: bool
     eos_token_ids: tuple = ()
+    # optional, each a PartSpec of STREAM_OPS: applied in place to the embeddings before the first layer (tensors of
+    # its own under embed_name + "post.") and to the logits after the head (under head_name + "post.")
+    embed_post: PartSpec | None = None
+    logits_post: PartSpec | None = None

@@ -1174,6 +1174,20 @@ def test_add_widen_fill(dtype):
     assert not wide.any()
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_scale_and_soft_cap(dtype):
+    x = (torch.randn(5, 333, device=DEV) * 20).to(dtype)
+    for scale, cap in ((0.5, None), (1.0, 30.0), (3.0, 7.5)):
+        got = x.clone()
+        ops().scale_softcap(got, 4, scale, cap)
+        want = x[:4].double() * scale
+        if cap:
+            want = cap * torch.tanh(want / cap)
+        torch.testing.assert_close(got[:4].double(), want, **tol(dtype))
+        assert torch.equal(got[4], x[4]), "rows beyond the count are left alone"
+        assert cap is None or float(got[:4].float().abs().max()) <= cap
+
+
 def test_measured_ceilings_are_plausible():
     """The two kernels that measure what the chip gives a kernel that only reads and one that only multiplies:
     between a fifth of the vendor's figures and the figures themselves."""

@@ -686,3 +686,92 @@ def test_toy_norm_and_block_arrangement(tmp_path):
         unregister_architecture("ToyParallelLM")
         NORMS.unregister("toy_centered")
         BLOCKS.unregister("toy_parallel")
+
+
+# ---- what a model does to its embeddings and to its logits is a matter of its spec -------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_operations_on_the_embeddings_and_the_logits(tmp_path, dtype):
+    """An architecture whose embeddings are multiplied by the root of the width and by a learned vector (a stream
+    operation defined here, with a tensor of its own in the weight file) and whose logits are softly capped (the
+    built-in one): both are named in its spec; DecoderModel is not touched. Whole, in portions, decoding from graphs."""
+    from dataclasses import dataclass as dc
+    from safetensors.torch import load_file
+    from dinfer_amd.config import EngineOptions, ModelConfig, key, register_architecture, unregister_architecture
+    from dinfer_amd.engine.batch import Entry
+    from dinfer_amd.engine.runner import ModelRunner
+    from dinfer_amd.parts import STREAM_OPS, LayerSpec, ModelSpec, Part, RunEntry, TensorSpec, part
+    from dinfer_amd.weights import write_random_model
+
+    class LearnedScale(Part):
+        """x = x * scale * gain, gain a vector of the file."""
+
+        def __init__(self, width, scale):
+            self.width, self.scale = width, scale
+
+        def tensors(self):
+            return {"gain": TensorSpec((self.width,), init="gain")}
+
+        def load(self, get):
+            self.gain = get("gain")
+
+        def forward(self, x, rows):
+            x[:rows] = (x[:rows].float() * self.scale * self.gain.float()).to(x.dtype)
+
+    @dc(frozen=True)
+    class CappedConfig(ModelConfig):
+        vocab_size: int = key(int)
+        hidden_size: int = key(int)
+        layers: int = key(int)
+        cap: float = key(float)
+        ARCHITECTURE = "ToyCappedLM"
+
+    def build_spec(c):
+        norm = part("rmsnorm", eps=1e-6)
+        attn = part("attention", heads=4, kv_heads=2, head_dim=16, position=part("rotary", theta=1e4, max_positions=128),
+                    qk_norm=norm)
+        layers = [LayerSpec(part("prenorm"), attn, part("gated_mlp", intermediate=72), norm, f"model.layers.{i}.")
+                  for i in range(c.layers)]
+        return ModelSpec("ToyCappedLM", c.vocab_size, c.hidden_size, 128, layers, [RunEntry(i) for i in range(c.layers)],
+                         norm, "model.norm.", "model.embed_tokens.weight", "lm_head.weight", tie_embeddings=False,
+                         embed_post=part("toy_learned_scale", scale=c.hidden_size ** 0.5),
+                         logits_post=part("scale_softcap", scale=20.0, softcap=c.cap))
+
+    STREAM_OPS.register("toy_learned_scale", LearnedScale)
+    register_architecture("ToyCappedLM", CappedConfig, build_spec)
+    try:
+        cfg = CappedConfig.from_dict(dict(vocab_size=211, hidden_size=40, layers=2, cap=3.0, architectures=["ToyCappedLM"]))
+        write_random_model(cfg, tmp_path, seed=8, dtype="float32")
+        w = {k: v.double() for k, v in load_file(str(tmp_path / "model.safetensors")).items()}
+        assert "model.embed_tokens.weight.post.gain" in w
+        pcfg = dict(num_attention_heads=4, num_key_value_heads=2, head_dim=16, rms_norm_eps=1e-6, rope_theta=1e4,
+                    num_hidden_layers=2)
+
+        def want(ids):
+            h = plain.embedding(ids, w["model.embed_tokens.weight"]) * 40 ** 0.5 * w["model.embed_tokens.weight.post.gain"]
+            for l in range(2):
+                h = plain.decoder_layer(h, list(range(len(ids))), w, l, pcfg)
+            z = plain.rms_norm(h, w["model.norm.weight"], 1e-6) @ w["lm_head.weight"].T
+            return 3.0 * torch.tanh(20.0 * z / 3.0)
+
+        opt = EngineOptions(dtype=dtype, max_model_len=128, max_num_seqs=2, max_num_batched_tokens=64, block_size=8,
+                            num_blocks=32, max_logits_rows=64, hip_graph=True)
+        r = ModelRunner.from_dir(tmp_path, opt)
+        rng = random.Random(3)
+        ids = [rng.randrange(211) for _ in range(50)]
+        ref = want(ids)
+        assert float(ref.abs().max()) > 2.0 and float(ref.abs().max()) < 3.0, "the cap is felt"
+        got, fed = [], 0
+        for n in (30, 7, 1, 1, 1, 1, 1, 8):
+            assert r.reserve("a", fed, n)
+            rows = list(range(n)) if n > 1 else [0]
+            got.append(r.step([Entry("a", ids[fed:fed + n], fed, rows)]).double().cpu())
+            fed += n
+        got = torch.cat(got)
+        assert r._graphs, "the single rows were replayed from a graph, the operations inside it"
+        if dtype == "float32":
+            torch.testing.assert_close(got, ref, rtol=2e-4, atol=2e-5)
+        else:
+            assert float(((got - ref).abs() / ref.std(-1, keepdim=True)).max()) < 0.08
+    finally:
+        unregister_architecture("ToyCappedLM")
+        STREAM_OPS.unregister("toy_learned_scale")
