@@ -6,12 +6,12 @@
 // (64 rows x K: 512 KB at K = 4,096), and what it loads of A crosses the same path into the CU as the weight it
 // streams. Here A costs that path no registers and no waiting: a workgroup is 8 waves, wave w owns the 64-wide
 // k steps w, w + 8, w + 16, ... and fetches the fragments of A it will need itself, one step ahead, straight into
-// LDS (global_load_lds: 16 bytes a lane, laid down in lane order, which is the order of the MFMA's B operand when
-// lane l asks for A[16 t + l % 16][k + 8 (l / 16) ..]). Nobody else reads them, so the waves never meet while
-// they stream: each is a chain of [fragments of the next step on their way into LDS | 12 weight loads of the next
-// step in flight (6 tiles of 16 rows x 64 k, line-shaped: lane l reads piece l % 8 of row l / 8) | this step's 48
-// MFMAs], and the compiler counts the loads itself (it knows which LDS object a load in flight writes: the two
-// staging buffers are objects of their own). A's fragments are read from LDS once per step and serve all six
+// LDS (a buffer load that writes LDS: 16 bytes a lane, laid down in lane order, which is the order of the MFMA's
+// B operand when lane l asks for A[16 t + l % 16][k + 8 (l / 16) ..]). Nobody else reads them, so the waves never
+// meet while they stream: each is a chain of [fragments of the next step on their way into LDS | 12 weight loads of
+// the next step in flight (6 tiles of 16 rows x 64 k, line-shaped: lane l reads piece l % 8 of row l / 8) | this
+// step's 48 MFMAs]. The wait for the fragments is written out (see fetch_a), the compiler counts the weight loads
+// itself. A's fragments are read from LDS once per step and serve all six
 // weight tiles, so LDS carries a sixth of what a wave-per-tile layout would ask of it.
 //
 // At the end the eight waves' partial sums meet in LDS, two tiles at a time, and are added in wave order (no
@@ -43,6 +43,16 @@ constexpr int STRIP_BYTES = 16 * ROW_BYTES;
 __device__ __forceinline__ void wave_sync() {
   __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
   __builtin_amdgcn_wave_barrier();
+}
+
+// Waits until at most N of the wave's vector memory loads are in flight (s_waitcnt with the other counters left
+// open: vmcnt is bits 3:0 and 15:14 of the operand, expcnt 6:4, lgkmcnt 11:8); nothing is scheduled across it.
+template <int N>
+__device__ __forceinline__ void wait_for_loads() {
+  static_assert(N >= 0 && N < 64, "vmcnt has six bits");
+  __builtin_amdgcn_sched_barrier(0);
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+  __builtin_amdgcn_sched_barrier(0);
 }
 
 // What the SCALED form needs beside the product's own operands.
@@ -80,26 +90,45 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_wide_kernel(const bf16* __res
     j = j < tiles ? j : tiles - 1;
     return (GATED && r >= 3 ? N : 0) + j * 16;
   };
-  // Addresses are a scalar base (what the wave, the tile and the step decide) plus one 32-bit offset a lane.
-  const uint32_t w_lane = (uint32_t)(lrow * (int)ldw + 8 * lpiece);  // inside a tile: row l / 8 (and + 8), piece l % 8
-  auto weights_at = [&](int r, int k0) { return W + ((int64_t)tile_row(r) * ldw + k0 + wave * 64); };
+  // Addresses are a scalar base (what the wave and the tile decide) plus one 32-bit offset in bytes a lane, to which
+  // the step's k is added inside the loop: so the compiler sees the widening of that sum where the load is and picks
+  // the form of load that takes its base from scalar registers (no lane holds a 64-bit address; hoisted out of the
+  // loop, the widened offsets took a register pair each and the 64-row form spilled inside its loop).
+  const char* const Wb = (const char*)W;
+  const uint32_t w_lane = (uint32_t)(lrow * (int)ldw + 8 * lpiece) * 2u;  // inside a tile: row l / 8, piece l % 8
+  const uint32_t w_half = (uint32_t)(16 * ldw);                            // eight rows further on
+  auto tile_base = [&](int r) { return Wb + ((int64_t)tile_row(r) * ldw + wave * 64) * 2; };
   uint32_t a_lane[MT];  // inside A: row 16 t + l % 16 (past the end: a copy of the last row, dropped), piece l / 16
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     const int m = t * 16 + i16;
-    a_lane[t] = (uint32_t)((m < M ? m : M - 1) * (int)lda + 8 * g4);
+    a_lane[t] = (uint32_t)((m < M ? m : M - 1) * (int)lda + 8 * g4) * 2u;
   }
-  // this wave's fragments of A for the step at k0, on their way into `stage`
+  // This wave's fragments of A for the step at k0, on their way into `stage`. The loads are buffer loads (a
+  // descriptor of A, an offset a lane), not global ones: after a global load into LDS the compiler waits for every
+  // load in flight at the next thing that depends on any of them, which was once a step and drained the wave's queue
+  // of weights each time. A buffer load into LDS it counts among the loads in flight like any other, but it does not
+  // reliably order a later read of that LDS behind it (it looks at the first such load into an object only), so the
+  // wait before the fragments are read is written out in `compute`, and nothing may move across the end of this.
+  const __amdgpu_buffer_rsrc_t a_desc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, (int)(((int64_t)(M - 1) * lda + K) * 2), 0x00020000);
   auto fetch_a = [&](bf16x8 (&stage)[WAVES * 2 * 4][64], int k0) {
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      const bf16* base = A + (k0 + wave * 64 + 32 * h);
 #pragma unroll
       for (int t = 0; t < MT; ++t)
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(base + a_lane[t]),
-                                         (__attribute__((address_space(3))) void*)&stage[(wave * 2 + h) * 4 + t][0],
-                                         16, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(a_desc,
+                                                 (__attribute__((address_space(3))) void*)&stage[(wave * 2 + h) * 4 + t][0],
+                                                 16, (int)a_lane[t], (k0 + wave * 64 + 32 * h) * 2, 0, 0);
     }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // the 16 rows x 64 k of tile r at k0, in the line-shaped order
+  auto fetch_w = [&](bf16x8 (&dst)[2], int r, int k0) {
+    const char* p = tile_base(r);
+    const uint32_t o = w_lane + (uint32_t)(k0 * 2);
+    dst[0] = __builtin_nontemporal_load((const bf16x8*)(p + o));
+    dst[1] = __builtin_nontemporal_load((const bf16x8*)(p + (o + w_half)));
   };
 
   f32x4 acc[RT][MT];
@@ -114,6 +143,10 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_wide_kernel(const bf16* __res
   // for every load in flight wherever it needs one of them)
   bf16x8 w[RT][2];
   auto compute = [&](const bf16x8 (&stage)[WAVES * 2 * 4][64], auto more, int k_next) {
+    // Loads return in the order they were issued. Behind this step's fragments came the 12 weight loads of this step
+    // and, unless this is the last step, the 2 MT fragment loads of the next: when no more than those are in flight,
+    // the fragments are in LDS.
+    wait_for_loads<12 + (decltype(more)::value ? 2 * MT : 0)>();
     bf16x8 af[MT][2];
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
@@ -125,9 +158,7 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_wide_kernel(const bf16* __res
       *(bf16x8*)put = w[r][0];
       *(bf16x8*)(put + 8 * ROW_BYTES) = w[r][1];
       if constexpr (decltype(more)::value) {
-        const bf16* p = weights_at(r, k_next);
-        w[r][0] = __builtin_nontemporal_load((const bf16x8*)(p + w_lane));
-        w[r][1] = __builtin_nontemporal_load((const bf16x8*)(p + 8 * ldw + w_lane));
+        fetch_w(w[r], r, k_next);
       }
       wave_sync();
       const bf16x8 wf0 = *(const bf16x8*)get, wf1 = *(const bf16x8*)(get + 64);
@@ -140,26 +171,31 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_wide_kernel(const bf16* __res
     }
   };
 
-  fetch_a(stage0, 0);
+  // K % CHUNK == 0. Workgroup b starts its walk at step b % steps and wraps round: workgroups that all stood at the
+  // same k would ask the same few memory channels at any moment when a row is a power of two long (measured on
+  // reads alone, 8 KB rows: 5.7 TB/s in step, 6.5 staggered).
+  const int steps = K / CHUNK;
+  const int first = blockIdx.x % steps;
+  auto k_of = [&](int it) {
+    const int s = it + first;
+    return (s < steps ? s : s - steps) * CHUNK;
+  };
+  fetch_a(stage0, k_of(0));
 #pragma unroll
-  for (int r = 0; r < RT; ++r) {
-    const bf16* p = weights_at(r, 0);
-    w[r][0] = __builtin_nontemporal_load((const bf16x8*)(p + w_lane));
-    w[r][1] = __builtin_nontemporal_load((const bf16x8*)(p + 8 * ldw + w_lane));
-  }
-  // K % CHUNK == 0; even steps stage in stage0, odd ones in stage1
+  for (int r = 0; r < RT; ++r) fetch_w(w[r], r, k_of(0));
+  // even steps stage in stage0, odd ones in stage1
   constexpr std::true_type MORE{};
   constexpr std::false_type LAST{};
-  int k0 = 0;
-  for (; k0 + 2 * CHUNK < K; k0 += 2 * CHUNK) {
-    fetch_a(stage1, k0 + CHUNK);
-    compute(stage0, MORE, k0 + CHUNK);
-    fetch_a(stage0, k0 + 2 * CHUNK);
-    compute(stage1, MORE, k0 + 2 * CHUNK);
+  int it = 0;
+  for (; it + 2 < steps; it += 2) {
+    fetch_a(stage1, k_of(it + 1));
+    compute(stage0, MORE, k_of(it + 1));
+    fetch_a(stage0, k_of(it + 2));
+    compute(stage1, MORE, k_of(it + 2));
   }
-  if (k0 + CHUNK < K) {
-    fetch_a(stage1, k0 + CHUNK);
-    compute(stage0, MORE, k0 + CHUNK);
+  if (it + 1 < steps) {
+    fetch_a(stage1, k_of(it + 1));
+    compute(stage0, MORE, k_of(it + 1));
     compute(stage1, LAST, 0);
   } else {
     compute(stage0, LAST, 0);
@@ -237,7 +273,7 @@ int launch(const bf16* A, int64_t lda, const bf16* W, int64_t ldw, O* C, int64_t
 
 // 1 if dinfer_gemm_wide takes these sizes (the caller uses another product otherwise).
 extern "C" int dinfer_gemm_wide_supports(int64_t M, int64_t N, int64_t K) {
-  return M > 0 && M <= 64 && N > 0 && N % 16 == 0 && K > 0 && K % CHUNK == 0 && N <= 0x7fffffff - 96 && K <= 0x7fffffff;
+  return M > 0 && M <= 64 && N > 0 && N % 16 == 0 && K > 0 && K % CHUNK == 0 && N <= 0x7fffffff - 96 && K <= 1 << 24;
 }
 
 // C[M,N] = A . W^T for up to 64 rows. gated: W is [2N, K] = [gate; up] and C[M,N] = silu(A . gate^T) * (A . up^T).
@@ -248,7 +284,7 @@ extern "C" int dinfer_gemm_wide(int out_f32, const void* A, int64_t lda, const v
                                 int cols, float eps, int64_t width, hipStream_t stream) {
   if (M <= 0 || N <= 0) return OK;
   if (!dinfer_gemm_wide_supports(M, N, K)) return ERR_UNSUPPORTED;
-  if (lda < K || ldw < K || ldc < N || lda % 8 || ldw % 8 || ((uintptr_t)A % 16) || ((uintptr_t)W % 16) ||
+  if (lda < K || ldw < K || ldc < N || lda > 1 << 24 || ldw > 1 << 24 || lda % 8 || ldw % 8 || ((uintptr_t)A % 16) || ((uintptr_t)W % 16) ||
       (gated && out_f32) || (stats && (cols <= 0 || width <= 0 || ld_stats < cols)))
     return ERR_BAD_SHAPE;
   Scale link{stats, ld_stats, cols, eps, width > 0 ? 1.f / (float)width : 0.f};
