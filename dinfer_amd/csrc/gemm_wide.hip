@@ -284,7 +284,7 @@ extern "C" int dinfer_gemm_wide(int out_f32, const void* A, int64_t lda, const v
                                 int cols, float eps, int64_t width, hipStream_t stream) {
   if (M <= 0 || N <= 0) return OK;
   if (!dinfer_gemm_wide_supports(M, N, K)) return ERR_UNSUPPORTED;
-  if (lda < K || ldw < K || ldc < N || lda > 1 << 24 || ldw > 1 << 24 || lda % 8 || ldw % 8 || ((uintptr_t)A % 16) || ((uintptr_t)W % 16) ||
+  if (lda < K || ldw < K || ldc < N || lda > 1 << 23 || ldw > 1 << 24 || lda % 8 || ldw % 8 || ((uintptr_t)A % 16) || ((uintptr_t)W % 16) ||
       (gated && out_f32) || (stats && (cols <= 0 || width <= 0 || ld_stats < cols)))
     return ERR_BAD_SHAPE;
   Scale link{stats, ld_stats, cols, eps, width > 0 ? 1.f / (float)width : 0.f};

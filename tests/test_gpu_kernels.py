@@ -1068,6 +1068,27 @@ def test_gemm_wide(M):
         torch.testing.assert_close(plainout.double().cpu(), (ad @ wd.T) * scale, rtol=2e-2, atol=2e-2)
 
 
+def test_gemm_wide_at_the_size_it_runs_at():
+    """The gate and up projections of the 8B sizes (256 workgroups, eight steps of k a wave, every wave's fragments of the
+    activations landing in LDS one step ahead of their use) at the row counts the rule sends there, on four weights in
+    turn so that the memory system is busy: a fragment read before it has landed would be the fragment of the step
+    before, an error as large as the result."""
+    N, K = 12288, 4096
+    g = torch.Generator().manual_seed(5)
+    ws = [(torch.randn(2 * N, K, generator=g) * 0.03).to(torch.bfloat16).to(DEV) for _ in range(4)]
+    for M in (33, 48, 64):
+        a = torch.randn(64, K, generator=g).to(torch.bfloat16).to(DEV)
+        outs = [torch.zeros(64, N, dtype=torch.bfloat16, device=DEV) for _ in ws]
+        for _ in range(3):
+            for w, out in zip(ws, outs):
+                ops().gemm_wide(a, w, out, M, gated=True)
+        for w, out in zip(ws, outs):
+            z = a[:M].double() @ w.double().T
+            want = plain.silu(z[:, :N]) * z[:, N:]
+            err = (out[:M].double() - want).abs()
+            assert bool((err <= 2e-2 * want.abs() + 2e-3 * want.std()).all()), f"{M} rows: {float(err.max())}"
+
+
 def test_products_of_17_to_64_rows_by_the_rule_of_sizes():
     """Between the few-row kernel and the library, a weight far wider than high goes to the LDS-resident kernel;
     whichever runs, the product is right, plain and gated, bfloat16 and float32 out, rows past the bucket untouched."""
