@@ -106,26 +106,32 @@ def matmul_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, may_p
     return _library(a, w, out, m, may_pad)
 
 
+WIDE_FROM = 17   # up to 16 rows the few-row kernel is level with it (and carries norms)
+
+
 def _wide(m: int, n: int, k: int) -> bool:
-    """33 to 64 rows of a gated product go to the kernel whose waves stage their own activations (csrc/gemm_wide.hip)
+    """17 to 64 rows of a gated product go to the kernel whose waves stage their own activations (csrc/gemm_wide.hip)
     where its workgroups of 48 columns make one round over the CUs that is at least three quarters full. Measured
-    against the library's product plus the activation kernel, weights taken in turn: 12,288 columns of K = 4,096 (256
-    workgroups) 38.8 against 50.5 us at 33 rows, 40.9 against 48.6 at 48, 46.6 against 48.7 at 64; with a round and a
-    half of workgroups (17,408 columns: 363) it loses, 84 to 105 against 75 to 76 us, and with two it loses too."""
+    with weights taken in turn, 12,288 columns of K = 4,096 (256 workgroups): against the few-row kernel 33.9 against
+    35.2 us at 17 rows, 33.9 against 36.6 at 24, 34.8 against 38.7 at 32 (level at 8 and 16); against the library's
+    product plus the activation kernel 37.1 against 51.1 us at 33 rows, 38.0 against 49.5 at 48, 42.6 against 49.6 at
+    64. With a round and a half of workgroups (17,408 columns: 363) it loses to the library, 84 to 105 against 76 us,
+    and with two it loses too."""
     groups = -(-n // 48)
-    return SMALL_M < m <= MID_M and WIDE_CUS * 3 // 4 < groups <= WIDE_CUS and ops.gemm_wide_supports(m, n, k)
+    return WIDE_FROM <= m <= MID_M and WIDE_CUS * 3 // 4 < groups <= WIDE_CUS and ops.gemm_wide_supports(m, n, k)
 
 
 def gated_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, scratch: torch.Tensor, m: int, act: str) -> torch.Tensor:
     """out[:m] = act(a @ wg.T) * (a @ wu.T) for w = [wg; wu] stacked [2N, K]: the two projections of a gated
-    feed-forward and its activation, in one weight-streaming kernel at decode sizes (up to 32 rows). scratch
+    feed-forward and its activation, in one weight-streaming kernel at decode sizes (up to 32 rows, up to 64 where
+    the kernel for wide weights takes it). scratch
     [rows, 2N] takes the projections where the activation is a pass of its own."""
     if m <= 0:
         return out
-    if a.dtype == torch.bfloat16 and act == "silu" and m <= SMALL_M and w.shape[1] % 8 == 0:
-        return ops.gemm_small_m_gated(a, w, out, m)
     if a.dtype == torch.bfloat16 and act == "silu" and _wide(m, w.shape[0] // 2, w.shape[1]):
         return ops.gemm_wide(a, w, out, m, gated=True)
+    if a.dtype == torch.bfloat16 and act == "silu" and m <= SMALL_M and w.shape[1] % 8 == 0:
+        return ops.gemm_small_m_gated(a, w, out, m)
     matmul_nt(a, w, scratch, m, may_pad=True)
     ops.gated_act(scratch, out, m, act)
     return out

@@ -1116,7 +1116,8 @@ def test_products_of_17_to_64_rows_by_the_rule_of_sizes():
             assert bool((err <= 2e-2 * want.abs() + 2e-3 * want.std()).all()), f"gated {M}x{N}x{K}: {float(err.max())}"
             assert bool((act[M:] == 7.0).all())
     assert seen == {True, False} and wide == {True, False}          # both sides of each rule were met
-    assert gemm._wide(64, 12288, 4096) and not gemm._wide(64, 17408, 5120) and not gemm._wide(32, 12288, 4096)
+    assert gemm._wide(64, 12288, 4096) and not gemm._wide(64, 17408, 5120)
+    assert gemm._wide(17, 12288, 4096) and not gemm._wide(16, 12288, 4096)
 
 
 def test_a_graph_keeps_its_partial_sums_when_the_buffer_grows():
