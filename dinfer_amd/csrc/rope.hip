@@ -231,47 +231,26 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_vec_kernel(
   const int64_t t = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int sub = lane / LPH, l = lane % LPH;  // which head of the wave, which 8 dims of it
-  const int item = (blockIdx.y * WAVES + wave) * HPW + sub;
   const int items = H + 2 * Hkv;
-  const bool live = item < items;
-  const bool is_v = live && item >= H + Hkv, is_q = live && item < H, is_k = live && !is_q && !is_v;
+  // The workgroups of a token (gridDim.y of them) take its heads in rounds of gridDim.y * WAVES * HPW; a lane keeps
+  // its 8 dims from round to round, so the angles of those dims are fetched once (with one workgroup a token, which
+  // is how many tokens are launched, a lane serves three heads of the 8B sizes with one fetch: the angles are four
+  // times the bytes of the head's own 8 values).
+  const int per_round = gridDim.y * WAVES * HPW;
+  const int first_item = (blockIdx.y * WAVES + wave) * HPW + sub;
   bf16* row = qkv + t * ld;
   const int64_t slot = slots ? slots[t] : -1;
   const int64_t blk = slot >= 0 ? slot / page : 0;
   const int off = slot >= 0 ? (int)(slot % page) : 0;
   const int d0 = 8 * l;
-  bf16* src = is_q ? row + q_off + (int64_t)item * D
-            : is_k ? row + k_off + (int64_t)(item - H) * D
-                   : row + v_off + (int64_t)(item - H - Hkv) * D;
-  const void* w = is_q ? wq : wk;
-  bf16x8 xv = zero8();
-  if (live) xv = *(const bf16x8*)(src + d0);
-  if (is_v) {
-    if (slot >= 0 && !skip_v) {
-      bf16* vd = v_cache + ((blk * Hkv + (item - H - Hkv)) * (int64_t)D + d0) * page + off;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) vd[(int64_t)e * page] = xv[e];
-    }
-  }
-  const bool qk = is_q || is_k;
-  // gains and angles of this lane's dims: the pair index of dim d is d mod D/2
-  float g[8], c[8], sn[8];
+  auto source = [&](int item) {
+    return item < H ? row + q_off + (int64_t)item * D
+                    : item < H + Hkv ? row + k_off + (int64_t)(item - H) * D : row + v_off + (int64_t)(item - H - Hkv) * D;
+  };
+  // angles of this lane's dims: the pair index of dim d is d mod D/2
+  float c[8], sn[8];
   const int pi = d0 % HALF;
-  if (qk && w) {
-    if (wf32) {
-      const f32x4 a = *(const f32x4*)((const float*)w + d0), b = *(const f32x4*)((const float*)w + d0 + 4);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) { g[e] = a[e] + w_offset; g[4 + e] = b[e] + w_offset; }
-    } else {
-      const bf16x8 gv = *(const bf16x8*)((const bf16*)w + d0);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) g[e] = (float)gv[e] + w_offset;
-    }
-  } else {
-#pragma unroll
-    for (int e = 0; e < 8; ++e) g[e] = 1.f;
-  }
-  if (qk && cos_sin) {
+  if (cos_sin) {
     const float* cs = cos_sin + (int64_t)pos[t] * D;
     const f32x4 c0 = *(const f32x4*)(cs + pi), c1 = *(const f32x4*)(cs + pi + 4);
     const f32x4 s0 = *(const f32x4*)(cs + HALF + pi), s1 = *(const f32x4*)(cs + HALF + pi + 4);
@@ -281,31 +260,69 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_vec_kernel(
 #pragma unroll
     for (int e = 0; e < 8; ++e) { c[e] = 1.f; sn[e] = 0.f; }
   }
-  float x[8], ss = 0.f;
+  // (a wave's lanes leave the loop together: the cross-lane steps below need all of them)
+  const int wave_first = (blockIdx.y * WAVES + wave) * HPW;
+  bf16x8 xv = zero8();
+  if (first_item < items) xv = *(const bf16x8*)(source(first_item) + d0);
+  for (int base = 0; wave_first + base < items; base += per_round) {
+    const int item = first_item + base;
+    const bool live = item < items;
+    const bool is_v = live && item >= H + Hkv, is_q = live && item < H, is_k = live && !is_q && !is_v;
+    bf16* src = live ? source(item) : row;
+    const bf16x8 xc = xv;
+    // the next round's values are on their way while this round is computed
+    xv = zero8();
+    if (item + per_round < items) xv = *(const bf16x8*)(source(item + per_round) + d0);
+    if (is_v) {
+      if (slot >= 0 && !skip_v) {
+        bf16* vd = v_cache + ((blk * Hkv + (item - H - Hkv)) * (int64_t)D + d0) * page + off;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    x[e] = (float)xv[e];
-    ss = add_square(ss, x[e]);
-  }
-  // every lane takes part in the cross-lane steps, whatever its head is
+        for (int e = 0; e < 8; ++e) vd[(int64_t)e * page] = xc[e];
+      }
+    }
+    const bool qk = is_q || is_k;
+    const void* w = is_q ? wq : wk;
+    float g[8];
+    if (qk && w) {
+      if (wf32) {
+        const f32x4 a = *(const f32x4*)((const float*)w + d0), b = *(const f32x4*)((const float*)w + d0 + 4);
 #pragma unroll
-  for (int o = LPH / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
-  const float inv = (qk && w) ? 1.f / sqrtf(ss / (float)D + eps) : 1.f;
-  float y[8], other[8];
+        for (int e = 0; e < 4; ++e) { g[e] = a[e] + w_offset; g[4 + e] = b[e] + w_offset; }
+      } else {
+        const bf16x8 gv = *(const bf16x8*)((const bf16*)w + d0);
 #pragma unroll
-  for (int e = 0; e < 8; ++e) y[e] = (qk && w) ? x[e] * inv * g[e] : x[e];
+        for (int e = 0; e < 8; ++e) g[e] = (float)gv[e] + w_offset;
+      }
+    } else {
 #pragma unroll
-  for (int e = 0; e < 8; ++e) other[e] = __shfl_xor(y[e], LPH / 2, 64);
-  if (!qk) return;
-  const bool first = l < LPH / 2;  // this lane holds the first elements of its pairs
-  bf16x8 r;
+      for (int e = 0; e < 8; ++e) g[e] = 1.f;
+    }
+    float x[8], ss = 0.f;
 #pragma unroll
-  for (int e = 0; e < 8; ++e)
-    r[e] = (bf16)(first ? rotated_first(y[e], other[e], c[e], sn[e]) : rotated_second(other[e], y[e], c[e], sn[e]));
-  if (is_q || !slots) {
-    *(bf16x8*)(src + d0) = r;
-  } else if (slot >= 0) {
-    *(bf16x8*)(k_cache + (blk * Hkv + (item - H)) * (int64_t)page * D + k_page_offset((int)off, d0, page)) = r;
+    for (int e = 0; e < 8; ++e) {
+      x[e] = (float)xc[e];
+      ss = add_square(ss, x[e]);
+    }
+    // every lane takes part in the cross-lane steps, whatever its head is
+#pragma unroll
+    for (int o = LPH / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+    const float inv = (qk && w) ? 1.f / sqrtf(ss / (float)D + eps) : 1.f;
+    float y[8], other[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) y[e] = (qk && w) ? x[e] * inv * g[e] : x[e];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) other[e] = __shfl_xor(y[e], LPH / 2, 64);
+    if (!qk) continue;
+    const bool first = l < LPH / 2;  // this lane holds the first elements of its pairs
+    bf16x8 r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      r[e] = (bf16)(first ? rotated_first(y[e], other[e], c[e], sn[e]) : rotated_second(other[e], y[e], c[e], sn[e]));
+    if (is_q || !slots) {
+      *(bf16x8*)(src + d0) = r;
+    } else if (slot >= 0) {
+      *(bf16x8*)(k_cache + (blk * Hkv + (item - H)) * (int64_t)page * D + k_page_offset((int)off, d0, page)) = r;
+    }
   }
 }
 
@@ -380,7 +397,8 @@ extern "C" int dinfer_qkv_post(int dtype, void* qkv, int64_t tokens, int64_t ld,
                       ((uintptr_t)k_cache % 16) == 0;
   if (whole_head_neox && vec_ok) {
     const int lph = head_dim / 8, hpw = 64 / lph;
-    const dim3 vgrid((unsigned)tokens, (unsigned)((items + WAVES * hpw - 1) / (WAVES * hpw)));
+    // many tokens fill the chip with one workgroup each; few tokens spread their heads over several
+    const dim3 vgrid((unsigned)tokens, tokens >= 512 ? 1u : (unsigned)((items + WAVES * hpw - 1) / (WAVES * hpw)));
     // many tokens: V goes to its transposed pages through the gathering kernel (16-byte stores)
     const int skip_v = (slot_mapping && token_runs && tokens >= 64 && page_size % 8 == 0 && ((uintptr_t)v_cache % 16) == 0) ? 1 : 0;
     if (skip_v)
