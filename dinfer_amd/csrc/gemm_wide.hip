@@ -1,5 +1,5 @@
 // C[M,N] = A[M,K] . W[N,K]^T for 17 to 64 rows and a weight of many rows (the gate and up projections of a
-// feed-forward, the LM head), bf16 operands, float accumulation: the products of a decode step of 33 to 64
+// feed-forward, the LM head), bf16 operands, float accumulation: the products of a decode step of 17 to 64
 // requests whose weight is so tall that 96 of its rows a workgroup still make a workgroup for every CU.
 //
 // At these row counts a weight-streaming kernel's trouble is the activations: every workgroup needs all of A

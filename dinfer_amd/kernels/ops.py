@@ -394,7 +394,7 @@ def gemm_mid_m_workspace(m: int, n: int, k: int, *, gated: bool = False, ks: int
 
 def gemm_mid_m(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, workspace: torch.Tensor | None = None, *,
                gated: bool = False, ks: int = 0, rt: int = 0) -> torch.Tensor:
-    """out[:m] = a[:m] @ w.T for m <= 64 (made for 33 to 64), bf16 operands; gated: w = [wg; wu] stacked
+    """out[:m] = a[:m] @ w.T for m <= 64 (made for 17 to 64), bf16 operands; gated: w = [wg; wu] stacked
     [2N, K] and out = silu(a @ wg.T) * (a @ wu.T). A narrow weight is cut into slices of k whose float
     partial sums go through `workspace` and are added in slice order by a second kernel."""
     _need_gpu(a, w, out, workspace)
