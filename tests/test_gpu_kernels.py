@@ -1089,6 +1089,37 @@ def test_gemm_wide_at_the_size_it_runs_at():
             assert bool((err <= 2e-2 * want.abs() + 2e-3 * want.std()).all()), f"{M} rows: {float(err.max())}"
 
 
+def test_gemm_wide_random_sizes_and_pitches():
+    """Sixty products of random sizes (1 to 64 rows, N a multiple of 16 up to 6,400, K of 1 to 12 steps), operands and
+    result with row pitches beyond their widths, plain, gated and as the consumer of a carried norm, bfloat16 and float
+    out: the result against float64, and nothing written beside it."""
+    import random
+    rng = random.Random(11)
+    for it in range(60):
+        M, N, K = rng.randint(1, 64), 16 * rng.randint(1, 400), 512 * rng.randint(1, 12)
+        pad_a, pad_w, pad_c = rng.choice([0, 8, 64]), rng.choice([0, 8, 128]), rng.choice([0, 4, 32])
+        gated, scaled = rng.random() < 0.5, rng.random() < 0.4
+        f32 = not gated and rng.random() < 0.3
+        g = torch.Generator().manual_seed(it)
+        a = (torch.randn(M + 2, K + pad_a, generator=g) * 0.5).to(torch.bfloat16).to(DEV)[:, :K]
+        w = (torch.randn(2 * N if gated else N, K + pad_w, generator=g) * 0.1).to(torch.bfloat16).to(DEV)[:, :K]
+        whole = torch.full((M + 2, N + pad_c), 7.0, dtype=torch.float32 if f32 else torch.bfloat16, device=DEV)
+        out, kw = whole[:, :N], {}
+        scale = torch.ones(M, 1, dtype=torch.float64, device=DEV)
+        if scaled:
+            cols, width = rng.randint(1, 40), rng.randint(100, 5000)
+            stats = (torch.rand(M, cols + 3, generator=g) * 50).to(DEV)
+            kw = dict(stats=stats, cols=cols, eps=1e-5, width=width)
+            scale = torch.rsqrt(stats[:, :cols].double().sum(-1, keepdim=True) / width + 1e-5)
+        ops().gemm_wide(a, w, out, M, gated=gated, **kw)
+        z = (a[:M].double() @ w.double().T) * scale
+        want = plain.silu(z[:, :N]) * z[:, N:] if gated else z
+        err = (out[:M].double() - want).abs()
+        tol = 1e-4 * want.abs() + 1e-3 * want.std() if f32 else 2e-2 * want.abs() + 2e-3 * want.std() + 1e-6
+        assert bool((err <= tol).all()), f"case {it}: {M}x{N}x{K} gated {gated} scaled {scaled}: {float(err.max())}"
+        assert bool((whole[M:] == 7.0).all()) and bool((whole[:, N:] == 7.0).all()), f"case {it}: wrote beside the result"
+
+
 def test_products_of_17_to_64_rows_by_the_rule_of_sizes():
     """Between the few-row kernel and the library, a weight far wider than high goes to the LDS-resident kernel;
     whichever runs, the product is right, plain and gated, bfloat16 and float32 out, rows past the bucket untouched."""
