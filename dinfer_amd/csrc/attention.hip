@@ -297,7 +297,8 @@ struct Tile {
   // per block); otherwise every block runs the masking body.
   // A block's loads are issued right before its use and other waves hide the latency: reading a
   // block ahead was measured and does not pay (neither with a second set of registers nor by
-  // refilling each fragment as soon as its last reader has issued).
+  // refilling each fragment as soon as its last reader has issued; the split-K kernel with a second set at 8 to 64
+  // requests of 2k and 4k keys, one wave a SIMD: within 1 % either way, 5.6 to 5.9 TB/s with it and without).
   // fence_last: the wave has stored the key and value at k_hi - 1 itself (other lanes than those that read them);
   // before the last block is loaded, those stores are waited for.
   template <bool TWO_BODIES, class MaskFn>
