@@ -562,8 +562,8 @@ def measured_hbm_read(device, nbytes: int = 4 << 30, repeats: int = 3) -> float:
     the best of `repeats` runs."""
     buf = torch.empty(nbytes // 4, dtype=torch.float32, device=device)
     buf.zero_()
-    blocks = 256 * 8
-    out = torch.empty(blocks * 4, dtype=torch.float32, device=device)
+    blocks = 256
+    out = torch.empty(blocks * 8, dtype=torch.float32, device=device)
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     best = float("inf")
     for _ in range(repeats + 1):      # the first run loads the kernel
