@@ -33,6 +33,8 @@
 //
 // Reference behaviour: crates/kernels/cuda/gemm_small_m.cu:42-114,148-285
 // (weight read once, split-K, M <= 32).
+#include <type_traits>
+
 #include "common.cuh"
 
 using namespace dinfer;
@@ -102,8 +104,14 @@ struct NormLink {
 // silu(gate) * up into C [M, N]: the activation costs no pass of its own.
 // CUT (not GATED): the last 8 rows of the workgroup's last tile are left out, so a workgroup takes
 // 16 RT - 8 weight rows: with two tiles 24 rows, which makes 256 workgroups of N = 6,144 where 32 rows make 192.
+// The waves a SIMD that a form is to keep room for (its registers are held to that): the form of one token tile and
+// two row tiles that is no producer of a carried norm (the gate/up pair, q/k/v, the LM head) runs with workgroups of
+// 4 or 8 waves, six workgroups of 4 on a CU, and loses a tenth of its rate at five (measured when two more registers
+// cost it the sixth). The other forms take what they need.
+constexpr int waves_a_simd(int mt, int rt, int mode, bool cut) { return mt == 1 && rt == 2 && mode != SINK && !cut ? 6 : 1; }
+
 template <int MT, int RT, class O, bool GATED, bool STREAM, int MODE = PLAIN, bool CUT = false>
-__global__ void __launch_bounds__(1024) gemm_small_m_kernel(const bf16* __restrict__ A, int64_t lda,
+__global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(waves_a_simd(MT, RT, MODE, CUT), 8))) gemm_small_m_kernel(const bf16* __restrict__ A, int64_t lda,
                                                             const bf16* __restrict__ W, int64_t ldw,
                                                             O* __restrict__ C, int64_t ldc, int M, int N, int K,
                                                             NormLink link = NormLink{}) {
@@ -176,21 +184,39 @@ __global__ void __launch_bounds__(1024) gemm_small_m_kernel(const bf16* __restri
   const int per_wave = (steps + nw - 1) / nw;
   const int s_begin = wave * per_wave;
   const int s_end = s_begin + per_wave < steps ? s_begin + per_wave : steps;
-  for (int s0 = s_begin; s0 < s_end; s0 += UNROLL) {
+  // One round: the loads of UNROLL steps, then their MFMAs. `masked` is a type: the rounds that lie wholly inside the
+  // wave's run and inside k load without a condition, so that the compiler issues them in one go and lets the first
+  // MFMAs start when the first loads are back (under a condition every load is a branch of its own, and the first use
+  // of any waits for all of them: measured 0.3 to 1.3 us a product at the 8B sizes); the last round of a run that
+  // does not divide evenly asks. (Rows of A past M are then copies of row 0, computed and dropped like weight rows
+  // past N.)
+  auto round = [&](int s0, auto masked) {
+    constexpr bool MASKED = decltype(masked)::value;
     bf16x8 wraw[UNROLL][RT][2], araw[UNROLL][MT][2];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
       const int kk = (s0 + u) * 64;
-      const bool ok = kk + 8 * lpiece < K && (s0 + u) < s_end;
+      const bool ok = !MASKED || (kk + 8 * lpiece < K && (s0 + u) < s_end);
 #pragma unroll
       for (int r = 0; r < RT; ++r)
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
-          wraw[u][r][h] = (CUT && r == RT - 1 && h == 1) ? zero8() : (ok ? ld_weight<STREAM>(wp[r][h] + kk) : zero8());
+        for (int h = 0; h < 2; ++h) {
+          if (CUT && r == RT - 1 && h == 1)
+            wraw[u][r][h] = zero8();
+          else if constexpr (MASKED)
+            wraw[u][r][h] = ok ? ld_weight<STREAM>(wp[r][h] + kk) : zero8();
+          else
+            wraw[u][r][h] = ld_weight<STREAM>(wp[r][h] + kk);
+        }
 #pragma unroll
       for (int t = 0; t < MT; ++t)
 #pragma unroll
-        for (int h = 0; h < 2; ++h) araw[u][t][h] = (ok && arow[t][h]) ? *(const bf16x8*)(ap[t][h] + kk) : zero8();
+        for (int h = 0; h < 2; ++h) {
+          if constexpr (MASKED)
+            araw[u][t][h] = (ok && arow[t][h]) ? *(const bf16x8*)(ap[t][h] + kk) : zero8();
+          else
+            araw[u][t][h] = *(const bf16x8*)(ap[t][h] + kk);
+        }
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
@@ -219,7 +245,13 @@ __global__ void __launch_bounds__(1024) gemm_small_m_kernel(const bf16* __restri
         }
       }
     }
-  }
+  };
+  // whole steps of k end at K / 64; the rounds before `plain_end` touch nothing else
+  const int whole = K / 64 < s_end ? K / 64 : s_end;
+  const int plain_end = whole > s_begin ? s_begin + (whole - s_begin) / UNROLL * UNROLL : s_begin;
+  int s0 = s_begin;
+  for (; s0 < plain_end; s0 += UNROLL) round(s0, std::false_type{});
+  for (; s0 < s_end; s0 += UNROLL) round(s0, std::true_type{});
   // SCALED: every token's 1 / rms from the producer's partial sums, added in a fixed order; kept behind the
   // strips and the sums (the launch sizes LDS for it)
   float* rs = (float*)(smem + lds_core_bytes(nw, RT, MT));
