@@ -299,15 +299,15 @@ struct Tile {
   // block ahead was measured and does not pay (neither with a second set of registers nor by
   // refilling each fragment as soon as its last reader has issued; the split-K kernel with a second set at 8 to 64
   // requests of 2k and 4k keys, one wave a SIMD: within 1 % either way, 5.6 to 5.9 TB/s with it and without).
-  // fence_last: the wave has stored the key and value at k_hi - 1 itself (other lanes than those that read them);
-  // before the last block is loaded, those stores are waited for.
-  template <bool TWO_BODIES, class MaskFn>
+  // hook(kb, last): called before block kb's loads are issued; `last` says that kb is the wave's last block. The wave
+  // that brings the row's own key issues that key's loads a block early there and stores it before the last block.
+  template <bool TWO_BODIES, class MaskFn, class Hook>
   __device__ __forceinline__ void walk(const bf16x8 (&qf)[NT][KS], const int (&col_lo)[NT], const int (&col_hi)[NT],
-                                       MaskFn mask, bool fence_last = false) {
+                                       MaskFn mask, Hook hook) {
     Frags<DT> f;
 #pragma nounroll
     for (int kb = k_lo & ~31; kb < k_hi; kb += 32) {
-      if (fence_last && kb + 32 >= k_hi) __threadfence_block();
+      hook(kb, kb + 32 >= k_hi);
       if (!TWO_BODIES || mask(kb)) {
         load<true>(f, kb);
         compute<true>(f, qf, kb, col_lo, col_hi);
@@ -316,6 +316,11 @@ struct Tile {
         compute<false>(f, qf, kb, col_lo, col_hi);
       }
     }
+  }
+  template <bool TWO_BODIES, class MaskFn>
+  __device__ __forceinline__ void walk(const bf16x8 (&qf)[NT][KS], const int (&col_lo)[NT], const int (&col_hi)[NT],
+                                       MaskFn mask) {
+    walk<TWO_BODIES>(qf, col_lo, col_hi, mask, [](int, bool) {});
   }
 
   // total of l over the four lane groups of a column
@@ -593,6 +598,8 @@ attn_decode_kernel(
   bf16x8 qf[1][KS];
   Tile<DT, 1, P2, STREAM> tl;
   bool writer = false;
+  int w_pos = 0;
+  int64_t w_slot = -1;
   if constexpr (POST) {
     // in the order of what is known when: the head, its gains, the row's position and slot at once; ...
     HeadPost<DT> qh;
@@ -614,12 +621,14 @@ attn_decode_kernel(
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) qf[0][ks] = zero8();
     }
-    if (writer) {
+    w_pos = pos_row;
+    w_slot = slot;
+    if (!STREAM && writer) {
+      // few requests, short parts: the new key and value are dealt with here, at once (the loads are asked for only now,
+      // when the registers of q's head are free); see below for the launches of many requests
       const int64_t blk = slot / ps;
       const int off = (int)(slot - blk * ps);
       const int64_t head = (blk * Hkv + hk) * (int64_t)ps * D;
-      // (asked for only now, when the registers of q's head are free: this part is on average half as long as the
-      // others, so its wave has the time)
       HeadPost<DT> kh;
       bf16x8 vv;
       kh.load(post.k_new + (int64_t)row * ld_q + (int64_t)hk * D, i16 == 0);
@@ -652,7 +661,62 @@ attn_decode_kernel(
   }
   const int col_lo[1] = {k_lo}, col_hi[1] = {k_hi};
   // (reading the first block before q is normed, or two blocks ahead, was measured at 1 and 8 requests: no gain)
-  tl.template walk<false>(qf, col_lo, col_hi, [&](int kb) { return kb < k_lo || kb + 32 > k_hi; }, writer);
+  const auto partial = [&](int kb) { return kb < k_lo || kb + 32 > k_hi; };
+  if constexpr (POST && !STREAM) {
+    // the key was stored in the prologue; the fence lets the wave's own loads of its last block see it
+    tl.template walk<false>(qf, col_lo, col_hi, partial, [&](int, bool last) {
+      if (writer && last) __threadfence_block();
+    });
+  } else if constexpr (POST) {
+    // Many requests (parts of dozens of blocks, every workgroup waiting for the wave that writes):
+    // The wave whose part ends with the row's own position brings the new key and value: their loads (the head, the
+    // value) go out three blocks before the end, a block later the key is normed (gains and angles asked for there:
+    // kept through a block they would cost the walk a hundred registers), rotated and stored with the value, and
+    // before the last block a fence lets the wave's own loads of that block see them: the latencies lie under the
+    // blocks' work instead of on the path of the wave that ends its workgroup (64 requests of 2,064 keys: 96.9 ->
+    // 92.3 us, of 4,080 keys 181 -> 174.5; at 8 requests, where a part is five blocks, the larger kernel loses 1.5 us,
+    // hence the two forms). A part of fewer blocks does the steps as early as it can.
+    HeadPost<DT> kh;   // only its head is kept from one block to the next: the gains and angles are asked for where
+    bf16x8 vv;         // they are used (they come from L2), or the walk would hold a hundred registers for them
+    bool fetched = false;
+    const auto fetch_key = [&]() {
+      kh.load(post.k_new + (int64_t)row * ld_q + (int64_t)hk * D, i16 == 0);
+      if (lane < D / 8) vv = *(const bf16x8*)(post.v_new + (int64_t)row * ld_q + (int64_t)hk * D + lane * 8);
+      fetched = true;
+    };
+    const auto store_key = [&]() {
+      const int64_t blk = w_slot / ps;
+      const int off = (int)(w_slot - blk * ps);
+      const int64_t head = (blk * Hkv + hk) * (int64_t)ps * D;
+      typename HeadPost<DT>::Angles kang;
+      if (post.wk) kh.load_gains(post.wk);
+      if (post.cos_sin) kang.load(post.cos_sin + (int64_t)w_pos * D);
+      bf16x8 kr[KS];
+      kh.finish(kang, post.wk != nullptr, post.eps, post.w_offset, post.cos_sin != nullptr, kr);
+      if (i16 == 0) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+          *(bf16x8*)(post.k_cache + head + k_page_offset(off, ks * 32 + g4 * 8, ps)) = kr[ks];
+      }
+      if (lane < D / 8) {  // V pages are transposed: the 8 dims of a piece go to 8 rows of keys
+        bf16* vd = post.v_cache + head + (int64_t)(lane * 8) * ps + off;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) vd[(int64_t)e * ps] = vv[e];
+      }
+    };
+    bool stored = false;
+    tl.template walk<false>(qf, col_lo, col_hi, partial, [&](int kb, bool last) {
+      if (!writer) return;
+      if (fetched && !stored) store_key(), stored = true;   // (the loads went out a block ago)
+      if (!fetched && kb + 96 >= k_hi) fetch_key();
+      if (last) {
+        if (!stored) store_key(), stored = true;
+        __threadfence_block();
+      }
+    });
+  } else {
+    tl.template walk<false>(qf, col_lo, col_hi, partial);
+  }
   const float lt = tl.sum_l(0);
   if constexpr (JOIN) {
     __shared__ __attribute__((aligned(16))) float joined[JOIN_SPLITS][16][D + 4];
