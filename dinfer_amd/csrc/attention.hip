@@ -114,8 +114,7 @@ struct Frags {
 //   k_lo, k_hi  the keys this wave may touch at all (held pages, written slots)
 // load() issues the loads of one block, compute() consumes them; walk() keeps the next block's
 // loads in flight while the current one is computed.
-// STREAM: K and V are read with non-temporal loads (each byte is used once: many requests, keys read once).
-template <int DT, int NT, bool P2, bool STREAM = false>
+template <int DT, int NT, bool P2>
 struct Tile {
   static constexpr int KS = (DT + 1) / 2;  // 32-wide steps over the head dimension
   static constexpr float LAZY = 6.f;       // weights up to 2^6 before the reference follows the maximum
@@ -147,7 +146,8 @@ struct Tile {
   // lies in a page the request holds, so straight-line code with all loads in flight at once. What
   // was loaded for such a key never counts: its score is masked, and accumulate() zeroes its value.
   // CLAMP = false: the block lies wholly inside [k_lo, k_hi), so no key needs replacing.
-  template <bool CLAMP>
+  // STREAM: K and V are read with non-temporal loads (a step's keys exceed the caches and each byte is used once).
+  template <bool CLAMP, bool STREAM>
   __device__ __forceinline__ void load_k(Frags<DT>& f, int kb) {
     constexpr int D = DT * 16;
     const int lane = threadIdx.x & 63, i16 = lane & 15, g4 = lane >> 4;
@@ -176,7 +176,7 @@ struct Tile {
     }
   }
 
-  template <bool CLAMP>
+  template <bool CLAMP, bool STREAM>
   __device__ __forceinline__ void load_v(Frags<DT>& f, int kb) {
     const int lane = threadIdx.x & 63, i16 = lane & 15, g4 = lane >> 4;
     const int ps = pages.ps;
@@ -192,11 +192,11 @@ struct Tile {
     for (int d = 0; d < DT; ++d) f.v[d] = ld16<STREAM>(vrow + d * 16 * ps);
   }
 
-  template <bool CLAMP>
+  template <bool CLAMP, bool STREAM>
   __device__ __forceinline__ void load(Frags<DT>& f, int kb) {
     pages.ensure(kb);
-    load_k<CLAMP>(f, kb);
-    load_v<CLAMP>(f, kb);
+    load_k<CLAMP, STREAM>(f, kb);
+    load_v<CLAMP, STREAM>(f, kb);
   }
 
   // S^T of one block: s[t][a] holds, for column i16 of tile t, the keys kb + 8 g4 + 4 a + {0..3}
@@ -301,7 +301,7 @@ struct Tile {
   // requests of 2k and 4k keys, one wave a SIMD: within 1 % either way, 5.6 to 5.9 TB/s with it and without).
   // hook(kb, last): called before block kb's loads are issued; `last` says that kb is the wave's last block. The wave
   // that brings the row's own key issues that key's loads a block early there and stores it before the last block.
-  template <bool TWO_BODIES, class MaskFn, class Hook>
+  template <bool TWO_BODIES, bool STREAM, class MaskFn, class Hook>
   __device__ __forceinline__ void walk(const bf16x8 (&qf)[NT][KS], const int (&col_lo)[NT], const int (&col_hi)[NT],
                                        MaskFn mask, Hook hook) {
     Frags<DT> f;
@@ -309,10 +309,10 @@ struct Tile {
     for (int kb = k_lo & ~31; kb < k_hi; kb += 32) {
       hook(kb, kb + 32 >= k_hi);
       if (!TWO_BODIES || mask(kb)) {
-        load<true>(f, kb);
+        load<true, STREAM>(f, kb);
         compute<true>(f, qf, kb, col_lo, col_hi);
       } else {
-        load<false>(f, kb);
+        load<false, STREAM>(f, kb);
         compute<false>(f, qf, kb, col_lo, col_hi);
       }
     }
@@ -320,7 +320,7 @@ struct Tile {
   template <bool TWO_BODIES, class MaskFn>
   __device__ __forceinline__ void walk(const bf16x8 (&qf)[NT][KS], const int (&col_lo)[NT], const int (&col_hi)[NT],
                                        MaskFn mask) {
-    walk<TWO_BODIES>(qf, col_lo, col_hi, mask, [](int, bool) {});
+    walk<TWO_BODIES, false>(qf, col_lo, col_hi, mask, [](int, bool) {});
   }
 
   // total of l over the four lane groups of a column
@@ -566,21 +566,25 @@ __device__ __forceinline__ void split_range(int seq, int window, int splits, int
 // JOIN (up to JOIN_SPLITS parts: many requests): the parts of a (kv head, request) are the waves of one workgroup,
 // meet in LDS and are combined there as attn_decode_merge_kernel combines them, so that kernel does not run.
 constexpr int JOIN_SPLITS = 4;
+constexpr int64_t STREAM_FROM_BYTES = 100 * 1000 * 1000;
 
 // POST: q arrives as the product left it; the kernel norms and rotates it on the way into its registers (every part
 // for itself: the head is 2 D bytes), and the wave whose part ends with the row's own position norms and rotates the
 // new key and stores it and the new value into their pages before it reads its last block.
 // (The pages are written through post.k_cache / v_cache and read through kc / vc: no __restrict__ on those.)
-template <int DT, bool P2, bool STREAM, bool JOIN = false, bool POST = false>
-// (JOIN runs where requests are many and parts few: a CU holds 4 to 8 of its waves, registers are no limit there;
-// POST without JOIN runs with about one wave per SIMD, and its prologue holds a head, gains and angles at once)
+// LATE (POST only): the new key is dealt with inside the walk instead of before it (see there).
+// stream_from: from this many bytes of keys and values in a step on (the request's own visible keys times the number
+// of requests: a wave knows no more) they are read with non-temporal loads.
+template <int DT, bool P2, bool LATE, bool JOIN = false, bool POST = false>
+// (These launches aim at about one wave a SIMD, and JOIN runs where a CU holds 4 to 8 of its waves: registers are no
+// limit; POST holds a head, gains and angles at once in its prologue.)
 __global__ void __launch_bounds__(JOIN ? 64 * JOIN_SPLITS : 64)
-__attribute__((amdgpu_waves_per_eu(JOIN || POST ? 2 : 4, 8)))
+__attribute__((amdgpu_waves_per_eu(2, 8)))
 attn_decode_kernel(
     const bf16* __restrict__ q, int64_t ld_q, float* __restrict__ part, const bf16* kc, const bf16* vc,
     const int32_t* __restrict__ block_table, int64_t max_blocks, const int32_t* __restrict__ cu_seqlens,
     const int32_t* __restrict__ seq_lens, int splits, float scale_log2e, int window, int H, int Hkv, int ps,
-    bf16* __restrict__ out = nullptr, int64_t ld_out = 0, DecodePost post = DecodePost{}) {
+    int64_t stream_from, bf16* __restrict__ out = nullptr, int64_t ld_out = 0, DecodePost post = DecodePost{}) {
   constexpr int D = DT * 16;
   constexpr int KS = (DT + 1) / 2;
   static_assert(!POST || DT % 4 == 0, "the fused norm and rotation keep both elements of a pair in one lane");
@@ -596,7 +600,8 @@ attn_decode_kernel(
   const bf16* qp = q + (int64_t)row * ld_q + (int64_t)(hk * G + (i16 < G ? i16 : 0)) * D;
   int k_lo, k_hi, kps;
   bf16x8 qf[1][KS];
-  Tile<DT, 1, P2, STREAM> tl;
+  Tile<DT, 1, P2> tl;
+  int seq;
   bool writer = false;
   int w_pos = 0;
   int64_t w_slot = -1;
@@ -607,7 +612,7 @@ attn_decode_kernel(
     if (post.wq) qh.load_gains(post.wq);
     const int pos_row = post.cos_sin ? post.pos[row] : 0;
     const int64_t slot = post.slots ? post.slots[row] : -1;
-    const int seq = seq_lens[b];
+    seq = seq_lens[b];
     split_range(seq, window, splits, sp, &k_lo, &k_hi, &kps);
     if (!JOIN && k_lo >= k_hi) return;
     // ... with the length the block table, with the position the angles; the part that ends with the row's own
@@ -623,7 +628,7 @@ attn_decode_kernel(
     }
     w_pos = pos_row;
     w_slot = slot;
-    if (!STREAM && writer) {
+    if (!LATE && writer) {
       // few requests, short parts: the new key and value are dealt with here, at once (the loads are asked for only now,
       // when the registers of q's head are free); see below for the launches of many requests
       const int64_t blk = slot / ps;
@@ -648,7 +653,8 @@ attn_decode_kernel(
       }
     }
   } else {
-    split_range(seq_lens[b], window, splits, sp, &k_lo, &k_hi, &kps);
+    seq = seq_lens[b];
+    split_range(seq, window, splits, sp, &k_lo, &k_hi, &kps);
     // an empty part writes nothing; the merge kernel skips it by the same rule. (JOIN: it walks no block and
     // leaves m = -inf, which weighs nothing; its wave must reach the barrier below.)
     if (!JOIN && k_lo >= k_hi) return;
@@ -662,9 +668,21 @@ attn_decode_kernel(
   const int col_lo[1] = {k_lo}, col_hi[1] = {k_hi};
   // (reading the first block before q is normed, or two blocks ahead, was measured at 1 and 8 requests: no gain)
   const auto partial = [&](int kb) { return kb < k_lo || kb + 32 > k_hi; };
-  if constexpr (POST && !STREAM) {
+  // Where a step's keys and values exceed the caches they are read past them (every layer has keys of its own, so
+  // none is read twice anyway): 8 kv heads of 128, 8 requests of 32k keys 193 -> 175 us, 16 of 2k 33.7 -> 31.7,
+  // 8 of 4k 33.6 -> 31.7; below about 100 MB a step the plain loads are faster (one request of 8k keys 19.0 against
+  // 21.6 us, 4 of 2k 16.1 against 17.6). Both walks are in the kernel, the choice is uniform over the wave.
+  const int seen = window > 0 && window < seq ? window : seq;
+  const auto walk = [&](auto hook) {
+    // (LATE is for many requests, whose keys exceed the caches at any length worth a thought)
+    if (LATE || (int64_t)gridDim.z * seen * (Hkv * D * 4) >= stream_from)
+      tl.template walk<false, true>(qf, col_lo, col_hi, partial, hook);
+    else
+      tl.template walk<false, false>(qf, col_lo, col_hi, partial, hook);
+  };
+  if constexpr (POST && !LATE) {
     // the key was stored in the prologue; the fence lets the wave's own loads of its last block see it
-    tl.template walk<false>(qf, col_lo, col_hi, partial, [&](int, bool last) {
+    walk([&](int, bool last) {
       if (writer && last) __threadfence_block();
     });
   } else if constexpr (POST) {
@@ -705,7 +723,7 @@ attn_decode_kernel(
       }
     };
     bool stored = false;
-    tl.template walk<false>(qf, col_lo, col_hi, partial, [&](int kb, bool last) {
+    walk([&](int kb, bool last) {
       if (!writer) return;
       if (fetched && !stored) store_key(), stored = true;   // (the loads went out a block ago)
       if (!fetched && kb + 96 >= k_hi) fetch_key();
@@ -715,7 +733,7 @@ attn_decode_kernel(
       }
     });
   } else {
-    tl.template walk<false>(qf, col_lo, col_hi, partial);
+    walk([](int, bool) {});
   }
   const float lt = tl.sum_l(0);
   if constexpr (JOIN) {
@@ -894,36 +912,41 @@ inline int compute_units() {
   return cached[dev];
 }
 
+// The form of the decode kernel for a launch. LATE exists where the new key is the kernel's business and its
+// registers allow it (head size 256 would spill).
+template <int DT, bool P2, bool JOIN, bool POST>
+auto decode_kernel_for(bool late) {
+  if constexpr (POST && DT <= 8) {
+    if (late) return attn_decode_kernel<DT, P2, true, JOIN, POST>;
+  }
+  return attn_decode_kernel<DT, P2, false, JOIN, POST>;
+}
+
 template <int DT, bool POST>
 int launch_decode(const bf16* q, int64_t ld_q, bf16* out, int64_t ld_out, float* part, const bf16* kc, const bf16* vc,
                   const int32_t* bt, int64_t max_blocks, const int32_t* cu, const int32_t* sl, int num_reqs,
                   int splits, float scale, int window, int H, int Hkv, int ps, const DecodePost& post,
                   hipStream_t stream) {
-  // many requests: the keys of a step exceed the caches and each is used once, so they are read past
-  // them (measured at 64 requests of 2k-4k keys: 10% faster; at 8 or fewer, slightly slower)
-  const bool p2 = (ps & (ps - 1)) == 0, stream_kv = num_reqs >= 32;
+  // many requests (parts of dozens of blocks): the new key is dealt with inside the walk
+  const bool p2 = (ps & (ps - 1)) == 0, late = num_reqs >= 32;
+  const int64_t stream_from = STREAM_FROM_BYTES;
   if constexpr (DT <= 8) {  // (the parts of head size 256 do not fit the LDS of a workgroup)
     // Workgroups of `splits` waves are placed whole: where their number leaves the last round over the CUs thin
     // (320 workgroups on 256 CUs: some CUs get two, most one) single waves spread better and the merge kernel is the
     // lesser cost. Measured at 8 kv heads: 32, 56 and 64 requests gain 0.12 to 0.17 ms a step, 40 and 48 lose.
     const double per_cu = (double)Hkv * num_reqs / compute_units();
     if (splits <= JOIN_SPLITS && (per_cu <= 1. || ceil(per_cu) <= 1.15 * per_cu)) {
-      auto kernel = p2 ? (stream_kv ? attn_decode_kernel<DT, true, true, true, POST>
-                                    : attn_decode_kernel<DT, true, false, true, POST>)
-                       : (stream_kv ? attn_decode_kernel<DT, false, true, true, POST>
-                                    : attn_decode_kernel<DT, false, false, true, POST>);
+      auto kernel = p2 ? decode_kernel_for<DT, true, true, POST>(late) : decode_kernel_for<DT, false, true, POST>(late);
       kernel<<<dim3(1, (unsigned)Hkv, (unsigned)num_reqs), 64 * splits, 0, stream>>>(
-          q, ld_q, part, kc, vc, bt, max_blocks, cu, sl, splits, scale * LOG2E, window, H, Hkv, ps, out, ld_out, post);
+          q, ld_q, part, kc, vc, bt, max_blocks, cu, sl, splits, scale * LOG2E, window, H, Hkv, ps, stream_from, out, ld_out,
+          post);
       return launch_status();
     }
   }
-  auto kernel = p2 ? (stream_kv ? attn_decode_kernel<DT, true, true, false, POST>
-                                : attn_decode_kernel<DT, true, false, false, POST>)
-                   : (stream_kv ? attn_decode_kernel<DT, false, true, false, POST>
-                                : attn_decode_kernel<DT, false, false, false, POST>);
+  auto kernel = p2 ? decode_kernel_for<DT, true, false, POST>(late) : decode_kernel_for<DT, false, false, POST>(late);
   kernel<<<dim3((unsigned)splits, (unsigned)Hkv, (unsigned)num_reqs), 64, 0, stream>>>(
-      q, ld_q, part, kc, vc, bt, max_blocks, cu, sl, splits, scale * LOG2E, window, H, Hkv, ps, (bf16*)nullptr,
-      (int64_t)0, post);
+      q, ld_q, part, kc, vc, bt, max_blocks, cu, sl, splits, scale * LOG2E, window, H, Hkv, ps, stream_from,
+      (bf16*)nullptr, (int64_t)0, post);
   const int D = DT * 16;
   attn_decode_merge_kernel<<<dim3((unsigned)H, (unsigned)num_reqs), 64, 0, stream>>>(part, out, ld_out, cu, sl, splits,
                                                                                      window, H, D);

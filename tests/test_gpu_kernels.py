@@ -500,6 +500,34 @@ def test_attention_decode_parts_longer_than_64_pages(page, window, side, entry):
                 assert (got[b, hk * (H // Hkv)] - vv[spikes[b][0], hk]).abs().max() < 0.1, f"request {b}: the spiked key"
 
 
+@pytest.mark.parametrize("entry", ["plain", "post"])
+@pytest.mark.parametrize("window", [0, 3230])
+def test_attention_decode_reads_past_the_caches_from_100_mb_a_step(window, entry):
+    """Where a request's visible keys times the number of requests come to 100 MB of keys and values (8 requests of
+    3,200 keys of 8 kv heads of 128: 105 MB) a wave of the decode kernel reads them with non-temporal loads; the short
+    requests of the same launch take the other walk. Sharp scores, and in every request one key anywhere decides the
+    row."""
+    H, Hkv, D, page, splits = 16, 8, 128, 16, 16
+    hist = [3300, 500, 3210, 64, 3500, 0, 3250, 1000]
+    B = len(hist)
+    first = lambda h: max(h + 1 - window, 0) if window else 0      # the row stands at position h
+    spikes = {b: (first(h) + (h - first(h)) * (b + 1) // (B + 1), 3.0) for b, h in enumerate(hist) if h > 0}
+    if entry == "post":
+        decode_post_case(H, Hkv, D, page, window, "bf16", hist, splits, device=DEV, spike=spikes, sharp=3.0)
+        return
+    q, kc, vc, m, outs = paged_case(torch.bfloat16, H, Hkv, D, page, hist, [1] * B, seed=29, spike=spikes, sharp=3.0)
+    out = torch.zeros(B, H * D, device=DEV, dtype=torch.bfloat16)
+    part = torch.full((B * H * splits * (D + 4),), float("nan"), device=DEV)
+    ops().attn_decode(q, out, part, kc, vc, m["bt"], None, m["sl"], B, splits, scale=D ** -0.5, window=window,
+                      heads=H, kv_heads=Hkv, head_dim=D, page_size=page)
+    want = expected_attention(outs, hist, D ** -0.5, window, DEV)
+    got = out.double().cpu().view(B, H, D)
+    torch.testing.assert_close(got, want, rtol=2e-2, atol=2e-2)
+    for b, (key, _) in spikes.items():
+        for hk in range(Hkv):
+            assert (got[b, hk * (H // Hkv)] - outs[b][2][key, hk]).abs().max() < 0.1, f"request {b}: the spiked key"
+
+
 def flash_wave_runs(hist, q_len, window, rows):
     """The runs of keys the four waves of the last workgroup of a request walk (csrc/attention.hip, attn_flash_kernel)."""
     q0 = (q_len - 1) // rows * rows
