@@ -217,17 +217,73 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_neox_kernel(
   }
 }
 
+// V into its transposed pages for many tokens: one wave takes 8 consecutive tokens of one kv head.
+// When their slots are 8 consecutive slots starting at a multiple of 8 (a prompt portion that starts
+// on such a boundary), a lane gathers two dims of the 8 tokens and stores them as two 16-byte rows
+// of V^T; otherwise it falls back to one 2-byte store per element.
+// (group: which run of 8 * WAVES tokens the workgroup takes.)
+__device__ __forceinline__ void v_write_transposed(const bf16* __restrict__ qkv, int64_t ld, int64_t v_off,
+                                                   bf16* __restrict__ v_cache, const int64_t* __restrict__ slots, int T,
+                                                   int Hkv, int D, int page, int group, int hk) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int t0 = (group * WAVES + wave) * 8;
+  if (t0 >= T) return;
+  const int n = T - t0 < 8 ? T - t0 : 8;
+  const int64_t s0 = slots[t0];
+  bool aligned = n == 8 && s0 >= 0 && (s0 & 7) == 0;
+  for (int j = 1; j < n && aligned; ++j) aligned = slots[t0 + j] == s0 + j;
+  const bf16* src = qkv + (int64_t)t0 * ld + v_off + (int64_t)hk * D;
+  for (int d2 = lane; d2 < D / 2; d2 += 64) {
+    bf16x2 v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (j < n) v[j] = *(const bf16x2*)(src + (int64_t)j * ld + 2 * d2);
+    if (aligned) {
+      const int64_t blk = s0 / page;
+      const int off = (int)(s0 % page);
+      bf16* vd = v_cache + ((blk * Hkv + hk) * (int64_t)D + 2 * d2) * page + off;
+      bf16x8 a, b;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        a[j] = v[j][0];
+        b[j] = v[j][1];
+      }
+      *(bf16x8*)vd = a;
+      *(bf16x8*)(vd + page) = b;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        if (j >= n) break;
+        const int64_t sl = slots[t0 + j];
+        if (sl < 0) continue;
+        bf16* vd = v_cache + (((sl / page) * Hkv + hk) * (int64_t)D + 2 * d2) * page + sl % page;
+        vd[0] = v[j][0];
+        vd[page] = v[j][1];
+      }
+    }
+  }
+}
+
 // bf16, whole-head neox rotation, D in {64, 128, 256}: LPH = D / 8 lanes share a head, each with 8
 // consecutive dims in one 16-byte load; the partner of a pair sits LPH / 2 lanes away and comes by a
 // cross-lane read. A wave covers 64 / LPH heads of one token per instruction, an order of magnitude
 // fewer memory instructions than 2-byte accesses.
+// gather_v > 0: V is not written by the heads' lanes; the workgroups from blockIdx.x = `tokens` on (gather_v of them,
+// one per kv head and run of 8 * WAVES tokens) gather it into its transposed pages, in the same launch (a kernel of
+// its own for that cost a prefill layer 5.7 us, a step of prompt portions beside decoding requests 7.8).
 template <int LPH>
 __global__ void __launch_bounds__(WAVES * 64) qkv_post_vec_kernel(
     bf16* __restrict__ qkv, int64_t ld, int64_t q_off, int64_t k_off, int64_t v_off, const void* __restrict__ wq,
     const void* __restrict__ wk, int wf32, float eps, float w_offset, const int32_t* __restrict__ pos,
     const float* __restrict__ cos_sin, bf16* __restrict__ k_cache, bf16* __restrict__ v_cache,
-    const int64_t* __restrict__ slots, int H, int Hkv, int page, int skip_v) {
+    const int64_t* __restrict__ slots, int H, int Hkv, int page, int tokens, int gather_v) {
   constexpr int D = LPH * 8, HALF = D / 2, HPW = 64 / LPH;  // heads per wave
+  if ((int)blockIdx.x >= tokens) {
+    const int j = (int)blockIdx.x - tokens;
+    if (blockIdx.y == 0) v_write_transposed(qkv, ld, v_off, v_cache, slots, tokens, Hkv, D, page, j / Hkv, j % Hkv);
+    return;
+  }
+  const bool skip_v = gather_v > 0;
   const int64_t t = blockIdx.x;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int sub = lane / LPH, l = lane % LPH;  // which head of the wave, which 8 dims of it
@@ -326,53 +382,6 @@ __global__ void __launch_bounds__(WAVES * 64) qkv_post_vec_kernel(
   }
 }
 
-// V into its transposed pages for many tokens: one wave takes 8 consecutive tokens of one kv head.
-// When their slots are 8 consecutive slots starting at a multiple of 8 (a prompt portion that starts
-// on such a boundary), a lane gathers two dims of the 8 tokens and stores them as two 16-byte rows
-// of V^T; otherwise it falls back to one 2-byte store per element.
-__global__ void __launch_bounds__(WAVES * 64) v_write_transposed_kernel(const bf16* __restrict__ qkv, int64_t ld,
-                                                                        int64_t v_off, bf16* __restrict__ v_cache,
-                                                                        const int64_t* __restrict__ slots, int T,
-                                                                        int Hkv, int D, int page) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int t0 = (blockIdx.x * WAVES + wave) * 8, hk = blockIdx.y;
-  if (t0 >= T) return;
-  const int n = T - t0 < 8 ? T - t0 : 8;
-  const int64_t s0 = slots[t0];
-  bool aligned = n == 8 && s0 >= 0 && (s0 & 7) == 0;
-  for (int j = 1; j < n && aligned; ++j) aligned = slots[t0 + j] == s0 + j;
-  const bf16* src = qkv + (int64_t)t0 * ld + v_off + (int64_t)hk * D;
-  for (int d2 = lane; d2 < D / 2; d2 += 64) {
-    bf16x2 v[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j)
-      if (j < n) v[j] = *(const bf16x2*)(src + (int64_t)j * ld + 2 * d2);
-    if (aligned) {
-      const int64_t blk = s0 / page;
-      const int off = (int)(s0 % page);
-      bf16* vd = v_cache + ((blk * Hkv + hk) * (int64_t)D + 2 * d2) * page + off;
-      bf16x8 a, b;
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        a[j] = v[j][0];
-        b[j] = v[j][1];
-      }
-      *(bf16x8*)vd = a;
-      *(bf16x8*)(vd + page) = b;
-    } else {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        if (j >= n) break;
-        const int64_t sl = slots[t0 + j];
-        if (sl < 0) continue;
-        bf16* vd = v_cache + (((sl / page) * Hkv + hk) * (int64_t)D + 2 * d2) * page + sl % page;
-        vd[0] = v[j][0];
-        vd[page] = v[j][1];
-      }
-    }
-  }
-}
-
 }  // namespace
 
 extern "C" int dinfer_qkv_post(int dtype, void* qkv, int64_t tokens, int64_t ld, int64_t q_off, int64_t k_off,
@@ -398,17 +407,16 @@ extern "C" int dinfer_qkv_post(int dtype, void* qkv, int64_t tokens, int64_t ld,
   if (whole_head_neox && vec_ok) {
     const int lph = head_dim / 8, hpw = 64 / lph;
     // many tokens fill the chip with one workgroup each; few tokens spread their heads over several
-    const dim3 vgrid((unsigned)tokens, tokens >= 512 ? 1u : (unsigned)((items + WAVES * hpw - 1) / (WAVES * hpw)));
-    // many tokens: V goes to its transposed pages through the gathering kernel (16-byte stores)
-    const int skip_v = (slot_mapping && token_runs && tokens >= 64 && page_size % 8 == 0 && ((uintptr_t)v_cache % 16) == 0) ? 1 : 0;
-    if (skip_v)
-      v_write_transposed_kernel<<<dim3((unsigned)((tokens + 8 * WAVES - 1) / (8 * WAVES)), (unsigned)kv_heads), WAVES * 64,
-                                  0, stream>>>((const bf16*)qkv, ld, v_off, (bf16*)v_cache, slot_mapping, (int)tokens,
-                                               kv_heads, head_dim, page_size);
+    // many tokens: V goes to its transposed pages through workgroups that gather it (16-byte stores)
+    const bool gather = slot_mapping && token_runs && tokens >= 64 && page_size % 8 == 0 && ((uintptr_t)v_cache % 16) == 0;
+    const int64_t gather_v = gather ? (tokens + 8 * WAVES - 1) / (8 * WAVES) * kv_heads : 0;
+    if (tokens + gather_v > 0x7fffffff) return ERR_BAD_SHAPE;
+    const dim3 vgrid((unsigned)(tokens + gather_v),
+                     tokens >= 512 ? 1u : (unsigned)((items + WAVES * hpw - 1) / (WAVES * hpw)));
 #define DINFER_QKV_VEC(LPH_)                                                                                          \
   qkv_post_vec_kernel<LPH_><<<vgrid, WAVES * 64, 0, stream>>>(                                                         \
       (bf16*)qkv, ld, q_off, k_off, v_off, q_gain, k_gain, w_f32, eps, w_offset, positions, cos_sin, (bf16*)k_cache, \
-      (bf16*)v_cache, slot_mapping, heads, kv_heads, page_size, skip_v)
+      (bf16*)v_cache, slot_mapping, heads, kv_heads, page_size, (int)tokens, (int)gather_v)
     if (lph == 8) DINFER_QKV_VEC(8);
     else if (lph == 16) DINFER_QKV_VEC(16);
     else DINFER_QKV_VEC(32);
