@@ -268,7 +268,10 @@ def test_attention_decode_takes_norm_rotation_and_cache_write_along(H, Hkv, D, p
     # parts of several blocks, a part of one block (the store is waited for at once), a single key, many short ones
     rng = random.Random(3)
     for hist, splits in (([299, 69, 0, 1000], 7), ([rng.randrange(64) for _ in range(32)], 2),
-                         ([0, 45, 1000, 130], 4), ([100, 31, 32, 33], 1)):
+                         ([0, 45, 1000, 130], 4), ([100, 31, 32, 33], 1),
+                         # 32 requests and more (the new key is dealt with inside the walk) with parts that a merge
+                         # kernel combines: parts of one and two blocks, then of three to five
+                         ([rng.randrange(200) for _ in range(33)], 6), ([300 + rng.randrange(400) for _ in range(34)], 5)):
         decode_post_case(H, Hkv, D, page, window, gains, hist, splits)
 
 
