@@ -567,6 +567,7 @@ __device__ __forceinline__ void split_range(int seq, int window, int splits, int
 // meet in LDS and are combined there as attn_decode_merge_kernel combines them, so that kernel does not run.
 constexpr int JOIN_SPLITS = 4;
 constexpr int64_t STREAM_FROM_BYTES = 100 * 1000 * 1000;
+constexpr int64_t STREAM_FROM_BYTES_FEW = 170 * 1000 * 1000;  // for one or two requests
 
 // POST: q arrives as the product left it; the kernel norms and rotates it on the way into its registers (every part
 // for itself: the head is 2 D bytes), and the wave whose part ends with the row's own position norms and rotates the
@@ -671,7 +672,8 @@ attn_decode_kernel(
   // Where a step's keys and values exceed the caches they are read past them (every layer has keys of its own, so
   // none is read twice anyway): 8 kv heads of 128, 8 requests of 32k keys 193 -> 175 us, 16 of 2k 33.7 -> 31.7,
   // 8 of 4k 33.6 -> 31.7; below about 100 MB a step the plain loads are faster (one request of 8k keys 19.0 against
-  // 21.6 us, 4 of 2k 16.1 against 17.6). Both walks are in the kernel, the choice is uniform over the wave.
+  // 21.6 us, 4 of 2k 16.1 against 17.6; one or two requests up to 170 MB: one of 32k 39.7 against 42.1, of 48k 51.5
+  // against 48.9). Both walks are in the kernel, the choice is uniform over the wave.
   const int seen = window > 0 && window < seq ? window : seq;
   const auto walk = [&](auto hook) {
     // (LATE is for many requests, whose keys exceed the caches at any length worth a thought)
@@ -929,7 +931,8 @@ int launch_decode(const bf16* q, int64_t ld_q, bf16* out, int64_t ld_out, float*
                   hipStream_t stream) {
   // many requests (parts of dozens of blocks): the new key is dealt with inside the walk
   const bool p2 = (ps & (ps - 1)) == 0, late = num_reqs >= 32;
-  const int64_t stream_from = STREAM_FROM_BYTES;
+  // (one or two requests: measured level at 134 MB a step or behind by 6 %, ahead by 5 to 8 % from 200 MB on)
+  const int64_t stream_from = num_reqs <= 2 ? STREAM_FROM_BYTES_FEW : STREAM_FROM_BYTES;
   if constexpr (DT <= 8) {  // (the parts of head size 256 do not fit the LDS of a workgroup)
     // Workgroups of `splits` waves are placed whole: where their number leaves the last round over the CUs thin
     // (320 workgroups on 256 CUs: some CUs get two, most one) single waves spread better and the merge kernel is the
