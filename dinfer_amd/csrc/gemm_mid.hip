@@ -17,9 +17,10 @@
 // load makes the compiler wait for everything in flight wherever it needs one of them.
 //
 // Slices of k are different workgroups (blockIdx.y); each writes float partial sums
-// P[slice][N / 4][MT * 16][4] (a wave's stores are whole lines), and gemm_mid_reduce_kernel adds them
-// in slice order (no atomics: a launch shape gives the same bits every time), applies
-// silu(gate) * up for the gated form, and rounds once.
+// P[slice][MT * 16][N] (a token's row is contiguous, so that the pass over them can take a token a workgroup), and
+// gemm_mid_reduce_kernel adds them in slice order (no atomics: a launch shape gives the same bits every time), applies
+// silu(gate) * up for the gated form, and rounds once. gemm_mid_reduce_norm_kernel is that pass for a product that
+// completes the residual stream before an RMSNorm: it adds into the stream and writes the norm's output as well.
 //
 // v_mfma_f32_16x16x32_bf16, weight as the A operand: a tile is 16 weight rows x 16 tokens.
 // K must be a multiple of 8 (16-byte loads), N of 4.
@@ -150,7 +151,7 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_mid_m_kernel(const bf16* __re
   char* const put = strip + lrow * ROW_BYTES + lpiece * 16;
   const char* const get = strip + i16 * ROW_BYTES + g4 * 16;
   const char* const a_get = smem + i16 * a_stride + g4 * 16;
-  // partial sums of this slice: [N / 4][MT * 16][4], so that a wave's stores are whole lines
+  // partial sums of this slice: [MT * 16][N]
   f32x4* const out = (f32x4*)P + (int64_t)blockIdx.y * (N >> 2) * (MT * 16);
 
   f32x4 acc[RT][MT];
@@ -196,7 +197,7 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_mid_m_kernel(const bf16* __re
       const int n = n0 + r * 16 + 4 * g4;
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
-        if (n < N) out[(int64_t)(n >> 2) * (MT * 16) + t * 16 + i16] = acc[r][t];  // N % 4 == 0: all four or none
+        if (n < N) out[(int64_t)(t * 16 + i16) * (N >> 2) + (n >> 2)] = acc[r][t];  // N % 4 == 0: all four or none
         acc[r][t] = f32x4{0.f, 0.f, 0.f, 0.f};
       }
     }
@@ -216,31 +217,105 @@ __global__ void __launch_bounds__(WAVES * 64) gemm_mid_m_kernel(const bf16* __re
   if (q + 1 < total) compute_round(1);
 }
 
-// C[m][n] = sum over slices of P[s][n / 4][m][n % 4] in slice order; GATED: the first N columns of P are the gate,
-// the next N the up projection, and C[m][n] = silu(sum gate) * sum up. One thread per token and four columns.
+// C[m][n] = sum over slices of P[s][m][n] in slice order; GATED: a row of P is the gate's N columns and then the up
+// projection's, and C[m][n] = silu(sum gate) * sum up. One thread per token and four columns.
 template <class O, bool GATED>
 __global__ void __launch_bounds__(256) gemm_mid_reduce_kernel(const float* __restrict__ P, int mp, int slices,
                                                               O* __restrict__ C, int64_t ldc, int M, int N) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int quads = N >> 2;
-  if (i >= (int64_t)quads * mp) return;
-  const int q = (int)(i / mp), m = (int)(i % mp);
-  if (m >= M) return;
-  const int64_t slice_stride = (int64_t)(GATED ? 2 * quads : quads) * mp;
-  const f32x4* p = (const f32x4*)P + (int64_t)q * mp + m;
+  if (i >= (int64_t)quads * M) return;
+  const int m = (int)(i / quads), q = (int)(i % quads);
+  const int row_quads = GATED ? 2 * quads : quads;
+  const int64_t slice_stride = (int64_t)row_quads * mp;
+  const f32x4* p = (const f32x4*)P + (int64_t)m * row_quads + q;
   f32x4 g = *p, u;
-  if (GATED) u = p[(int64_t)quads * mp];
+  if (GATED) u = p[quads];
   for (int s = 1; s < slices; ++s) {
     const f32x4 v = p[s * slice_stride];
     g[0] += v[0]; g[1] += v[1]; g[2] += v[2]; g[3] += v[3];
     if (GATED) {
-      const f32x4 w = p[s * slice_stride + (int64_t)quads * mp];
+      const f32x4 w = p[s * slice_stride + quads];
       u[0] += w[0]; u[1] += w[1]; u[2] += w[2]; u[3] += w[3];
     }
   }
   O* c = C + (int64_t)m * ldc + 4 * q;
 #pragma unroll
   for (int e = 0; e < 4; ++e) c[e] = from_f32<O>(GATED ? (g[e] / (1.f + expf(-g[e]))) * u[e] : g[e]);
+}
+
+// The pass over the partial sums for a product that completes the residual stream before an RMSNorm, a token a
+// workgroup: H[m][n] += sum over slices of P[s][m][n] (the float sum of the slices in their order and the stream,
+// rounded once), and OUT[m][n] = H[m][n] / sqrt(mean(H[m]^2) + eps) * (gain[n] + gain_offset), from the rounded H as
+// the norm's own kernel reads it. Stands for this file's pass, the add and the norm: two kernels of about 5 us fewer a
+// layer. A thread keeps its columns (four at a time, up to QMAX times) between the sum and the division.
+constexpr int SINK_THREADS = 1024, SINK_QMAX = 2;
+__global__ void __launch_bounds__(SINK_THREADS) gemm_mid_reduce_norm_kernel(
+    const float* __restrict__ P, int mp, int slices, bf16* __restrict__ H, int64_t ldh, bf16* __restrict__ OUT,
+    int64_t ld_out, const void* __restrict__ gain, int gain_f32, float gain_offset, float eps, int N) {
+  __shared__ float red[16];
+  const int m = blockIdx.x, quads = N >> 2;
+  const int64_t slice_stride = (int64_t)quads * mp;
+  const f32x4* p = (const f32x4*)P + (int64_t)m * quads;
+  bf16* h = H + (int64_t)m * ldh;
+  float v[SINK_QMAX][4], g[SINK_QMAX][4];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < SINK_QMAX; ++j) {
+    const int q = threadIdx.x + j * SINK_THREADS;
+    if (q < quads) {
+      f32x4 a = p[q];
+      const bf16x4 old = *(const bf16x4*)(h + 4 * q);
+      if (gain_f32) {
+        const f32x4 gv = *(const f32x4*)((const float*)gain + 4 * q);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) g[j][e] = gv[e] + gain_offset;
+      } else {
+        const bf16x4 gv = *(const bf16x4*)((const bf16*)gain + 4 * q);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) g[j][e] = (float)gv[e] + gain_offset;
+      }
+      // (eight slices' loads at a time: the pass is a chain of trips to L2 otherwise; added in slice order)
+      int s = 1;
+      for (; s + 8 <= slices; s += 8) {
+        f32x4 b[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) b[i] = p[(s + i) * slice_stride + q];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { a[0] += b[i][0]; a[1] += b[i][1]; a[2] += b[i][2]; a[3] += b[i][3]; }
+      }
+      for (; s + 2 <= slices; s += 2) {
+        const f32x4 b0 = p[s * slice_stride + q], b1 = p[(s + 1) * slice_stride + q];
+        a[0] += b0[0]; a[1] += b0[1]; a[2] += b0[2]; a[3] += b0[3];
+        a[0] += b1[0]; a[1] += b1[1]; a[2] += b1[2]; a[3] += b1[3];
+      }
+      for (; s < slices; ++s) {
+        const f32x4 b = p[s * slice_stride + q];
+        a[0] += b[0]; a[1] += b[1]; a[2] += b[2]; a[3] += b[3];
+      }
+      bf16x4 r;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        r[e] = (bf16)(a[e] + (float)old[e]);
+        v[j][e] = (float)r[e];
+        ss += v[j][e] * v[j][e];
+      }
+      *(bf16x4*)(h + 4 * q) = r;
+    }
+  }
+  ss = block_sum(ss, red);
+  const float inv = 1.f / sqrtf(ss / (float)N + eps);
+  bf16* o = OUT + (int64_t)m * ld_out;
+#pragma unroll
+  for (int j = 0; j < SINK_QMAX; ++j) {
+    const int q = threadIdx.x + j * SINK_THREADS;
+    if (q < quads) {
+      bf16x4 y;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) y[e] = (bf16)(v[j][e] * inv * g[j][e]);
+      *(bf16x4*)(o + 4 * q) = y;
+    }
+  }
 }
 
 inline bool streams_weight(int64_t rows, int64_t K) { return rows * K * (int64_t)sizeof(bf16) >= (int64_t)40 << 20; }
@@ -328,14 +403,12 @@ extern "C" int dinfer_gemm_mid_m_workspace(int64_t M, int64_t N, int64_t K, int 
 
 namespace {
 
-// The product and the pass that adds up its slices, with the partial sums in `P` (at least `capacity` bytes).
-int run_mid_m(int out_f32, const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, int64_t M, int64_t N,
-              int64_t K, int gated, int ks, int rt, void* P_, int64_t capacity, int too_small, hipStream_t stream) {
-  if (M <= 0 || N <= 0) return OK;
+// The slices' partial sums of A . W^T (W of `rows` rows) into `P` (at least `capacity` bytes); *slices: how many.
+int partial_sums(const void* A, int64_t lda, const void* W, int64_t ldw, int64_t M, int64_t rows, int64_t K, int ks, int rt,
+                 void* P_, int64_t capacity, int too_small, int* slices, hipStream_t stream) {
   if (M > 64) return ERR_UNSUPPORTED;
-  const int64_t rows = gated ? 2 * N : N;
-  if (K <= 0 || K % 8 || N % 4 || lda < K || ldw < K || ldc < N || lda % 8 || ldw % 8 || rows > 0x7fffffff ||
-      K > 0x7fffffff || ((uintptr_t)A % 16) || ((uintptr_t)W % 16) || (gated && out_f32))
+  if (K <= 0 || K % 8 || rows % 4 || lda < K || ldw < K || lda % 8 || ldw % 8 || rows > 0x7fffffff || K > 0x7fffffff ||
+      ((uintptr_t)A % 16) || ((uintptr_t)W % 16))
     return ERR_BAD_SHAPE;
   Shape s;
   if (!choose(M, rows, K, ks, rt, &s)) return ERR_UNSUPPORTED;
@@ -350,6 +423,19 @@ int run_mid_m(int out_f32, const void* A, int64_t lda, const void* W, int64_t ld
   else if (mt == 3) GO(3);
   else GO(4);
 #undef GO
+  *slices = s.slices;
+  return st;
+}
+
+// The product and the pass that adds up its slices, with the partial sums in `P` (at least `capacity` bytes).
+int run_mid_m(int out_f32, const void* A, int64_t lda, const void* W, int64_t ldw, void* C, int64_t ldc, int64_t M, int64_t N,
+              int64_t K, int gated, int ks, int rt, void* P_, int64_t capacity, int too_small, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return OK;
+  if (N % 4 || ldc < N || (gated && out_f32)) return M > 64 ? ERR_UNSUPPORTED : ERR_BAD_SHAPE;
+  struct { int slices; } s{0};
+  const int mt = (int)(M + 15) / 16;
+  const float* P = (const float*)P_;
+  const int st = partial_sums(A, lda, W, ldw, M, gated ? 2 * N : N, K, ks, rt, P_, capacity, too_small, &s.slices, stream);
   if (st != OK) return st;
   const unsigned blocks = (unsigned)(((int64_t)(mt * 16) * (N / 4) + 255) / 256);
   if (gated)
@@ -370,6 +456,28 @@ extern "C" int dinfer_gemm_mid_m(int out_f32, const void* A, int64_t lda, const 
                                  int64_t M, int64_t N, int64_t K, int gated, int ks, int rt, void* workspace,
                                  int64_t workspace_bytes, hipStream_t stream) {
   return run_mid_m(out_f32, A, lda, W, ldw, C, ldc, M, N, K, gated, ks, rt, workspace, workspace_bytes, ERR_WORKSPACE, stream);
+}
+
+// H[:M] += A . W^T in place (H bf16, the residual stream) and OUT[:M] = the RMSNorm of the new H (gain [N] bf16 or
+// float, each plus gain_offset; eps): the product, the add and the norm that reads the stream next, in two kernels.
+// N % 4 == 0 and N <= 8,192; ks, rt, workspace as for dinfer_gemm_mid_m (not gated).
+extern "C" int dinfer_gemm_mid_m_sink(const void* A, int64_t lda, const void* W, int64_t ldw, void* H, int64_t ldh, void* OUT,
+                                      int64_t ld_out, const void* gain, int gain_f32, float gain_offset, float eps,
+                                      int64_t M, int64_t N, int64_t K, int ks, int rt, void* workspace,
+                                      int64_t workspace_bytes, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return OK;
+  if (N > 4 * SINK_THREADS * SINK_QMAX) return ERR_UNSUPPORTED;
+  if (N % 4 || ldh < N || ld_out < N || ldh % 4 || ld_out % 4 || !gain || ((uintptr_t)H % 8) || ((uintptr_t)OUT % 8) ||
+      ((uintptr_t)gain % (gain_f32 ? 16 : 8)))
+    return ERR_BAD_SHAPE;
+  int slices = 0;
+  const int st = partial_sums(A, lda, W, ldw, M, N, K, ks, rt, workspace, workspace_bytes, ERR_WORKSPACE, &slices, stream);
+  if (st != OK) return st;
+  const int mt = (int)(M + 15) / 16;
+  gemm_mid_reduce_norm_kernel<<<(unsigned)M, SINK_THREADS, 0, stream>>>((const float*)workspace, mt * 16, slices, (bf16*)H, ldh,
+                                                                       (bf16*)OUT, ld_out, gain, gain_f32, gain_offset, eps,
+                                                                       (int)N);
+  return launch_status();
 }
 
 // ---- the same product for callers that cannot allocate ---------------------------------------------------------

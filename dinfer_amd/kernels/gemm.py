@@ -96,14 +96,36 @@ def matmul_nt(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, may_p
         raise RuntimeError("matrix products run on the GPU only")
     n, k = w.shape
     if k % 8 == 0 and _tall(m, n, k):
-        # slices of 1,536 with one row tile a wave where LDS holds them (up to 32 rows), else of 1,024 with two
-        ks, rt = (1536, 1) if m <= 32 else (1024, 2)
+        ks, rt = _mid_shape(m)
         ws = _mid_workspace(a.device, ops.gemm_mid_m_workspace(m, n, k, ks=ks, rt=rt))
         if ws is not None:
             return ops.gemm_mid_m(a, w, out, m, ws, ks=ks, rt=rt)
     if m <= SMALL_M and k % 8 == 0:
         return ops.gemm_small_m(a, w, out, m)
     return _library(a, w, out, m, may_pad)
+
+
+def _mid_shape(m: int) -> tuple[int, int]:
+    # slices of 1,536 with one row tile a wave where LDS holds them (up to 32 rows), else of 1,024 with two
+    return (1536, 1) if m <= 32 else (1024, 2)
+
+
+def mid_sink_nt(a: torch.Tensor, w: torch.Tensor, stream: torch.Tensor, gain: torch.Tensor, offset: float, eps: float,
+                out: torch.Tensor, m: int) -> bool:
+    """stream[:m] += a[:m] @ w.T in place and out[:m] = the RMSNorm (gain + offset, eps) of the new stream, for the
+    products of 17 to 64 rows that the LDS-resident kernel takes (a weight far wider than high: the down projection):
+    the pass over its partial sums is the add and the norm as well. False (nothing done) otherwise."""
+    n, k = w.shape
+    if not (a.is_cuda and a.dtype == torch.bfloat16 and stream.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
+            and k % 8 == 0 and _tall(m, n, k) and n <= ops.GEMM_MID_SINK_MAX_N
+            and gain.dtype in (torch.bfloat16, torch.float32)):
+        return False
+    ks, rt = _mid_shape(m)
+    ws = _mid_workspace(a.device, ops.gemm_mid_m_workspace(m, n, k, ks=ks, rt=rt))
+    if ws is None:
+        return False
+    ops.gemm_mid_m_sink(a, w, stream, out, gain, offset, eps, m, ws, ks=ks, rt=rt)
+    return True
 
 
 WIDE_FROM = 17   # up to 16 rows the few-row kernel is level with it (and carries norms)

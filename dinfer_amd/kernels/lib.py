@@ -55,6 +55,7 @@ SIGNATURES = {
     "dinfer_gemm_small_m_sink_stats_columns": ("gemm", [_L, _L, _L]),
     "dinfer_gemm_small_m_sink": ("gemm", [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _F, _P, _L, _L, _L, _L, _P]),
     "dinfer_gemm_mid_m": ("gemm_mid", [_I, _P, _L, _P, _L, _P, _L, _L, _L, _L, _I, _I, _I, _P, _L, _P]),
+    "dinfer_gemm_mid_m_sink": ("gemm_mid", [_P, _L, _P, _L, _P, _L, _P, _L, _P, _I, _F, _F, _L, _L, _L, _I, _I, _P, _L, _P]),
     "dinfer_gemm_mid_m_workspace": ("gemm_mid", [_L, _L, _L, _I, _I, _I, _P]),
     "dinfer_gemm_mid_m_static": ("gemm_mid", [_I, _P, _L, _P, _L, _P, _L, _L, _L, _L, _I, _I, _I, _P]),
     "dinfer_gemm_mid_m_static_init": ("gemm_mid", []),

@@ -409,6 +409,25 @@ def gemm_mid_m(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, m: int, work
     return out
 
 
+GEMM_MID_SINK_MAX_N = 8192   # columns a workgroup of gemm_mid_m_sink's second kernel holds in registers
+
+
+def gemm_mid_m_sink(a: torch.Tensor, w: torch.Tensor, stream_: torch.Tensor, out: torch.Tensor, gain: torch.Tensor,
+                    gain_offset: float, eps: float, m: int, workspace: torch.Tensor, *, ks: int = 0, rt: int = 0) -> None:
+    """stream_[:m] += a[:m] @ w.T in place (the float sum of the slices and the stream, rounded once) and out[:m] = the
+    RMSNorm of the new rows (gain + gain_offset, eps): gemm_mid_m's product with a second kernel that is also the add
+    and the norm. bf16, m <= 64, N <= GEMM_MID_SINK_MAX_N."""
+    _need_gpu(a, w, stream_, out, gain, workspace)
+    n, k = w.shape
+    assert a.dtype == w.dtype == stream_.dtype == out.dtype == torch.bfloat16 and a.shape[1] == k
+    assert stream_.shape[1] == n and out.shape[1] == n and gain.numel() == n and gain.is_contiguous()
+    assert a.shape[0] >= m and stream_.shape[0] >= m and out.shape[0] >= m and workspace.is_contiguous()
+    assert gain.dtype in (torch.bfloat16, torch.float32)
+    lib.call("dinfer_gemm_mid_m_sink", a.data_ptr(), _rows(a), w.data_ptr(), _rows(w), stream_.data_ptr(), _rows(stream_),
+             out.data_ptr(), _rows(out), gain.data_ptr(), 1 if gain.dtype == torch.float32 else 0, float(gain_offset),
+             float(eps), m, n, k, ks, rt, workspace.data_ptr(), workspace.numel() * workspace.element_size(), _stream())
+
+
 def gemm_wide_supports(m: int, n: int, k: int) -> bool:
     """Whether gemm_wide takes a product of m rows with a weight of n rows (gated: n of each half) and k columns."""
     return bool(lib.get("dinfer_gemm_wide_supports")(m, n, k))

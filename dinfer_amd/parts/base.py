@@ -95,19 +95,20 @@ class Carried:
     sums of the squares of the stream); a product that takes xg as its operand and multiplies its result rows by
     rsqrt(sum(stats) / width + eps) has applied the norm. A consumer that cannot do that calls `materialise()`,
     which runs the norm's own kernel on the (complete) stream. Without xg (`scaled` False) the product has only
-    added into the stream (steps of many rows), and `materialise()` is the one way on."""
-    __slots__ = ("xg", "stats", "cols", "eps", "width", "norm", "stream", "buf", "rows")
+    added into the stream (steps of many rows), and `materialise()` is the one way on; `ready`: the product's last
+    kernel has written the norm's output into `buf` already, and `materialise()` only hands it over."""
+    __slots__ = ("xg", "stats", "cols", "eps", "width", "norm", "stream", "buf", "rows", "ready")
 
-    def __init__(self, xg, stats, cols, eps, width, norm, stream, buf, rows):
+    def __init__(self, xg, stats, cols, eps, width, norm, stream, buf, rows, ready=False):
         self.xg, self.stats, self.cols, self.eps, self.width = xg, stats, cols, eps, width
-        self.norm, self.stream, self.buf, self.rows = norm, stream, buf, rows
+        self.norm, self.stream, self.buf, self.rows, self.ready = norm, stream, buf, rows, ready
 
     @property
     def scaled(self) -> bool:
         return self.xg is not None
 
     def materialise(self) -> torch.Tensor:
-        return self.norm.forward(self.stream, self.buf, self.rows)
+        return self.buf if self.ready else self.norm.forward(self.stream, self.buf, self.rows)
 
 
 class Into:

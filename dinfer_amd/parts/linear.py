@@ -39,6 +39,9 @@ class Linear:
             cols = gemm.sink_nt(x, self.weight, into.stream, into.xg, gain, offset, into.stats, m)
             if cols:
                 return Carried(into.xg, into.stats, cols, eps, width, into.norm, into.stream, into.buf, m)
+        if params is not None and params[0] is not None and gemm.mid_sink_nt(x, self.weight, into.stream, params[0],
+                                                                            params[1], params[2], into.buf, m):
+            return Carried(None, None, 0, 0.0, width, into.norm, into.stream, into.buf, m, ready=True)
         if gemm.add_nt(x, self.weight, into.stream, m):
             return Carried(None, None, 0, 0.0, width, into.norm, into.stream, into.buf, m)
         return None

@@ -1068,6 +1068,45 @@ def test_gemm_mid_m(M):
     assert ran >= 60
 
 
+@pytest.mark.parametrize("gain_dtype,offset", [(torch.bfloat16, 0.0), (torch.float32, 1.0)])
+@pytest.mark.parametrize("M", [1, 17, 33, 50, 64])
+def test_gemm_mid_m_adds_into_the_stream_and_norms_it(M, gain_dtype, offset):
+    """The LDS-resident product whose pass over the partial sums is also the add into the residual stream and the
+    RMSNorm that reads the stream next: the stream against float64 (one rounding), the norm's output against the plain
+    norm of the stream the kernel left, rows beyond m and columns beyond N untouched; rows of very different sizes."""
+    g = torch.Generator().manual_seed(M)
+    for N, K, ks, rt in ((96, 512, 0, 0), (332, 1096, 256, 1), (4096, 12288, 1024, 2), (4096, 12288, 1536, 1),
+                         (1000, 2600, 1024, 1), (5120, 1024, 0, 0), (8192, 512, 0, 0)):
+        if ks > 1024 and M > 32:
+            continue
+        a = torch.randn(M + 1, K, generator=g).to(torch.bfloat16).to(DEV)
+        w = (torch.randn(N, K, generator=g) * 0.05).to(torch.bfloat16).to(DEV)
+        rows = torch.exp(torch.randn(M + 2, 1, generator=g) * 2)
+        whole = (torch.randn(M + 2, N + 8, generator=g) * rows).to(torch.bfloat16).to(DEV)
+        before = whole.clone()
+        stream = whole[:, :N]
+        gain = (torch.rand(N, generator=g) + 0.5 - offset).to(gain_dtype).to(DEV)
+        out_whole = torch.full((M + 2, N + 4), 7.0, dtype=torch.bfloat16, device=DEV)
+        out = out_whole[:, :N]
+        need = ops().gemm_mid_m_workspace(M, N, K, ks=ks, rt=rt)
+        ws = torch.full((need // 4 + 8,), float("nan"), device=DEV)
+        ops().gemm_mid_m_sink(a, w, stream, out, gain, offset, 1e-5, M, ws, ks=ks, rt=rt)
+        want = before[:M, :N].double() + a[:M].double() @ w.double().T
+        err = (stream[:M].double() - want).abs()
+        assert bool((err <= 1e-2 * want.abs() + 1e-3 * want.std()).all()), f"stream, N={N} K={K}: {float(err.max())}"
+        assert torch.equal(whole[M:], before[M:]) and torch.equal(whole[:, N:], before[:, N:]), "wrote beside the stream"
+        normed = plain.rms_norm(stream[:M].double(), gain.double() + offset, 1e-5)
+        err = (out[:M].double() - normed).abs()
+        assert bool((err <= 1e-2 * normed.abs() + 1e-3).all()), f"norm, N={N} K={K}: {float(err.max())}"
+        assert bool((out_whole[M:] == 7.0).all()) and bool((out_whole[:, N:] == 7.0).all()), "wrote beside the norm's output"
+    from dinfer_amd.kernels.lib import KernelError
+    with pytest.raises(KernelError):      # more columns than a workgroup of the second kernel holds
+        N, K = 8192 + 64, 512
+        ops().gemm_mid_m_sink(torch.zeros(M, K, dtype=torch.bfloat16, device=DEV), torch.zeros(N, K, dtype=torch.bfloat16, device=DEV),
+                              torch.zeros(M, N, dtype=torch.bfloat16, device=DEV), torch.zeros(M, N, dtype=torch.bfloat16, device=DEV),
+                              torch.ones(N, dtype=gain_dtype, device=DEV), 0.0, 1e-5, M, torch.zeros(1 << 22, device=DEV))
+
+
 @pytest.mark.parametrize("M", [1, 17, 33, 48, 49, 64])
 def test_gemm_wide(M):
     """The product for up to 64 rows whose waves stage their own activations in LDS: plain with bf16 and float output,
