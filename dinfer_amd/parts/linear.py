@@ -28,8 +28,10 @@ class Linear:
 
     def forward_into(self, x: torch.Tensor, into: Into, m: int) -> Carried | None:
         """into.stream[:m] += x[:m] @ W^T, returning the Carried for into.norm; None (nothing done) where no kernel
-        does this for the sizes. In steps of few rows the norm rides along (where it can be carried); in steps of many
-        the product only adds, and the norm's kernel reads one matrix instead of two and writes one instead of two."""
+        does this for the sizes. In steps of few rows the norm rides along (where it can be carried); a product of 17 to
+        64 rows whose slices meet in a kernel of their own has that kernel write the norm's output as well (a Carried
+        that is `ready`); in steps of many rows the product only adds, and the norm's kernel reads one matrix instead
+        of two and writes one instead of two."""
         if into is None or into.norm is None or isinstance(x, Carried):
             return None
         width = self.out_features
