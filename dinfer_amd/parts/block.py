@@ -21,7 +21,8 @@ from .spec import LayerSpec
 # A norm is carried by the products around it in steps of up to this many tokens (one token tile of the few-row
 # kernel). Measured at the 8B sizes: a step of 1 token 3.82 -> 3.68 ms, of 8 4.07 -> 4.00, of 16 4.65 -> 4.62; at 32
 # tokens (two token tiles) the longer ends of four kernels cost more than the two norm kernels did (5.93 -> 6.11 ms);
-# carrying only the norm after the mixer there (the down projection has another kernel at those rows) 5.39 -> 5.44 ms.
+# carrying only the norm after the mixer there (the down projection has another kernel at those rows) 5.39 -> 5.44 ms,
+# and with the kernel for wide weights as the gate/up product that applies it 5.22 -> 5.28 (4.88 -> 4.92 at 24 tokens).
 CARRY_ROWS = 16
 
 
